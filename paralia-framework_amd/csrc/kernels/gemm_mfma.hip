@@ -1,0 +1,318 @@
+// Tile GEMM for gfx950 (MI355X): C = alpha * op(A) * op(B) + beta * C, column-major, fp64 and fp32.
+//
+// This is the compute of one PARALiA "subkernel": the reference hands each T x T x T tile product to
+// cublasDgemm / cublasSgemm through backend_run_operation (Library_scheduler/src/Subkernel.cpp:168,228;
+// direct call form Database_builder/CuCuBLAS/src/dgemm_microbench.cu:141-142).  Here it is a hand-written
+// MFMA kernel:
+//   * one workgroup = 256 threads = 4 wavefronts (2 x 2), macro tile 128 x 128, each wave owns 64 x 64;
+//   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2);
+//   * A and B k-panels (16 doubles / 32 floats deep) are staged global -> registers -> LDS, double-buffered,
+//     one barrier per k-panel; the next panel's global loads are in flight while the current one is multiplied;
+//   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
+//   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
+//     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
+//   * workgroup ids are re-mapped so the eight XCDs each own a compact block of C tiles (private L2 per XCD),
+//     and inside an XCD neighbouring ids share A row-panels.
+// Arbitrary M, N, K and leading dimensions are handled; 16-byte vector loads are used when pointer and
+// leading dimension allow it and the workgroup's tile is interior, element loads with zero fill otherwise.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Row index (MFMA i) of accumulator element r for lane group g = lane / 16 in the 16x16 fp64 result block.
+#ifndef PLK_F64_DROW
+#define PLK_F64_DROW(r, g) (4 * (r) + (g))
+#endif
+
+namespace plk {
+
+typedef double double4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef double dvec2 __attribute__((ext_vector_type(2)));
+typedef float fvec4 __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 128, BN = 128, NTHREADS = 256, WM = 64, WN = 64;
+
+template <typename T> struct Traits;
+
+template <> struct Traits<double> {
+  using vec_t = dvec2;
+  using acc_t = double4_t;
+  static constexpr int VEC = 2;      // elements per 16-byte vector
+  static constexpr int BK = 16;      // k-panel depth
+  static constexpr int BLK = 16;     // MFMA block edge
+  static constexpr int KSTEP = 4;    // k consumed per MFMA
+  static constexpr int NACC = 4;     // accumulator elements per lane per block
+  static constexpr int S_MN = 144;   // LDS row stride, [k][mn] layout (1152 B = 128 mod 256)
+  static constexpr int S_K = 18;     // LDS row stride, [mn][k] layout (144 B)
+  static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  // Row (MFMA i index) held by accumulator element r of a lane in lane-group g = lane / 16.
+  static __device__ __forceinline__ int drow(int r, int g) { return PLK_F64_DROW(r, g); }
+};
+
+template <> struct Traits<float> {
+  using vec_t = fvec4;
+  using acc_t = float16_t;
+  static constexpr int VEC = 4;
+  static constexpr int BK = 32;
+  static constexpr int BLK = 32;
+  static constexpr int KSTEP = 2;
+  static constexpr int NACC = 16;
+  static constexpr int S_MN = 160;   // 640 B = 128 mod 256
+  static constexpr int S_K = 36;     // 144 B
+  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int drow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+};
+
+template <typename T, bool KMAJOR> struct Lds {
+  using Tr = Traits<T>;
+  // elements of one staged panel (128 x BK plus padding)
+  static constexpr int SIZE = KMAJOR ? 128 * Tr::S_K : Tr::BK * Tr::S_MN;
+  static __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * Tr::S_K + k : k * Tr::S_MN + mn; }
+};
+
+// One thread's share of a 128 x BK panel: four 16-byte vectors.  "c" runs along the memory-contiguous
+// dimension (mn for MN-major operands, k for K-major ones), "s" along the leading-dimension stride.
+template <typename T, bool KMAJOR> struct Slot {
+  using Tr = Traits<T>;
+  static constexpr int CVECS = (KMAJOR ? Tr::BK : 128) / Tr::VEC;  // vectors per contiguous run
+  static __device__ __forceinline__ void coords(int tid, int i, int& c, int& s) {
+    int v = tid + NTHREADS * i;
+    c = (v % CVECS) * Tr::VEC;
+    s = v / CVECS;
+  }
+};
+
+template <typename T, bool KMAJOR, bool GUARD>
+__device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int crem, int srem, bool vec_ok,
+                                      typename Traits<T>::vec_t (&regs)[4], int tid) {
+  using Tr = Traits<T>;
+  using vec_t = typename Tr::vec_t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int c, s;
+    Slot<T, KMAJOR>::coords(tid, i, c, s);
+    const T* p = base + c + (long)s * ld;
+    if (!GUARD) {
+      regs[i] = *reinterpret_cast<const vec_t*>(p);
+    } else {
+      vec_t v;
+#pragma unroll
+      for (int e = 0; e < Tr::VEC; ++e) v[e] = T(0);
+      if (s < srem) {
+        if (vec_ok && c + Tr::VEC <= crem) {
+          v = *reinterpret_cast<const vec_t*>(p);
+        } else {
+#pragma unroll
+          for (int e = 0; e < Tr::VEC; ++e)
+            if (c + e < crem) v[e] = p[e];
+        }
+      }
+      regs[i] = v;
+    }
+  }
+}
+
+template <typename T, bool KMAJOR>
+__device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[4], int tid) {
+  using Tr = Traits<T>;
+  using vec_t = typename Tr::vec_t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int c, s;
+    Slot<T, KMAJOR>::coords(tid, i, c, s);
+    // the contiguous run is also contiguous in LDS for both layouts
+    int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
+    *reinterpret_cast<vec_t*>(xs + off) = regs[i];
+  }
+}
+
+// Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
+// give each XCD a contiguous range of logical ids, then walk that range in groups of 8 block rows.
+__device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, int& bn) {
+  const int nb = gm * gn;
+  const int q = nb >> 3, r = nb & 7;
+  const int xcd = bid & 7, loc = bid >> 3;
+  const int pid = (xcd < r) ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+  constexpr int GM = 8;
+  const int width = GM * gn;
+  const int group = pid / width;
+  const int first_m = group * GM;
+  const int gsz = min(gm - first_m, GM);
+  const int in = pid - group * width;
+  bm = first_m + in % gsz;
+  bn = in / gsz;
+}
+
+// AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
+template <typename T, bool AK, bool BKM>
+__global__ __launch_bounds__(NTHREADS, 2) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
+                                                          const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
+                                                          long ldc, int gm, int gn, int vecA, int vecB) {
+  using Tr = Traits<T>;
+  using vec_t = typename Tr::vec_t;
+  using acc_t = typename Tr::acc_t;
+  constexpr int BK = Tr::BK, BLK = Tr::BLK, NB = WM / BLK;
+  constexpr int ASZ = Lds<T, AK>::SIZE, BSZ = Lds<T, BKM>::SIZE;
+
+  __shared__ __attribute__((aligned(16))) T smem[2 * (ASZ + BSZ)];
+  constexpr int STAGE = ASZ + BSZ;  // buffer b holds A at smem + b*STAGE and B right behind it
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int idx = lane % BLK, kk = lane / BLK;
+  const int wm = (wave & 1) * WM, wn = (wave >> 1) * WN;
+
+  int bm, bn;
+  block_coords(blockIdx.x, gm, gn, bm, bn);
+  const int m0 = bm * BM, n0 = bn * BN;
+  const int mrem = min(M - m0, BM), nrem = min(N - n0, BN);
+  const bool fast = (mrem == BM) && (nrem == BN) && vecA && vecB;
+
+  // tile origins; element (mn, k) of op(X) lives at base[mn + k*ld] (MN-major) or base[k + mn*ld] (K-major)
+  const T* Ab = AK ? A + (long)m0 * lda : A + m0;
+  const T* Bb = BKM ? B + (long)n0 * ldb : B + (long)n0;
+  const long a_kstep = AK ? (long)BK : (long)BK * lda;
+  const long b_kstep = BKM ? (long)BK : (long)BK * ldb;
+
+  acc_t acc[NB][NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < Tr::NACC; ++r) acc[i][j][r] = T(0);
+
+  const int nkt = (K + BK - 1) / BK;
+  const int nfull = K / BK;
+  vec_t ra[4], rb[4];
+
+  auto fetch = [&](int kt) {
+    const T* ap = Ab + kt * a_kstep;
+    const T* bp = Bb + kt * b_kstep;
+    if (fast && kt < nfull) {
+      gload<T, AK, false>(ap, lda, 0, 0, true, ra, tid);
+      gload<T, BKM, false>(bp, ldb, 0, 0, true, rb, tid);
+    } else {
+      const int krem = min(K - kt * BK, BK);
+      gload<T, AK, true>(ap, lda, AK ? krem : mrem, AK ? mrem : krem, vecA, ra, tid);
+      gload<T, BKM, true>(bp, ldb, BKM ? krem : nrem, BKM ? nrem : krem, vecB, rb, tid);
+    }
+  };
+
+  if (nkt > 0) {
+    fetch(0);
+    lds_store<T, AK>(smem, ra, tid);
+    lds_store<T, BKM>(smem + ASZ, rb, tid);
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nkt) fetch(kt + 1);
+    const T* as = smem + cur * STAGE;
+    const T* bs = as + ASZ;
+#pragma unroll
+    for (int ks = 0; ks < BK / Tr::KSTEP; ++ks) {
+      T am[NB], bnv[NB];
+      const int k = ks * Tr::KSTEP + kk;
+#pragma unroll
+      for (int j = 0; j < NB; ++j) am[j] = as[Lds<T, AK>::at(k, wm + j * BLK + idx)];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) bnv[i] = bs[Lds<T, BKM>::at(k, wn + i * BLK + idx)];
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[i], am[j], acc[i][j]);
+    }
+    if (kt + 1 < nkt) {
+      lds_store<T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
+      lds_store<T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk))
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+#pragma unroll
+    for (int r = 0; r < Tr::NACC; ++r) {
+      const int n = wn + i * BLK + Tr::drow(r, kk);
+      if (n < nrem) {
+        T* ccol = C + (long)(n0 + n) * ldc + m0;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          const int m = wm + j * BLK + idx;
+          if (m < mrem) {
+            T v = alpha * acc[i][j][r];
+            if (beta != T(0)) v += beta * ccol[m];
+            ccol[m] = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+// C = beta * C on an M x N column-major view (alpha == 0 or K == 0: A and B are not referenced).
+template <typename T>
+__global__ void scale_kernel(int M, int N, T beta, T* __restrict__ C, long ldc) {
+  const long total = (long)M * N;
+  for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    const long m = e % M, n = e / M;
+    T* p = C + n * ldc + m;
+    *p = (beta == T(0)) ? T(0) : beta * *p;
+  }
+}
+
+template <typename T>
+int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
+                T* C, long ldc, hipStream_t stream) {
+  using Tr = Traits<T>;
+  const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
+  const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
+  if (!(at || an) || !(bt || bnn)) return 1;
+  if (M < 0 || N < 0 || K < 0) return 2;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 2;
+  const long rowsA = an ? M : K, rowsB = bnn ? K : N;
+  if (lda < (rowsA > 1 ? rowsA : 1) || ldb < (rowsB > 1 ? rowsB : 1) || ldc < (M > 1 ? M : 1)) return 3;
+  if (M == 0 || N == 0) return 0;
+  if (K == 0 || alpha == T(0)) {
+    if (beta == T(1)) return 0;
+    const long total = M * N;
+    int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(scale_kernel<T>, dim3(blocks), dim3(256), 0, stream, (int)M, (int)N, beta, C, ldc);
+    return hipGetLastError() == hipSuccess ? 0 : 4;
+  }
+  if (!A || !B || !C) return 5;
+  const int gm = (int)((M + BM - 1) / BM), gn = (int)((N + BN - 1) / BN);
+  if ((long)gm * gn > INT32_MAX) return 2;
+  const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
+  const int vecB = ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % Tr::VEC == 0) ? 1 : 0;
+  dim3 grid(gm * gn), block(NTHREADS);
+#define PLK_LAUNCH(AKF, BKF)                                                                                    \
+  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF>), grid, block, 0, stream, (int)M, (int)N, (int)K, alpha, A, lda, B, \
+                     ldb, beta, C, ldc, gm, gn, vecA, vecB)
+  // op(A) K-major <=> TransA == 'T'; op(B) K-major <=> TransB == 'N'
+  if (an && bnn) PLK_LAUNCH(false, true);
+  else if (an && bt) PLK_LAUNCH(false, false);
+  else if (at && bnn) PLK_LAUNCH(true, true);
+  else PLK_LAUNCH(true, false);
+#undef PLK_LAUNCH
+  return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+}  // namespace plk
+
+extern "C" int pl_dgemm_tile(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                             const double* B, long ldb, double beta, double* C, long ldc, void* stream) {
+  return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream);
+}
+
+extern "C" int pl_sgemm_tile(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                             const float* B, long ldb, float beta, float* C, long ldc, void* stream) {
+  return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream);
+}
