@@ -100,6 +100,70 @@ long pl_ddot_workspace_doubles(void);
 int pl_ddot(long n, const double* x, long incx, const double* y, long incy, double* result, int accumulate,
             double* workspace, void* stream);
 
+/* ---- routines: plain-C faces of Library_scheduler/include/PARALiA.hpp:33-72 ----
+ * Operands may be host (pinned or pageable) or device pointers; the library detects which.  Calls return
+ * after the result has reached the caller's buffer.  T > 0 / cache_limit > 0 preset the tile size and the
+ * device block-pool limit in bytes (the ...Controled variants, PARALiA.hpp:37-38; unset: T <= 0, limit 0,
+ * Autotuner.cpp:27-31).  info, when not null, receives what the returned ATC_p carries in C++. */
+typedef struct pl_atc_info {
+  long T;                 /* tile size used */
+  double pred_t;          /* predicted seconds */
+  long subkernel_num;
+  int order_id;           /* subkernel order family picked by the pipeline model */
+  int exec_queues;
+  long long cache_limit;
+  int has_db;             /* autotuner database found */
+  char selected_by[32];   /* user | resident | pipeline-model | cocopelia-reuse | cocopelia-bidirectional | heuristic */
+  double slowdowns[6];    /* T_aggregate, imbalance, remainder, small, sknum, big (Autotuner.cpp:561-569) */
+  double pipe_total, pipe_h2d, pipe_exec, pipe_d2h;
+} pl_atc_info;
+
+const char* PARALiA_last_error(void);
+/* PARALiADgemm / PARALiADgemmControled (dgemm.cpp:318,697) */
+int PARALiA_dgemm(char TransA, char TransB, long M, long N, long K, double alpha, double* A, long ldA, double* B, long ldB,
+                  double beta, double* C, long ldC, long T, long long cache_limit, pl_atc_info* info);
+/* PARALiASgemm / PARALiASgemmControled (sgemm.cpp:296) */
+int PARALiA_sgemm(char TransA, char TransB, long M, long N, long K, float alpha, float* A, long ldA, float* B, long ldB,
+                  float beta, float* C, long ldC, long T, long long cache_limit, pl_atc_info* info);
+/* PARALiADaxpy / PARALiADaxpyControled (daxpy.cpp:200) */
+int PARALiA_daxpy(long N, double alpha, double* x, long incx, double* y, long incy, long T, pl_atc_info* info);
+/* PARALiADdot / PARALiADdotControled (ddot.cpp:201): the dot product is ADDED to *result (ddot.cpp:431) */
+int PARALiA_ddot(long N, double* x, long incx, double* y, long incy, double* result, long T, pl_atc_info* info);
+/* PARALiADevCacheFree (Subkernel.cpp:488) */
+int PARALiA_dev_cache_free(int dev_id);
+/* metadata-cache and pool counters (PMD_cache, dgemm.cpp:342-368); reset drops the cached problems */
+int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries);
+int PARALiA_runtime_reset(void);
+/* directory holding Processed/ lookup tables and link models (DEPLOYDB, CMakeLists.txt:376) */
+int PARALiA_set_db_dir(const char* dir);
+
+/* ---- driver helper surface (CoCoMalloc / CoCoFree / CoCoVecInit / Dtest_equality, dgemm_runner.cpp:55-99) ---- */
+int PARALiA_malloc(void** ptr, long long bytes, int loc);
+int PARALiA_free(void* ptr, int loc);
+int PARALiA_vec_init_f64(double* p, long long n, int seed, int loc);
+int PARALiA_vec_init_f32(float* p, long long n, int seed, int loc);
+int PARALiA_test_equality_f64(double* ref, double* x, long long n);
+int PARALiA_test_equality_f32(float* ref, float* x, long long n);
+
+/* ---- host-logic probes: no GPU call is made by any of these ---- */
+/* ATC::optimize_tile / get_T_slowdowns for one unit (Autotuner.cpp:571-655); returns T */
+long PARALiA_heuristic_tile(long D1, long D2, long D3, double slowdowns[6]);
+int PARALiA_T_slowdowns(long D1, long D2, long D3, long T, double slowdowns[6]);
+/* Modeler::predict (ModelLvl3.cpp:287-551, ModelLvl1.cpp:262): mode = ModelType value, loc[i] = -1 host / 0 device */
+double PARALiA_model_predict(const char* db_dir, const char* func, int mode, long D1, long D2, long D3, char ta, char tb,
+                             const int loc[3], long T);
+/* ATC::autotune_problem (Autotuner.cpp:279) without touching the GPU */
+int PARALiA_autotune(const char* db_dir, const char* func, long D1, long D2, long D3, char ta, char tb, const int loc[3],
+                     int beta_zero, long T_in, long long pool_budget_bytes, pl_atc_info* info);
+/* static GEMM plan (CreateSubkernelsDgemm + request_data + run_operation, dgemm.cpp:123-205, Subkernel.cpp:90-247) */
+#define PL_PLAN_MAX_WAITS 12
+#define PL_PLAN_ROW (10 + PL_PLAN_MAX_WAITS)
+long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
+                       int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]);
+double PARALiA_gemm_plan_simulate(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero,
+                                  int elem, int exec_queues, long pool_blocks, int order_id, double t_exec, double h2d_ti,
+                                  double h2d_tb, double d2h_ti, double d2h_tb, double t_reduce, int* picked, double busy[3]);
+
 #ifdef __cplusplus
 }
 #endif

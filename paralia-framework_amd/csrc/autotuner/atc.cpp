@@ -1,0 +1,418 @@
+// Autotuning controller: picks the tile size T (and, for GEMM, the subkernel order) for one call on one GPU.
+//
+// Three selectors, all available at run time (PARALIA_T_SELECT = pipeline | reuse | heuristic):
+//   heuristic  the reference's main-branch scan of every integer T under penalty terms
+//              (Autotuner/src/Autotuner.cpp:571-655);
+//   reuse      the reference's model-driven search, argmin of the CoCoPeLia data-reuse model over the
+//              benchmarked T values (Model_functions.cpp:195-244 with ModelLvl3.cpp:476-551);
+//   pipeline   (default) the same search, but each T is priced by simulating this runtime's actual H2D /
+//              compute / D2H command streams for the best subkernel order (runtime/gemm_plan.cpp).
+// Without a database only the heuristic is possible.
+#include <cfloat>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include "Autotuner.hpp"
+#include "backend_wrappers.hpp"
+#include "runtime/gemm_plan.hpp"
+
+ATC::ATC() {
+  active_unit_id_list = (int*)malloc(LOC_NUM * sizeof(int));
+  active_unit_score = (double*)malloc(LOC_NUM * sizeof(double));
+  Subkernels_per_unit_num = (int*)malloc(LOC_NUM * sizeof(int));
+  Subkernels_per_unit_list = (int**)malloc(LOC_NUM * sizeof(int*));
+  for (int d = 0; d < LOC_NUM; d++) {
+    active_unit_id_list[d] = -42;
+    active_unit_score[d] = -42.0;
+    Subkernels_per_unit_list[d] = NULL;
+    Subkernels_per_unit_num[d] = 0;
+  }
+  T = active_unit_num = subkernel_num = -1;
+  pred_t = pred_J = power_delay = energy_delay = -1.0;
+  pred_t_pesimistic = pred_J_pesimistic = power_delay_pesimistic = energy_delay_pesimistic = -1.0;
+  T_aggregate_sl = T_imbalance_sl = T_remainder_sl = T_small_sl = T_sknum_sl = T_big_sl = 0.0;
+  cache_limit = 0;
+  unit_modeler_list = (MD_p*)calloc(LOC_NUM, sizeof(MD_p));
+  has_db = false;
+  owns_modelers = true;
+  order_id = 10000;
+  exec_queues = 2;
+  T_selected_by = "unset";
+}
+
+ATC::~ATC() {
+  free(active_unit_id_list);
+  free(active_unit_score);
+  free(Subkernels_per_unit_num);
+  for (int d = 0; d < LOC_NUM; d++) free(Subkernels_per_unit_list[d]);
+  free(Subkernels_per_unit_list);
+  if (owns_modelers)
+    for (int d = 0; d < LOC_NUM; d++) delete unit_modeler_list[d];
+  free(unit_modeler_list);
+}
+
+void ATC::reset() {
+  for (int d = 0; d < LOC_NUM; d++) {
+    free(Subkernels_per_unit_list[d]);
+    Subkernels_per_unit_list[d] = NULL;
+    Subkernels_per_unit_num[d] = 0;
+  }
+  T = active_unit_num = subkernel_num = -1;
+  pred_t = -1.0;
+  cache_limit = 0;
+}
+
+int ATC::diff_intialized_params_ATC(ATC_p other) {
+  int result = 0;
+  if (other->T != -1 && other->T != T) result++;
+  if (other->active_unit_num != -1 && other->active_unit_num != active_unit_num) result++;
+  else if (other->active_unit_num != -1 && other->active_unit_num == active_unit_num) {
+    for (int ctr = 0; ctr < active_unit_num; ctr++)
+      if (other->active_unit_id_list[ctr] != active_unit_id_list[ctr]) { result++; break; }
+  }
+  if (other->cache_limit != 0 && other->cache_limit != cache_limit) result++;
+  return result;
+}
+
+void ATC::mimic_ATC(ATC_p other) {
+  T = other->T;
+  T_aggregate_sl = other->T_aggregate_sl; T_imbalance_sl = other->T_imbalance_sl; T_remainder_sl = other->T_remainder_sl;
+  T_small_sl = other->T_small_sl; T_sknum_sl = other->T_sknum_sl; T_big_sl = other->T_big_sl;
+  active_unit_num = other->active_unit_num;
+  for (int d = 0; d < LOC_NUM; d++) {
+    active_unit_id_list[d] = other->active_unit_id_list[d];
+    active_unit_score[d] = other->active_unit_score[d];
+    Subkernels_per_unit_num[d] = other->Subkernels_per_unit_num[d];
+    free(Subkernels_per_unit_list[d]);
+    Subkernels_per_unit_list[d] = NULL;
+    if (other->Subkernels_per_unit_list[d] && other->subkernel_num > 0) {
+      Subkernels_per_unit_list[d] = (int*)malloc(other->subkernel_num * sizeof(int));
+      memcpy(Subkernels_per_unit_list[d], other->Subkernels_per_unit_list[d], other->subkernel_num * sizeof(int));
+    }
+  }
+  split_homogeneously = other->split_homogeneously;
+  pred_t = other->pred_t; pred_J = other->pred_J; power_delay = other->power_delay; energy_delay = other->energy_delay;
+  pred_t_pesimistic = other->pred_t_pesimistic; pred_J_pesimistic = other->pred_J_pesimistic;
+  power_delay_pesimistic = other->power_delay_pesimistic; energy_delay_pesimistic = other->energy_delay_pesimistic;
+  subkernel_num = other->subkernel_num;
+  cache_limit = other->cache_limit;
+  if (owns_modelers)
+    for (int d = 0; d < LOC_NUM; d++) delete unit_modeler_list[d];
+  owns_modelers = false;  // the original keeps them alive (it sits in the problem-metadata cache)
+  for (int d = 0; d < LOC_NUM; d++) unit_modeler_list[d] = other->unit_modeler_list[d];
+  problem = other->problem;
+  has_db = other->has_db;
+  order_id = other->order_id;
+  exec_queues = other->exec_queues;
+  T_selected_by = other->T_selected_by;
+  pipeline = other->pipeline;
+}
+
+void ATC::update_sk_num(long long subkernel_num_in) {
+  const long prev = subkernel_num;
+  subkernel_num = (long)subkernel_num_in;
+  if (prev != subkernel_num)
+    for (int d = 0; d < LOC_NUM; d++) {
+      free(Subkernels_per_unit_list[d]);
+      Subkernels_per_unit_list[d] = (int*)malloc(subkernel_num * sizeof(int));
+      for (long s = 0; s < subkernel_num; s++) Subkernels_per_unit_list[d][s] = -1;
+    }
+}
+
+// One unit owns every subkernel: all distributions of the reference (Subkernel_distributions.cpp) collapse
+// to the identity list 0 .. n-1 on unit 0.
+void ATC::distribute_subkernels(int D1GridSz, int D2GridSz, int D3GridSz) {
+  (void)D1GridSz; (void)D2GridSz; (void)D3GridSz;
+  for (int d = 0; d < LOC_NUM; d++) Subkernels_per_unit_num[d] = 0;
+  Subkernels_per_unit_num[0] = (int)subkernel_num;
+  for (long s = 0; s < subkernel_num; s++) Subkernels_per_unit_list[0][s] = (int)s;
+}
+
+void ATC::init_modelers(const char* routine_name, const ProblemDesc& desc) {
+  (void)routine_name;
+  const std::string db = paralia_db_dir();
+  if (owns_modelers)
+    for (int d = 0; d < LOC_NUM; d++) { delete unit_modeler_list[d]; unit_modeler_list[d] = nullptr; }
+  owns_modelers = true;
+  // only the GPU unit executes; the host "unit" of the reference (CPU workload) is not used on this path
+  unit_modeler_list[0] = new Modeler(db, 0, desc);
+}
+
+void ATC::set_T_slowdowns(double* sl) {
+  T_aggregate_sl = sl[0]; T_imbalance_sl = sl[1]; T_remainder_sl = sl[2];
+  T_small_sl = sl[3]; T_sknum_sl = sl[4]; T_big_sl = sl[5];
+}
+
+static long sk_num_of(const ProblemDesc& P, long T) {
+  auto cdiv = [](long a, long b) { return a / b + ((a % b) ? 1 : 0); };
+  if (P.problem == BLAS3) return cdiv(P.D1, T) * cdiv(P.D2, T) * cdiv(P.D3, T);
+  return cdiv(P.D1, T);
+}
+
+void ATC::get_T_slowdowns(double* slowdown, int candidate_T) {
+  // int arithmetic and conversion order as in Autotuner.cpp:571-603
+  const int D1 = (int)problem.D1, D2 = (problem.D2 == -1) ? D1 : (int)problem.D2, D3 = (problem.D3 == -1) ? D1 : (int)problem.D3;
+  for (int idx = 0; idx < 6; idx++) slowdown[idx] = 0.0;
+  ProblemDesc cube = problem;
+  cube.problem = BLAS3; cube.D1 = D1; cube.D2 = D2; cube.D3 = D3;
+  const long sk = sk_num_of(cube, candidate_T);
+  int bucket_num = (int)(sk / (D3 / candidate_T + ((D3 % candidate_T) ? 1 : 0)));
+  slowdown[1] = (bucket_num / active_unit_num)
+                    ? 1.0 * (bucket_num % active_unit_num) / (bucket_num / active_unit_num) * active_unit_num
+                    : 1.0 * bucket_num / active_unit_num;
+  if (D1 % candidate_T) slowdown[2] += 1.0 / (D1 / candidate_T);
+  if (D2 % candidate_T) slowdown[2] += 1.0 / (D2 / candidate_T);
+  if (D3 % candidate_T) slowdown[2] += 1.0 / (D3 / candidate_T);
+  if (candidate_T < TILE_MIN) slowdown[3] += 1.0 * TILE_MIN / candidate_T * TILE_MIN_SLOWDOWN;
+  long dev_sks = (long)((1.0 * sk) / active_unit_num);
+  slowdown[4] += 2.0 / (dev_sks);
+  if (dev_sks > MAX_DESIRED_SK_DEV) slowdown[4] += (1.0 * dev_sks / MAX_DESIRED_SK_DEV) * MAX_DESIRED_SK_DEV_SLOWDOWN;
+  if (candidate_T > TILE_MAX) slowdown[5] += candidate_T / TILE_MAX * TILE_MAX_SLOWDOWN;
+  slowdown[0] = slowdown[1] + slowdown[2] + slowdown[3] + slowdown[4] + slowdown[5];
+}
+
+double ATC::optimize_tile() {
+  double timer = csecond();
+  if (active_unit_num <= 0) error("ATC::optimize_tile: Called with active_unit_num = %d\n", active_unit_num);
+  const int D1 = (int)problem.D1, D2 = (problem.D2 == -1) ? D1 : (int)problem.D2, D3 = (problem.D3 == -1) ? D1 : (int)problem.D3;
+  const int max_allowed_T = std::min(D1, std::min(D2, D3));
+  int best_T = -1;
+  double best_sl[6], cur[6];
+  for (int i = 0; i < 6; i++) best_sl[i] = DBL_MAX;
+  for (int cand = max_allowed_T; cand > 0; cand--) {
+    get_T_slowdowns(cur, cand);
+    if (cur[0] < best_sl[0]) {
+      for (int i = 0; i < 6; i++) best_sl[i] = cur[i];
+      best_T = cand;
+    }
+  }
+  T = best_T;
+  set_T_slowdowns(best_sl);
+  return csecond() - timer;
+}
+
+double ATC::optimize_tile_CoCoPeLia(int model_idx, ModelType mode) {
+  double timer = csecond();
+  MD_p model = unit_modeler_list[model_idx];
+  if (!model) error("ATC::optimize_tile_CoCoPeLia: no modeler for unit index %d (database missing?)\n", model_idx);
+  long min_T = model->getMinT();
+  const long max_allowed_T = model->getMaxT();
+  if (min_T > max_allowed_T) {
+    T = max_allowed_T;
+    pred_t = 0;  // undefined performance below the smallest benchmarked tile
+    return csecond() - timer;
+  }
+  double min_t = model->predict(mode, model->exec->T[0]);
+  if (min_t < 0) error("CoCoPeLiaModelOptimizeTile: First value in DM results in negative prediction");
+  long prev_trial_T = 0;
+  for (long ctr = 1; ctr < model->exec->lines(); ctr++) {
+    const long trial_T = model->exec->T[ctr];
+    if (trial_T > max_allowed_T) break;
+    if (trial_T == prev_trial_T) continue;
+    const double temp_t = model->predict(mode, trial_T);
+    if (temp_t >= 0 && temp_t < min_t) {
+      min_t = temp_t;
+      min_T = trial_T;
+    }
+    prev_trial_T = trial_T;
+  }
+  T = min_T;
+  pred_t = min_t;
+  return csecond() - timer;
+}
+
+namespace {
+
+paralia::GemmProblem gemm_problem_of(const ProblemDesc& d, long T, int exec_queues) {
+  paralia::GemmProblem gp;
+  gp.M = d.D1; gp.N = d.D2; gp.K = d.D3; gp.T = T;
+  gp.a_remote = remote(d.loc[0], 0); gp.b_remote = remote(d.loc[1], 0); gp.c_remote = remote(d.loc[2], 0);
+  gp.beta_zero = d.beta_is_zero;
+  gp.elem = d.dtype_sz;
+  gp.exec_queues = exec_queues;
+  const long full = paralia::gemm_full_block_num(gp);
+  gp.pool_blocks = full;
+  if (d.pool_budget_bytes > 0) {
+    const long long blk = (long long)T * T * d.dtype_sz;
+    gp.pool_blocks = (long)std::min<long long>(full, d.pool_budget_bytes / blk);
+  }
+  return gp;
+}
+
+// Nominal MI355X stage costs, used only when no database has been deployed.
+paralia::StageTimes nominal_stage_times(const ProblemDesc& d, long T) {
+  paralia::StageTimes st;
+  const double flops = d.dtype_sz == 8 ? 60e12 : 120e12;
+  st.t_exec = 2.0 * T * T * T / flops;
+  st.h2d_ti = st.d2h_ti = 10e-6;
+  st.h2d_tb = st.d2h_tb = 1.0 / 50e9;
+  st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
+  return st;
+}
+
+}  // namespace
+
+paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
+  const ProblemDesc& d = atc->problem;
+  if (!atc->has_db || !atc->unit_modeler_list[0]) return nominal_stage_times(d, T);
+  const Modeler* m = atc->unit_modeler_list[0];
+  paralia::StageTimes st;
+  st.t_exec = m->exec->predict(T, d.TransA, d.TransB);
+  const comm_data* h2d = m->link[idxize(-1)];
+  const comm_data* d2h = m->revlink[idxize(-1)];
+  st.h2d_ti = h2d->ti; st.h2d_tb = h2d->tb;
+  st.d2h_ti = d2h->ti; st.d2h_tb = d2h->tb;
+  st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
+  return st;
+}
+
+double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) {
+  double timer = csecond();
+  problem = desc;
+  problem.func = routine_name;
+  if (!strcmp(routine_name, "Dgemm") || !strcmp(routine_name, "Sgemm")) problem.problem = BLAS3;
+  else if (!strcmp(routine_name, "Daxpy") || !strcmp(routine_name, "Ddot")) problem.problem = BLAS1;
+  else error("ATC::autotune_problem: routine %s not integrated\n", routine_name);
+
+  // one GPU: the unit list is {0} whatever was asked for (predefined lists naming other units are an error)
+  if (active_unit_num > 1) error("ATC::autotune_problem: %d units requested, this build drives one GPU\n", active_unit_num);
+  if (active_unit_num == 1 && active_unit_id_list[0] != 0)
+    error("ATC::autotune_problem: unit id %d requested, only device 0 is driven\n", active_unit_id_list[0]);
+  active_unit_num = 1;
+  active_unit_id_list[0] = 0;
+  active_unit_score[0] = 1.0;
+
+  const char* sel_env = getenv("PARALIA_T_SELECT");
+  std::string selector = sel_env ? sel_env : "pipeline";
+  has_db = false;
+  try {
+    init_modelers(routine_name, problem);
+    has_db = true;
+  } catch (const paralia_error& e) {
+    static bool warned = false;
+    if (!warned) warning("autotuner database not usable (%s); falling back to the tile heuristic\n", e.what());
+    warned = true;
+    if (owns_modelers)
+      for (int d = 0; d < LOC_NUM; d++) { delete unit_modeler_list[d]; unit_modeler_list[d] = nullptr; }
+  }
+
+  bool any_remote = false;
+  for (int i = 0; i < problem.numT; i++) any_remote |= remote(problem.loc[i], 0) != 0;
+  const char* q_env = getenv("PARALIA_EXEC_QUEUES");
+  if (q_env && atoi(q_env) > 0) exec_queues = std::min(atoi(q_env), (int)paralia::MAX_EXEC_QUEUES);
+  pipeline = PipelineEstimate();
+
+  if (problem.problem == BLAS3) {
+    const long min_dim = std::min(problem.D1, std::min(problem.D2, problem.D3));
+    const long max_dim = std::max(problem.D1, std::max(problem.D2, problem.D3));
+    if (T > 0) {
+      if (T > max_dim) T = max_dim;  // a tile larger than every dimension is the whole problem
+      T_selected_by = "user";
+    } else if (!any_remote) {
+      // nothing to stream: one launch over the caller's matrices, T only labels the call
+      T = max_dim;
+      T_selected_by = "resident";
+    } else if (!has_db || selector == "heuristic") {
+      optimize_tile();
+      T_selected_by = "heuristic";
+    } else if (selector == "reuse") {
+      optimize_tile_CoCoPeLia(0, COCOPELIA_REUSE);
+      T_selected_by = "cocopelia-reuse";
+    } else {
+      const Modeler* m = unit_modeler_list[0];
+      long best_T = -1, prev = -1;
+      double best_t = DBL_MAX;
+      for (long i = 0; i < m->exec->lines(); i++) {
+        const long cand = m->exec->T[i];
+        if (cand == prev) continue;
+        prev = cand;
+        // tiles may be shallower than T in K (depth min(T, K)), so only M and N bound the candidates
+        if (cand > std::min(problem.D1, problem.D2)) continue;
+        paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
+        if (gp.pool_blocks < 3 || gp.subkernels() > 20000) continue;
+        paralia::PipelineResult r;
+        try {
+          paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
+        } catch (const std::runtime_error&) { continue; }
+        if (r.t_total < best_t) { best_t = r.t_total; best_T = cand; }
+      }
+      if (best_T < 0) {
+        // C narrower than every benchmarked tile: one tile across the short side, as square as that allows
+        T = std::max(std::min(problem.D1, problem.D2), std::min(max_dim, m->exec->MinT()));
+        T_selected_by = "heuristic";
+      } else {
+        T = best_T;
+        T_selected_by = "pipeline-model";
+      }
+    }
+    if (T <= 0) error("ATC::autotune_problem: T = %ld after tuning\n", T);
+    if (T <= min_dim) {
+      double sl[6];
+      get_T_slowdowns(sl, (int)T);
+      set_T_slowdowns(sl);
+    }
+    // order + predicted time for the chosen T
+    paralia::GemmProblem gp = gemm_problem_of(problem, T, exec_queues);
+    if (any_remote && gp.pool_blocks < 3)
+      error("PARALiA gemm: Problem cannot run with less memory than %lld\n", 3LL * T * T * problem.dtype_sz);
+    paralia::PipelineResult r;
+    try {
+      order_id = paralia::pick_gemm_order(gp, paralia_stage_times(this, T), &r);
+    } catch (const std::runtime_error& e) { error("%s\n", e.what()); }
+    pipeline.t_total = r.t_total; pipeline.t_h2d_busy = r.t_h2d; pipeline.t_exec_busy = r.t_exec;
+    pipeline.t_d2h_busy = r.t_d2h; pipeline.order_id = order_id;
+    pred_t = r.t_total;
+    pred_t_pesimistic = r.t_h2d + r.t_exec + r.t_d2h;
+    update_sk_num(gp.subkernels());
+    distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
+  } else {
+    const long N = problem.D1;
+    if (T > 0) {
+      if (T > N) T = N;
+      T_selected_by = "user";
+    } else if (!any_remote) {
+      T = N;
+      T_selected_by = "resident";
+    } else if (has_db) {
+      optimize_tile_CoCoPeLia(0, COCOPELIA_BIDIRECTIONAL);
+      T_selected_by = "cocopelia-bidirectional";
+    } else {
+      T = std::min(N, 1L << 22);  // 32 MiB tiles: large enough to run the link at its asymptotic rate
+      T_selected_by = "heuristic";
+    }
+    if (T <= 0) T = std::max(1L, N);
+    if (has_db && any_remote) pred_t = unit_modeler_list[0]->predict(COCOPELIA_BIDIRECTIONAL, T);
+    else if (has_db) pred_t = unit_modeler_list[0]->exec->predict(T);
+    update_sk_num(sk_num_of(problem, T));
+    distribute_subkernels((int)subkernel_num, 1, 1);
+  }
+  pred_J = -1.0;  // no power sampling on this platform
+  const char* verbose = getenv("PARALIA_VERBOSE");
+  if (verbose && atoi(verbose) > 0) {
+    fprintf(stderr, "====================================\n");
+    fprintf(stderr, "ATC::autotune_problem: %s (%ld,%ld,%ld) -> T = %ld [%s], order %d, %ld subkernels, "
+            "predicted %.3lf ms (h2d %.3lf, exec %.3lf, d2h %.3lf busy)\n", routine_name, problem.D1, problem.D2, problem.D3,
+            T, T_selected_by, order_id, subkernel_num, pred_t * 1000, pipeline.t_h2d_busy * 1000,
+            pipeline.t_exec_busy * 1000, pipeline.t_d2h_busy * 1000);
+    fprintf(stderr, "====================================\n");
+  }
+  return csecond() - timer;
+}
+
+void ATC::print() {
+  fprintf(stderr, "Autotune controller:\n->T = %ld\n->active_unit_num = %d\n->pred_t = %lf\n->subkernel_num = %ld\n"
+          "->cache_limit = %lld\n->order_id = %d\n->T_selected_by = %s\n\n", T, active_unit_num, pred_t, subkernel_num,
+          cache_limit, order_id, T_selected_by);
+}
+
+// "T,active_unit_num,dev_ids_token,cache_limit" -- the first four columns of a runner log row
+// (Autotuner.cpp:839-846; testing.cpp:420-428).
+const char* ATC::print_csv() {
+  char* outstring = (char*)malloc(256 * sizeof(char));
+  int dev_ids_token = 0;
+  if (active_unit_num > 0)
+    for (int i = 0; i < active_unit_num; i++) dev_ids_token += (int)pow(10, idxize(active_unit_id_list[i]));
+  snprintf(outstring, 256, "%ld,%d,%d,%lld", T, active_unit_num, dev_ids_token, cache_limit);
+  return outstring;
+}

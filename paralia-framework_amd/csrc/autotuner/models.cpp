@@ -1,0 +1,150 @@
+// Modeler: per-unit bundle of link models + exec lookup, and the CoCoPeLia overlap predictions.
+// Arithmetic follows the reference's Autotuner/src/ModelLvl3.cpp:20-73 (full overlap), :239-284 (no overlap),
+// :287-346 (baseline), :348-408 (data location), :410-474 (bidirectional), :476-551 (reuse) and
+// ModelLvl1.cpp:262-326 (BLAS-1 bidirectional), reduced to one GPU plus the host.
+#include <cmath>
+#include <cstring>
+
+#include "Autotuner.hpp"
+#include "backend_wrappers.hpp"
+
+Modeler::Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc) : P(desc), unit_id(dev_id) {
+  for (int idx = 0; idx < LOC_NUM; ++idx) {
+    const int other = deidxize(idx);
+    if (other != dev_id) {
+      link[idx] = CoModel_init(db_dir, dev_id, other);     // into this unit (Modeler.cpp:26)
+      revlink[idx] = CoModel_init(db_dir, other, dev_id);  // out of this unit (Modeler.cpp:27)
+    } else {
+      link[idx] = revlink[idx] = CoModel_init_local(dev_id);
+    }
+  }
+  exec = GPUexecModel_init(db_dir, dev_id, desc.func);
+}
+
+Modeler::~Modeler() {
+  for (int idx = 0; idx < LOC_NUM; ++idx) {
+    if (revlink[idx] != link[idx]) delete revlink[idx];
+    delete link[idx];
+  }
+  delete exec;
+}
+
+long Modeler::getMinT() const {
+  if (P.problem == BLAS3) return std::max(exec->MinT(), 1024L);  // MinAllowedTBLAS3
+  return exec->MinT();
+}
+long Modeler::getMaxT() const {
+  if (P.problem == BLAS3) return std::min(std::min(P.D1, P.D2), P.D3);
+  return P.D1;
+}
+long Modeler::getSKNum(long T) const {
+  auto cdiv = [](long a, long b) { return a / b + ((a % b) ? 1 : 0); };
+  if (P.problem == BLAS3) return cdiv(P.D1, T) * cdiv(P.D2, T) * cdiv(P.D3, T);
+  return cdiv(P.D1, T);
+}
+long Modeler::getFlops() const {
+  if (P.problem == BLAS3) return gemm_flops(P.D1, P.D2, P.D3);
+  return axpy_flops(P.D1);
+}
+
+namespace {
+// Dim1 x Dim2 of operand i: A is D1 x D3, B is D3 x D2, C is D1 x D2 (CoCoModel_gemm_init); vectors are D1 x 1.
+void dims_of(const ProblemDesc& P, int i, double* d1, double* d2) {
+  if (P.problem != BLAS3) { *d1 = (double)P.D1; *d2 = 1; return; }
+  *d1 = (i == 1) ? (double)P.D3 : (double)P.D1;
+  *d2 = (i == 0) ? (double)P.D3 : (double)P.D2;
+}
+}  // namespace
+
+double Modeler::predict(ModelType mode, long T) const {
+  // The location that prices a tile transfer is the one holding the most operands, the host winning ties
+  // (ModelLvl3.cpp:306-312): with one GPU that is the host unless the device holds strictly more.
+  int on_host = 0;
+  for (int i = 0; i < P.numT; ++i) on_host += remote(P.loc[i], unit_id);
+  const int mv_idx = (on_host >= P.numT - on_host) ? idxize(-1) : idxize(unit_id);
+  const comm_data* recv_m = link[mv_idx];
+  const comm_data* send_m = revlink[mv_idx];
+
+  if (P.problem == BLAS1) {
+    if (mode != COCOPELIA_BIDIRECTIONAL) error("Modeler::predict: BLAS-1 supports only COCOPELIA_BIDIRECTIONAL\n");
+    const double t_exec = exec->predict(T);
+    if (t_exec < 0) return -1.0;
+    const double bytes = (double)T * P.dtype_sz;
+    const double t_recv = t_com_predict(recv_m, bytes), t_send = t_com_predict(send_m, bytes);
+    int numTin = 0, numTout = 0;
+    for (int i = 0; i < P.numT; ++i) {
+      numTin += P.in[i] * remote(P.loc[i], unit_id);
+      numTout += P.out[i] * remote(P.loc[i], unit_id);
+    }
+    const double ker_over = (1.0 * P.D1 / T) - 1;
+    const double t_over = t_com_bid_predict(recv_m, send_m, bytes * numTin, bytes * numTout);
+    return fmax(t_exec, t_over) * ker_over + fmax(t_exec, numTout * t_send) + numTin * t_recv + numTout * t_send;
+  }
+
+  if (mode == FULL_OVERLAP || mode == NO_OVERLAP) {
+    const long maxT = exec->MaxT();
+    const long Tbig = exec->NearestT((long)fmin((double)maxT, fmin(fmin((double)P.D1, (double)P.D2), (double)P.D3)));
+    const double t_exec = (P.D1 * 1.0 / Tbig * P.D2 * 1.0 / Tbig * P.D3 * 1.0 / Tbig) * exec->predict(Tbig, P.TransA, P.TransB);
+    if (t_exec < 0) return -1.0;
+    double t_recv = 0, t_send = 0;
+    for (int i = 0; i < P.numT; ++i) {
+      double d1, d2;
+      dims_of(P, i, &d1, &d2);
+      // the reference prices both directions with the same (receive-side) link model here
+      t_recv += P.in[i] * t_com_predict(link[idxize(P.loc[i])], d1 * d2 * P.dtype_sz);
+      t_send += P.out[i] * t_com_predict(link[idxize(P.out_loc[i])], d1 * d2 * P.dtype_sz);
+    }
+    return mode == FULL_OVERLAP ? fmax(t_exec, fmax(t_recv, t_send)) : t_exec + t_recv + t_send;
+  }
+
+  const double t_exec = exec->predict(T, P.TransA, P.TransB);
+  if (t_exec < 0) return -1.0;
+  const double tile_bytes = (double)T * T * P.dtype_sz;
+  const double t_recv = t_com_predict(recv_m, tile_bytes), t_send = t_com_predict(send_m, tile_bytes);
+  const double ker_over = (1.0 * P.D1 / T) * (1.0 * P.D2 / T) * (1.0 * P.D3 / T) - 1;
+  int numTin = 0, numTout = 0;
+
+  switch (mode) {
+    case COCOPELIA_BASELINE: {
+      for (int i = 0; i < P.numT; ++i) { numTin += P.in[i]; numTout += P.out[i]; }
+      const double t_over = fmax(numTin * t_recv, t_send * numTout);
+      return fmax(t_exec, t_over) * ker_over + t_exec + numTin * t_recv + numTout * t_send;
+    }
+    case COCOPELIA_DATALOC:
+    case COCOPELIA_BIDIRECTIONAL: {
+      for (int i = 0; i < P.numT; ++i) {
+        numTin += P.in[i] * remote(P.loc[i], unit_id);
+        numTout += P.out[i] * remote(P.loc[i], unit_id);
+      }
+      const double t_over = (mode == COCOPELIA_DATALOC)
+                                ? fmax(numTin * t_recv, t_send * numTout)
+                                : t_com_bid_predict(recv_m, send_m, tile_bytes * numTin, tile_bytes * numTout);
+      return fmax(t_exec, t_over) * ker_over + t_exec + numTin * t_recv + numTout * t_send;
+    }
+    case COCOPELIA_REUSE: {
+      double zero_over = ker_over, one_over = 0, two_over = 0;
+      for (int i = 0; i < P.numT; ++i) {
+        double d1, d2;
+        dims_of(P, i, &d1, &d2);
+        const int rin = P.in[i] * remote(P.loc[i], unit_id);
+        numTin += rin;
+        numTout += P.out[i] * remote(P.out_loc[i], unit_id);
+        one_over += rin * (d1 / T) * (d2 / T);
+        if (t_recv > t_exec)
+          for (int j = i + 1; j < P.numT; ++j)
+            if (rin && P.in[j] * remote(P.loc[j], unit_id)) {
+              // tiles of operands i and j that can be fetched under one kernel share a dimension:
+              // A-C share D1 (= Dim1 of A); A-B share D3 and B-C share D2 (= Dim2 of the first)
+              two_over += ((i == 0 && j == 2) ? d1 : d2) / T - 1;
+            }
+      }
+      if (2 * t_recv > t_exec && t_exec > t_recv) two_over += (1.0 * P.D3 / T);
+      one_over -= (2 * two_over + numTin);
+      zero_over -= (one_over + two_over);
+      return t_exec * (1 + zero_over) + fmax(t_exec, t_recv) * one_over + fmax(t_exec, t_recv * 2) * two_over +
+             numTin * t_recv + numTout * t_send;
+    }
+    default:
+      error("Modeler::predict: mode %s not available\n", printModel(mode));
+  }
+}

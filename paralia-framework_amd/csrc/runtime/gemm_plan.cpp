@@ -1,0 +1,327 @@
+// Static GEMM plan: order families, block assignment with farthest-next-use eviction, dependency edges, and
+// the three-resource pipeline simulation used to choose among orders (and, by the autotuner, among tile sizes).
+#include "gemm_plan.hpp"
+
+#include <algorithm>
+#include <climits>
+#include <deque>
+#include <stdexcept>
+#include <string>
+
+namespace paralia {
+
+std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
+  const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
+  const int orient = order_id / 10000;
+  int w = order_id % 10000;
+  std::vector<int> order;
+  order.reserve((size_t)Mg * Ng * Kg);
+  auto id = [&](int mi, int ni, int ki) { return (mi * Ng + ni) * Kg + ki; };
+  if (orient == 0) {
+    w = std::min(w, Ng);
+    for (int ki = 0; ki < Kg; ++ki)
+      for (int ni = 0; ni < w; ++ni)
+        for (int mi = 0; mi < Mg; ++mi) order.push_back(id(mi, ni, ki));
+    for (int ni = w; ni < Ng; ++ni)
+      for (int mi = 0; mi < Mg; ++mi)
+        for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+  } else {
+    w = std::min(w, Mg);
+    for (int ki = 0; ki < Kg; ++ki)
+      for (int mi = 0; mi < w; ++mi)
+        for (int ni = 0; ni < Ng; ++ni) order.push_back(id(mi, ni, ki));
+    for (int mi = w; mi < Mg; ++mi)
+      for (int ni = 0; ni < Ng; ++ni)
+        for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+  }
+  return order;
+}
+
+std::vector<int> gemm_candidate_orders(const GemmProblem& p) {
+  std::vector<int> ids;
+  ids.push_back(order_id_of(1, 0));  // the reference's index order; needs the fewest blocks
+  if (!(p.a_remote || p.b_remote || p.c_remote)) return ids;
+  static const int widths[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 48, 64};
+  for (int orient = 0; orient < 2; ++orient) {
+    const int g = orient == 0 ? p.Ng() : p.Mg();
+    if (orient == 0) ids.push_back(order_id_of(0, 0));
+    for (int w : widths)
+      if (w < g) ids.push_back(order_id_of(orient, w));
+    ids.push_back(order_id_of(orient, g));
+  }
+  return ids;
+}
+
+long gemm_full_block_num(const GemmProblem& p) {
+  const long a = (long)p.Mg() * p.Kg(), b = (long)p.Kg() * p.Ng(), c = (long)p.Mg() * p.Ng();
+  // dgemm.cpp:80-82: one spare block plus every tile of A, B and C, plus C once more for the lazy write-back.
+  return 1 + a + b + 2 * c;
+}
+
+namespace {
+
+struct Block {
+  int kind = -1;  // -1 free, 0 A tile, 1 B tile, 2 accumulator, 3 source C
+  int idx = -1;
+  int content_cmd = -1;        // command after which the content is valid (the fetch)
+  std::vector<int> pending;    // commands that must complete before the block may be overwritten
+  bool ever_used = false;
+};
+
+void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w) {
+  if (w < 0) return;
+  if (cmds[w].stream == c.stream) return;  // stream order already covers it
+  for (int i = 0; i < c.nwait; ++i)
+    if (c.wait[i] == w) return;
+  if (c.nwait >= MAX_WAITS) throw std::runtime_error("gemm plan: too many dependencies on one command");
+  c.wait[c.nwait++] = w;
+  cmds[w].signals = true;
+}
+
+}  // namespace
+
+GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
+  if (p.T <= 0 || p.M <= 0 || p.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
+  GemmPlan plan;
+  plan.p = p;
+  plan.order_id = order_id;
+  plan.task_order = gemm_task_order(p, order_id);
+  const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
+  const int NQ = std::max(1, std::min(p.exec_queues, MAX_EXEC_QUEUES));
+  const bool any_remote = p.a_remote || p.b_remote || p.c_remote;
+  if (any_remote && p.pool_blocks < 3)
+    throw std::runtime_error("PARALiA gemm: Not able to run with < 3 blocks per cache");
+
+  // positions at which every A / B tile is used, for farthest-next-use eviction
+  std::vector<std::vector<int>> a_uses((size_t)Mg * Kg), b_uses((size_t)Kg * Ng);
+  for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
+    const int t = plan.task_order[pos];
+    const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
+    a_uses[(size_t)mi * Kg + ki].push_back(pos);
+    b_uses[(size_t)ki * Ng + ni].push_back(pos);
+  }
+  std::vector<int> a_ptr(a_uses.size(), 0), b_ptr(b_uses.size(), 0);
+  std::vector<int> a_blk(a_uses.size(), -1), b_blk(b_uses.size(), -1), c_blk((size_t)Mg * Ng, -1);
+  std::vector<int> fired((size_t)Mg * Ng, 0), queue_of((size_t)Mg * Ng, 0);
+  std::vector<Block> blocks((size_t)(any_remote ? p.pool_blocks : 0));
+  // FIFO: never-used blocks first, then released blocks oldest first, so a recycled block's previous users
+  // (a write-back still in flight, say) have had the longest time to finish before its new writer waits on them
+  std::deque<int> free_list;
+  for (int b = 0; b < (int)blocks.size(); ++b) free_list.push_back(b);
+  int c_seq = 0;
+  std::vector<Cmd>& cmds = plan.cmds;
+  cmds.reserve(plan.task_order.size() * 2 + 16);
+
+  auto release = [&](int b, int after_cmd) {
+    blocks[b].kind = -1;
+    blocks[b].idx = -1;
+    blocks[b].pending.assign(1, after_cmd);
+    free_list.push_back(b);
+  };
+
+  // Returns a block whose previous content may be dropped; "waits" receives what a writer must wait for.
+  auto alloc = [&](int pin1, int pin2, std::vector<int>& waits) -> int {
+    int b = -1;
+    if (!free_list.empty()) {
+      b = free_list.front();
+      free_list.pop_front();
+    } else {
+      int best_next = -1;
+      for (int i = 0; i < (int)blocks.size(); ++i) {
+        if (i == pin1 || i == pin2) continue;
+        int next;
+        if (blocks[i].kind == 0) {
+          const auto& u = a_uses[blocks[i].idx];
+          next = a_ptr[blocks[i].idx] < (int)u.size() ? u[a_ptr[blocks[i].idx]] : INT_MAX;
+        } else if (blocks[i].kind == 1) {
+          const auto& u = b_uses[blocks[i].idx];
+          next = b_ptr[blocks[i].idx] < (int)u.size() ? u[b_ptr[blocks[i].idx]] : INT_MAX;
+        } else {
+          continue;  // accumulators and source-C blocks are exclusive: never evicted
+        }
+        if (next > best_next) {
+          best_next = next;
+          b = i;
+        }
+      }
+      if (b < 0) throw std::runtime_error("PARALiA gemm: device block pool too small for this subkernel order");
+      if (blocks[b].kind == 0) a_blk[blocks[b].idx] = -1;
+      else b_blk[blocks[b].idx] = -1;
+      ++plan.n_evictions;
+    }
+    waits.insert(waits.end(), blocks[b].pending.begin(), blocks[b].pending.end());
+    blocks[b].pending.clear();
+    blocks[b].ever_used = true;
+    return b;
+  };
+
+  auto note_reader = [&](int b, int cmd_idx) {
+    // one pending reader per stream is enough: streams run their commands in order
+    auto& pend = blocks[b].pending;
+    for (int& w : pend)
+      if (cmds[w].stream == cmds[cmd_idx].stream) {
+        w = cmd_idx;
+        return;
+      }
+    pend.push_back(cmd_idx);
+  };
+
+  for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
+    const int t = plan.task_order[pos];
+    const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
+    const int ai = mi * Kg + ki, bi = ki * Ng + ni, ci = mi * Ng + ni;
+    ++a_ptr[ai];
+    ++b_ptr[bi];
+    int ablk = -1, bblk = -1;
+    std::vector<int> gemm_waits;
+
+    if (p.a_remote) {
+      if (a_blk[ai] < 0) {
+        std::vector<int> w;
+        const int b = alloc(p.b_remote ? b_blk[bi] : -1, -1, w);
+        Cmd c;
+        c.kind = CMD_FETCH_A; c.mi = mi; c.ki = ki; c.stream = STREAM_H2D; c.block = b;
+        cmds.push_back(c);
+        for (int x : w) add_wait(cmds, cmds.back(), x);
+        blocks[b].kind = 0; blocks[b].idx = ai; blocks[b].content_cmd = (int)cmds.size() - 1;
+        a_blk[ai] = b;
+        ++plan.n_fetch[0];
+      }
+      ablk = a_blk[ai];
+      gemm_waits.push_back(blocks[ablk].content_cmd);
+    }
+    if (p.b_remote) {
+      if (b_blk[bi] < 0) {
+        std::vector<int> w;
+        const int b = alloc(ablk, -1, w);
+        Cmd c;
+        c.kind = CMD_FETCH_B; c.ki = ki; c.ni = ni; c.stream = STREAM_H2D; c.block = b;
+        cmds.push_back(c);
+        for (int x : w) add_wait(cmds, cmds.back(), x);
+        blocks[b].kind = 1; blocks[b].idx = bi; blocks[b].content_cmd = (int)cmds.size() - 1;
+        b_blk[bi] = b;
+        ++plan.n_fetch[1];
+      }
+      bblk = b_blk[bi];
+      gemm_waits.push_back(blocks[bblk].content_cmd);
+    }
+
+    int beta_mode = BETA_ONE;
+    if (fired[ci] == 0) {
+      // reference: each C tile's K-chain is pinned to one exec queue, handed out round-robin (Subkernel.cpp:18-22)
+      queue_of[ci] = c_seq++ % NQ;
+      if (p.c_remote) {
+        const int b = alloc(ablk, bblk, gemm_waits);
+        blocks[b].kind = 2; blocks[b].idx = ci;
+        c_blk[ci] = b;
+        beta_mode = BETA_ZERO;  // lazy write-back: accumulate locally first (dgemm.cpp:273-279)
+      } else {
+        beta_mode = BETA_USER;  // resident C: plain read-modify-write (dgemm.cpp:259-260)
+      }
+    }
+    {
+      Cmd c;
+      c.kind = CMD_GEMM; c.mi = mi; c.ni = ni; c.ki = ki; c.stream = STREAM_EXEC0 + queue_of[ci];
+      c.block = p.c_remote ? c_blk[ci] : -1; c.a_block = ablk; c.b_block = bblk; c.beta_mode = beta_mode;
+      cmds.push_back(c);
+      for (int x : gemm_waits) add_wait(cmds, cmds.back(), x);
+    }
+    const int gemm_idx = (int)cmds.size() - 1;
+    if (ablk >= 0) note_reader(ablk, gemm_idx);
+    if (bblk >= 0) note_reader(bblk, gemm_idx);
+
+    if (++fired[ci] == Kg && p.c_remote) {
+      const int accb = c_blk[ci];
+      int last = gemm_idx;
+      if (!p.beta_zero) {
+        // lazy reduce: fetch the caller's tile now, out = beta * src + acc (dgemm.cpp:173-179)
+        std::vector<int> w;
+        const int sb = alloc(accb, -1, w);
+        Cmd f;
+        f.kind = CMD_FETCH_C; f.mi = mi; f.ni = ni; f.stream = STREAM_H2D; f.block = sb;
+        cmds.push_back(f);
+        for (int x : w) add_wait(cmds, cmds.back(), x);
+        const int fetch_idx = (int)cmds.size() - 1;
+        blocks[sb].kind = 3; blocks[sb].idx = ci; blocks[sb].content_cmd = fetch_idx;
+        ++plan.n_fetch[2];
+        Cmd r;
+        r.kind = CMD_REDUCE; r.mi = mi; r.ni = ni; r.stream = STREAM_EXEC0 + queue_of[ci]; r.block = accb; r.a_block = sb;
+        cmds.push_back(r);
+        add_wait(cmds, cmds.back(), fetch_idx);
+        last = (int)cmds.size() - 1;
+        release(sb, last);
+      }
+      Cmd wb;
+      wb.kind = CMD_WRITEBACK; wb.mi = mi; wb.ni = ni; wb.stream = STREAM_D2H; wb.block = accb;
+      cmds.push_back(wb);
+      add_wait(cmds, cmds.back(), last);
+      release(accb, (int)cmds.size() - 1);
+      c_blk[ci] = -1;
+    }
+  }
+  for (const Block& b : blocks) plan.blocks_used += b.ever_used ? 1 : 0;
+  return plan;
+}
+
+PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
+  const GemmProblem& p = plan.p;
+  const double T2 = (double)p.T * p.T, T3 = T2 * p.T;
+  std::vector<double> finish(plan.cmds.size(), 0.0);
+  double h2d = 0, d2h = 0, exec = 0;
+  double qclock[MAX_EXEC_QUEUES] = {0};
+  PipelineResult r;
+  for (size_t i = 0; i < plan.cmds.size(); ++i) {
+    const Cmd& c = plan.cmds[i];
+    double ready = 0;
+    for (int w = 0; w < c.nwait; ++w) ready = std::max(ready, finish[c.wait[w]]);
+    double dur = 0;
+    switch (c.kind) {
+      case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
+      case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
+      case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+      case CMD_GEMM: dur = st.t_exec * ((double)p.tm(c.mi) * p.tn(c.ni) * std::max(1L, p.tk(c.ki))) / T3; break;
+      case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
+      case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+    }
+    if (c.stream == STREAM_H2D) {
+      const double s = std::max(ready, h2d);
+      finish[i] = h2d = s + dur;
+      r.t_h2d += dur;
+    } else if (c.stream == STREAM_D2H) {
+      const double s = std::max(ready, d2h);
+      finish[i] = d2h = s + dur;
+      r.t_d2h += dur;
+    } else {
+      // exec queues are in-order each and share the one compute resource
+      const int q = c.stream - STREAM_EXEC0;
+      const double s = std::max(std::max(ready, qclock[q]), exec);
+      finish[i] = qclock[q] = exec = s + dur;
+      r.t_exec += dur;
+    }
+    r.t_total = std::max(r.t_total, finish[i]);
+  }
+  return r;
+}
+
+int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best_out) {
+  int best_id = -1;
+  PipelineResult best;
+  std::string last_err;
+  for (int id : gemm_candidate_orders(p)) {
+    try {
+      GemmPlan plan = build_gemm_plan(p, id);
+      PipelineResult r = simulate_plan(plan, st);
+      if (best_id < 0 || r.t_total < best.t_total * (1.0 - 1e-9)) {
+        best = r;
+        best_id = id;
+      }
+    } catch (const std::runtime_error& e) {
+      last_err = e.what();  // this order does not fit the pool; others may
+    }
+  }
+  if (best_id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
+  if (best_out) *best_out = best;
+  return best_id;
+}
+
+}  // namespace paralia

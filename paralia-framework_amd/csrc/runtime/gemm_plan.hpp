@@ -1,0 +1,94 @@
+// Static plan of one tiled GEMM call on one GPU: subkernel order, device-block assignment (with eviction when
+// the pool is smaller than the working set) and the cross-stream dependencies, all decided on the host before
+// anything is enqueued.  Pure host logic -- no HIP types -- so it is unit-tested without a GPU.
+//
+// Where the reference does this work: subkernel creation and beta schedule in
+// Library_scheduler/src/Functions/dgemm.cpp:123-205,273-279; block grabbing and tile fetch in
+// Subkernel.cpp:90-135; readiness polling and launch in Subkernel.cpp:192-247 and dgemm.cpp:290-314;
+// subkernel choice in Subkernel.cpp:384-448; write-back in Subkernel_backup.cpp:1128-1260.
+// The reference decides these dynamically with a manager thread polling events every 100 us; here the order
+// is fixed up front from a simulated H2D / compute / D2H pipeline and the dependencies are handed to the HIP
+// streams as event waits, so the host never polls.
+#ifndef PARALIA_GEMM_PLAN_HPP
+#define PARALIA_GEMM_PLAN_HPP
+
+#include <vector>
+
+namespace paralia {
+
+constexpr int MAX_EXEC_QUEUES = 8;  // MAX_BACKEND_L of the reference (CMakeLists.txt:69)
+constexpr int MAX_WAITS = 2 + MAX_EXEC_QUEUES + 2;
+
+struct GemmProblem {
+  long M = 0, N = 0, K = 0, T = 0;
+  bool a_remote = true, b_remote = true, c_remote = true;  // operand lives off the device
+  bool beta_zero = false;                                    // caller's beta == 0: C is never fetched
+  int elem = 8;                                              // bytes per element
+  int exec_queues = 2;
+  long pool_blocks = 0;                                      // device blocks available (>= 3 when anything is remote)
+  int Mg() const { return (int)((M + T - 1) / T); }
+  int Ng() const { return (int)((N + T - 1) / T); }
+  int Kg() const { return K > 0 ? (int)((K + T - 1) / T) : 1; }
+  long tm(int mi) const { return mi == Mg() - 1 ? M - (long)mi * T : T; }
+  long tn(int ni) const { return ni == Ng() - 1 ? N - (long)ni * T : T; }
+  long tk(int ki) const { return K <= 0 ? 0 : (ki == Kg() - 1 ? K - (long)ki * T : T); }
+  long subkernels() const { return (long)Mg() * Ng() * Kg(); }
+};
+
+enum CmdKind : int { CMD_FETCH_A = 0, CMD_FETCH_B = 1, CMD_FETCH_C = 2, CMD_GEMM = 3, CMD_REDUCE = 4, CMD_WRITEBACK = 5 };
+enum : int { STREAM_H2D = 0, STREAM_D2H = 1, STREAM_EXEC0 = 2 };
+enum : int { BETA_ZERO = 0, BETA_ONE = 1, BETA_USER = 2 };
+
+struct Cmd {
+  int kind = 0;
+  int mi = -1, ni = -1, ki = -1;  // FETCH_A: (mi, ki); FETCH_B: (ki, ni); everything on C: (mi, ni)
+  int stream = 0;
+  int block = -1;     // block written by a FETCH; accumulator block of GEMM / REDUCE / WRITEBACK (-1: caller's C)
+  int a_block = -1;   // GEMM: block of the A tile (-1: caller's memory); REDUCE: block holding the fetched source C
+  int b_block = -1;   // GEMM: block of the B tile (-1: caller's memory)
+  int beta_mode = BETA_ONE;
+  int nwait = 0;
+  int wait[MAX_WAITS];  // earlier commands on other streams that must have completed
+  bool signals = false; // some later command on another stream waits on this one
+};
+
+struct GemmPlan {
+  GemmProblem p;
+  int order_id = 0;
+  std::vector<int> task_order;  // subkernel ids mi*Ng*Kg + ni*Kg + ki in firing order
+  std::vector<Cmd> cmds;
+  long blocks_used = 0;
+  long n_fetch[3] = {0, 0, 0};  // A, B, C tile fetches issued (re-fetches after eviction included)
+  long n_evictions = 0;
+};
+
+// Order families.  id = orient * 10000 + w.  orient 0: the first w column-tiles of C are processed as one
+// panel in k-outer (outer-product) order, the remaining columns tile by tile (ni, mi, ki);
+// orient 1: the same with row-tiles (remaining rows in the reference's index order mi, ni, ki).
+// w = 0 with orient 1 is exactly the reference's subkernel index order (dgemm.cpp:139-142).
+inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
+std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
+std::vector<int> gemm_candidate_orders(const GemmProblem& p);
+
+// Throws std::runtime_error when pool_blocks cannot hold the minimum working set (3 blocks, dgemm.cpp:90-93).
+GemmPlan build_gemm_plan(const GemmProblem& p, int order_id);
+
+// Block pool size the reference would ask for (dgemm.cpp:23-36,80-82).
+long gemm_full_block_num(const GemmProblem& p);
+
+// Stage costs of a full T x T (x T) tile; edge tiles scale with their area / volume.
+struct StageTimes {
+  double t_exec = 0;                 // one T^3 subkernel
+  double h2d_ti = 0, h2d_tb = 0;     // seconds, seconds per byte
+  double d2h_ti = 0, d2h_tb = 0;
+  double t_reduce = 0;               // one T^2 scale-add
+};
+struct PipelineResult {
+  double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource
+};
+PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st);
+// Builds every candidate order, simulates it, returns the id with the smallest makespan.
+int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best);
+
+}  // namespace paralia
+#endif

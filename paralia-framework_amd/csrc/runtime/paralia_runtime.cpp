@@ -1,0 +1,577 @@
+// PARALiA routines on one MI355X: argument checks, operand location detection, problem-metadata cache, device
+// block pool, stream/event inventory and the executor that turns a static GEMM plan into HIP stream work.
+//
+// Reference counterparts: Library_scheduler/src/Functions/dgemm.cpp:318-705 (PARALiADgemm: metadata cache
+// :342-368, decomposition :409-440, cache sizing :23-121, fire loop :512-546, sync :596-597, reuse :627-649),
+// sgemm.cpp:296, daxpy.cpp:200, ddot.cpp:201, Subkernel.cpp:249-306 (queue inventory), :488 (cache free).
+// All device work goes through the C ABI in paralia_hip.h; this file includes no HIP header.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "PARALiA.hpp"
+#include "backend_wrappers.hpp"
+#include "gemm_plan.hpp"
+#include "paralia_hip.h"
+
+namespace paralia {
+
+static void chk(int rc, const char* what) {
+  if (rc != 0) throw paralia_error(rc, std::string(what) + " failed: " + (rc == PL_ERR_HIP ? pl_last_error() : "invalid argument"));
+}
+
+// ------------------------------------------------------------------------------------------ block pool
+// Equal-size device blocks, kept between calls (the reference's Buffer with BUFFER_REUSE_ENABLE,
+// dgemm.cpp:95-117): reallocated only when the block size changes or more blocks are needed.
+struct DevicePool {
+  void* base = nullptr;
+  long long block_sz = 0;
+  long blocks = 0;
+  long long bytes() const { return block_sz * blocks; }
+  void* at(long b) const { return (char*)base + block_sz * b; }
+  void ensure(long need_blocks, long long need_block_sz) {
+    if (base && block_sz == need_block_sz && blocks >= need_blocks) return;
+    release();
+    chk(pl_malloc_device(&base, need_block_sz * need_blocks), "device block pool allocation");
+    block_sz = need_block_sz;
+    blocks = need_blocks;
+  }
+  void release() {
+    if (base) chk(pl_free_device(base), "device block pool free");
+    base = nullptr;
+    block_sz = 0;
+    blocks = 0;
+  }
+};
+
+// ------------------------------------------------------------------------------- streams, events, scratch
+// One H2D stream, one D2H stream, up to MAX_BACKEND_L compute streams (Subkernel.cpp:249-306 keeps
+// recv/wb queues per link and 8 exec queues per device); created once and reused (BACKEND_RES_REUSE_ENABLE).
+struct Resources {
+  void* h2d = nullptr;
+  void* d2h = nullptr;
+  void* exec[MAX_EXEC_QUEUES] = {nullptr};
+  int nexec = 0;
+  std::vector<void*> events;
+  double* dot_ws = nullptr;      // ddot partials
+  double* dot_result = nullptr;  // device scalar
+  double* dot_host = nullptr;    // pinned scalar
+  void ensure_streams(int nq) {
+    if (!h2d) chk(pl_stream_create(&h2d), "stream create");
+    if (!d2h) chk(pl_stream_create(&d2h), "stream create");
+    for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
+  }
+  void ensure_events(size_t n) {
+    while (events.size() < n) {
+      void* e = nullptr;
+      chk(pl_event_create(&e, 0), "event create");
+      events.push_back(e);
+    }
+  }
+  void ensure_dot() {
+    if (dot_ws) return;
+    void* p = nullptr;
+    chk(pl_malloc_device(&p, (pl_ddot_workspace_doubles() + 8) * (long long)sizeof(double)), "ddot workspace");
+    dot_ws = (double*)p;
+    dot_result = dot_ws + pl_ddot_workspace_doubles();
+    chk(pl_malloc_pinned(&p, 64), "ddot host scalar");
+    dot_host = (double*)p;
+  }
+  void* stream(int id) const { return id == STREAM_H2D ? h2d : id == STREAM_D2H ? d2h : exec[id - STREAM_EXEC0]; }
+  void sync_all() {
+    if (h2d) chk(pl_stream_sync(h2d), "stream sync");
+    for (int q = 0; q < nexec; ++q) chk(pl_stream_sync(exec[q]), "stream sync");
+    if (d2h) chk(pl_stream_sync(d2h), "stream sync");
+  }
+  void destroy() {
+    if (h2d) pl_stream_destroy(h2d);
+    if (d2h) pl_stream_destroy(d2h);
+    for (int q = 0; q < nexec; ++q) pl_stream_destroy(exec[q]);
+    for (void* e : events) pl_event_destroy(e);
+    if (dot_ws) pl_free_device(dot_ws);
+    if (dot_host) pl_free_pinned(dot_host);
+    *this = Resources();
+  }
+};
+
+// ------------------------------------------------------------------------------------ metadata cache
+struct PMDKey {
+  std::string routine;
+  char ta = 'N', tb = 'N';
+  long D1 = 0, D2 = 0, D3 = 0;
+  int loc[3] = {0, 0, 0};
+  bool beta_zero = false;
+  long predef_T = -1;
+  long long cache_limit = 0;
+  bool operator==(const PMDKey& o) const {
+    return routine == o.routine && ta == o.ta && tb == o.tb && D1 == o.D1 && D2 == o.D2 && D3 == o.D3 && loc[0] == o.loc[0] &&
+           loc[1] == o.loc[1] && loc[2] == o.loc[2] && beta_zero == o.beta_zero && predef_T == o.predef_T &&
+           cache_limit == o.cache_limit;
+  }
+};
+struct PMDEntry {
+  PMDKey key;
+  std::unique_ptr<ATC> atc;
+  GemmPlan plan;
+};
+
+struct Runtime {
+  std::mutex mu;  // serialises calls: the routines are not re-entrant (file-scope state in the reference too)
+  DevicePool pool;
+  Resources res;
+  std::vector<std::unique_ptr<PMDEntry>> pmd;  // at most PROBLEM_MD_CACHE entries, oldest dropped first
+  long pmd_hits = 0, pmd_misses = 0;
+};
+static Runtime& rt() {
+  static Runtime r;
+  return r;
+}
+
+static int host_or_dev(int loc) { return loc >= 0 ? 0 : -1; }  // the scheduler routes by "on device 0" vs "host"
+
+static long long pool_budget(long long cache_limit, long long prev_pool_bytes) {
+  long long free_b = 0, total_b = 0;
+  chk(pl_mem_info(&free_b, &total_b), "mem info");
+  // dgemm.cpp:73-78: leave (100 - PROBLEM_GPU_PERCENTAGE)% of the device alone; the old pool is reusable
+  long long budget = free_b - (long long)(total_b * (1 - PROBLEM_GPU_PERCENTAGE / 100.0)) + prev_pool_bytes;
+  if (cache_limit > 0) budget = std::min(budget, cache_limit);
+  return std::max(budget, 0LL);
+}
+
+static ATC_p atc_copy(ATC* src) {
+  ATC_p out = new ATC();
+  out->mimic_ATC(src);
+  return out;
+}
+
+// ------------------------------------------------------------------------------------------- GEMM
+template <typename T> struct GemmFns;
+template <> struct GemmFns<double> {
+  static constexpr const char* name = "Dgemm";
+  static int tile(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
+                  double be, double* C, long ldc, void* s) { return pl_dgemm_tile(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, s); }
+  static int geadd(long M, long N, double be, const double* s, long lds, const double* a, long lda, double* o, long ldo, void* st) {
+    return pl_dgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
+  }
+};
+template <> struct GemmFns<float> {
+  static constexpr const char* name = "Sgemm";
+  static int tile(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
+                  float be, float* C, long ldc, void* s) { return pl_sgemm_tile(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, s); }
+  static int geadd(long M, long N, float be, const float* s, long lds, const float* a, long lda, float* o, long ldo, void* st) {
+    return pl_sgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
+  }
+};
+
+template <typename T>
+static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb, T alpha, const T* A, long lda, const T* B,
+                              long ldb, T beta, T* C, long ldc) {
+  const GemmProblem& p = plan.p;
+  const bool at = (ta == 'T'), bt = (tb == 'T');
+  const long Tt = p.T;
+  R.res.ensure_streams(std::max(1, std::min(p.exec_queues, MAX_EXEC_QUEUES)));
+  size_t nsig = 0;
+  for (const Cmd& c : plan.cmds) nsig += c.signals ? 1 : 0;
+  R.res.ensure_events(nsig);
+  std::vector<void*> ev(plan.cmds.size(), nullptr);
+  size_t next_ev = 0;
+
+  for (size_t i = 0; i < plan.cmds.size(); ++i) {
+    const Cmd& c = plan.cmds[i];
+    void* s = R.res.stream(c.stream);
+    for (int w = 0; w < c.nwait; ++w) chk(pl_stream_wait_event(s, ev[c.wait[w]]), "stream wait event");
+    switch (c.kind) {
+      case CMD_FETCH_A: {
+        const long rows = at ? p.tk(c.ki) : p.tm(c.mi), cols = at ? p.tm(c.mi) : p.tk(c.ki);
+        const T* src = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda;
+        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, lda, rows, cols, sizeof(T), s), "fetch A tile");
+      } break;
+      case CMD_FETCH_B: {
+        const long rows = bt ? p.tn(c.ni) : p.tk(c.ki), cols = bt ? p.tk(c.ki) : p.tn(c.ni);
+        const T* src = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb;
+        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
+      } break;
+      case CMD_FETCH_C: {
+        const long rows = p.tm(c.mi), cols = p.tn(c.ni);
+        const T* src = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
+        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
+      } break;
+      case CMD_GEMM: {
+        const long m = p.tm(c.mi), n = p.tn(c.ni), k = p.tk(c.ki);
+        const T* a;
+        long la;
+        if (c.a_block >= 0) { a = (const T*)R.pool.at(c.a_block); la = at ? k : m; }
+        else { a = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda; la = lda; }
+        const T* b;
+        long lb;
+        if (c.b_block >= 0) { b = (const T*)R.pool.at(c.b_block); lb = bt ? n : k; }
+        else { b = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb; lb = ldb; }
+        T* cc;
+        long lc;
+        if (c.block >= 0) { cc = (T*)R.pool.at(c.block); lc = m; }
+        else { cc = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc; lc = ldc; }
+        const T bp = c.beta_mode == BETA_ZERO ? T(0) : c.beta_mode == BETA_ONE ? T(1) : beta;
+        if (la < 1) la = 1;
+        if (lb < 1) lb = 1;
+        chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, s), "tile gemm launch");
+      } break;
+      case CMD_REDUCE: {
+        const long m = p.tm(c.mi), n = p.tn(c.ni);
+        T* acc = (T*)R.pool.at(c.block);
+        chk(GemmFns<T>::geadd(m, n, beta, (const T*)R.pool.at(c.a_block), m, acc, m, acc, m, s), "lazy reduce launch");
+      } break;
+      case CMD_WRITEBACK: {
+        const long m = p.tm(c.mi), n = p.tn(c.ni);
+        T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
+        chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
+      } break;
+    }
+    if (c.signals) {
+      ev[i] = R.res.events[next_ev++];
+      chk(pl_event_record(ev[i], s), "event record");
+    }
+  }
+  R.res.sync_all();
+}
+
+template <typename T>
+static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alpha, T* A, long ldA, T* B, long ldB, T beta,
+                        T* C, long ldC, ATC_p predef) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  const char ta = (char)toupper(TransA), tb = (char)toupper(TransB);
+  if ((ta != 'N' && ta != 'T') || (tb != 'N' && tb != 'T'))
+    error("PARALiA%s: invalid transpose flags '%c','%c' (only N and T)\n", GemmFns<T>::name, TransA, TransB);
+  if (M < 0 || N < 0 || K < 0) error("PARALiA%s: negative dimension (M=%ld N=%ld K=%ld)\n", GemmFns<T>::name, M, N, K);
+  const long rowsA = ta == 'N' ? M : K, rowsB = tb == 'N' ? K : N;
+  if (ldA < std::max(1L, rowsA) || ldB < std::max(1L, rowsB) || ldC < std::max(1L, M))
+    error("PARALiA%s: leading dimension too small (ldA=%ld ldB=%ld ldC=%ld)\n", GemmFns<T>::name, ldA, ldB, ldC);
+
+  int prev_dev = 0;
+  chk(pl_get_device(&prev_dev), "get device");
+  if (prev_dev != 0) chk(pl_set_device(0), "set device");
+  struct Restore { int d; ~Restore() { if (d != 0) pl_set_device(d); } } restore{prev_dev};
+
+  if (M == 0 || N == 0) {
+    ATC_p out = new ATC();
+    out->T = 0; out->active_unit_num = 1; out->active_unit_id_list[0] = 0; out->subkernel_num = 0; out->pred_t = 0;
+    return out;
+  }
+  if (!C) error("PARALiA%s: C is null\n", GemmFns<T>::name);
+  const bool no_ab = (K == 0 || alpha == T(0));
+  if (!no_ab && (!A || !B)) error("PARALiA%s: A or B is null\n", GemmFns<T>::name);
+
+  int locA = 0, locB = 0, locC = 0;
+  chk(pl_ptr_location(C, &locC), "pointer location");
+  if (no_ab) locA = locB = 0;  // not referenced: treat as resident so nothing is fetched
+  else { chk(pl_ptr_location(A, &locA), "pointer location"); chk(pl_ptr_location(B, &locB), "pointer location"); }
+  if (locA > 0 || locB > 0 || locC > 0) error("PARALiA%s: operand on device %d; only device 0 is driven\n", GemmFns<T>::name, std::max(locA, std::max(locB, locC)));
+
+  PMDKey key;
+  key.routine = GemmFns<T>::name; key.ta = ta; key.tb = tb; key.D1 = M; key.D2 = N; key.D3 = no_ab ? 0 : K;
+  key.loc[0] = host_or_dev(locA); key.loc[1] = host_or_dev(locB); key.loc[2] = host_or_dev(locC);
+  key.beta_zero = (beta == T(0));
+  key.predef_T = predef ? predef->T : -1;
+  key.cache_limit = predef ? predef->cache_limit : 0;
+
+  PMDEntry* entry = nullptr;
+  for (auto& e : R.pmd)
+    if (e->key == key) { entry = e.get(); break; }
+  if (entry) ++R.pmd_hits;
+  else {
+    ++R.pmd_misses;
+    std::unique_ptr<PMDEntry> ne(new PMDEntry());
+    ne->key = key;
+    ne->atc.reset(new ATC());
+    ATC* atc = ne->atc.get();
+    if (predef) {
+      atc->T = predef->T;
+      atc->cache_limit = predef->cache_limit;
+      atc->active_unit_num = predef->active_unit_num;
+      for (int i = 0; i < std::min(LOC_NUM, std::max(0, predef->active_unit_num)); ++i)
+        atc->active_unit_id_list[i] = predef->active_unit_id_list[i];
+    }
+    ProblemDesc d;
+    d.func = GemmFns<T>::name; d.problem = BLAS3;
+    d.D1 = M; d.D2 = N; d.D3 = no_ab ? 0 : K;
+    d.TransA = ta; d.TransB = tb; d.dtype_sz = sizeof(T); d.numT = 3;
+    d.loc[0] = d.out_loc[0] = key.loc[0]; d.loc[1] = d.out_loc[1] = key.loc[1]; d.loc[2] = d.out_loc[2] = key.loc[2];
+    d.beta_is_zero = key.beta_zero;
+    const bool any_remote = key.loc[0] < 0 || key.loc[1] < 0 || key.loc[2] < 0;
+    d.pool_budget_bytes = any_remote ? pool_budget(atc->cache_limit, R.pool.bytes()) : 0;
+    if (any_remote && atc->cache_limit > 0 && atc->T > 0 && atc->cache_limit < 3LL * atc->T * atc->T * (long long)sizeof(T))
+      error("PARALiA%s: Problem cannot run with less memory than %lld\n", GemmFns<T>::name, 3LL * atc->T * atc->T * (long long)sizeof(T));
+    // alpha == 0 or K == 0: C <- beta*C only, one "subkernel" per C tile with an empty K; K must not
+    // constrain the tile choice then
+    if (d.D3 == 0) d.D3 = std::min(M, N);
+    atc->autotune_problem(GemmFns<T>::name, d);
+    if (any_remote) {
+      GemmProblem gp;
+      gp.M = M; gp.N = N; gp.K = no_ab ? 0 : K; gp.T = atc->T;
+      gp.a_remote = key.loc[0] < 0; gp.b_remote = key.loc[1] < 0; gp.c_remote = key.loc[2] < 0;
+      gp.beta_zero = key.beta_zero; gp.elem = sizeof(T); gp.exec_queues = atc->exec_queues;
+      const long long blk = (long long)atc->T * atc->T * (long long)sizeof(T);
+      gp.pool_blocks = (long)std::min<long long>(gemm_full_block_num(gp), d.pool_budget_bytes / blk);
+      try {
+        ne->plan = build_gemm_plan(gp, atc->order_id);
+      } catch (const std::runtime_error&) {
+        // the order chosen for the model's K does not fit (K == 0 path): the reference order always does
+        try { ne->plan = build_gemm_plan(gp, order_id_of(1, 0)); }
+        catch (const std::runtime_error& e2) { error("%s\n", e2.what()); }
+        atc->order_id = order_id_of(1, 0);
+      }
+      atc->update_sk_num(gp.subkernels());
+      atc->distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
+    }
+    if ((int)R.pmd.size() >= PROBLEM_MD_CACHE) R.pmd.erase(R.pmd.begin());
+    R.pmd.push_back(std::move(ne));
+    entry = R.pmd.back().get();
+  }
+
+  ATC* atc = entry->atc.get();
+  const bool any_remote = key.loc[0] < 0 || key.loc[1] < 0 || key.loc[2] < 0;
+  if (!any_remote) {
+    // Every operand already in HBM: one launch over the caller's matrices.
+    R.res.ensure_streams(1);
+    chk(GemmFns<T>::tile(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, R.res.exec[0]), "gemm launch");
+    chk(pl_stream_sync(R.res.exec[0]), "stream sync");
+  } else {
+    const GemmPlan& plan = entry->plan;
+    R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T));
+    execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC);
+  }
+  return atc_copy(atc);
+}
+
+// ------------------------------------------------------------------------------------------ BLAS-1
+struct Blas1Key { long N; int locx, locy; long T; };
+
+static ATC* blas1_tune(Runtime& R, const char* routine, long N, int locx, int locy, bool y_out, ATC_p predef, size_t elem_span_bytes) {
+  PMDKey key;
+  key.routine = routine; key.D1 = N; key.D2 = 1; key.D3 = 1;
+  key.loc[0] = host_or_dev(locx); key.loc[1] = host_or_dev(locy); key.loc[2] = 0;
+  key.predef_T = predef ? predef->T : -1;
+  key.cache_limit = predef ? predef->cache_limit : 0;
+  for (auto& e : R.pmd)
+    if (e->key == key) { ++R.pmd_hits; return e->atc.get(); }
+  ++R.pmd_misses;
+  std::unique_ptr<PMDEntry> ne(new PMDEntry());
+  ne->key = key;
+  ne->atc.reset(new ATC());
+  ATC* atc = ne->atc.get();
+  if (predef) { atc->T = predef->T; atc->cache_limit = predef->cache_limit; }
+  ProblemDesc d;
+  d.func = routine; d.problem = BLAS1; d.D1 = N; d.D2 = 1; d.D3 = 1; d.dtype_sz = 8; d.numT = 2;
+  d.in[0] = 1; d.in[1] = 1; d.in[2] = 0;
+  d.out[0] = 0; d.out[1] = y_out ? 1 : 0; d.out[2] = 0;
+  d.loc[0] = d.out_loc[0] = key.loc[0]; d.loc[1] = d.out_loc[1] = key.loc[1]; d.loc[2] = d.out_loc[2] = 0;
+  atc->autotune_problem(routine, d);
+  if (atc->cache_limit > 0) {
+    // daxpy.cpp:282-321 sizes the pool as 1 + 2*tiles blocks; under a limit keep at least a 2-deep ring per vector
+    const long long need = 4LL * atc->T * (long long)elem_span_bytes;
+    if (atc->cache_limit < need) error("PARALiA%s: Problem cannot run with less memory than %lld\n", routine, need);
+  }
+  if ((int)R.pmd.size() >= PROBLEM_MD_CACHE) R.pmd.erase(R.pmd.begin());
+  R.pmd.push_back(std::move(ne));
+  return R.pmd.back()->atc.get();
+}
+
+// Streams 1-D tiles of x and y through a ring of device blocks.  op(tile, xdev, ydev, len, stream) enqueues
+// the kernel; write_y sends every y tile back.  Strided vectors move as their contiguous span.
+template <typename Op>
+static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int locx, double* y, long incy, int locy, bool write_y, Op op) {
+  const long tiles = (N + T - 1) / T;
+  const long ax = std::labs(incx), ay = std::labs(incy);
+  const bool rx = locx < 0, ry = locy < 0;
+  const int ring = (int)std::min<long>(tiles, 3);
+  const long long span_x = ((long long)(T - 1) * ax + 1) * 8, span_y = ((long long)(T - 1) * ay + 1) * 8;
+  const long long blk = std::max(span_x, span_y);
+  R.pool.ensure(2L * ring, blk);
+  R.res.ensure_streams(1);
+  R.res.ensure_events(3 * (size_t)ring);
+  void* s_in = R.res.h2d; void* s_ex = R.res.exec[0]; void* s_out = R.res.d2h;
+  std::vector<void*> ev_in(ring), ev_ex(ring), ev_out(ring);
+  for (int r = 0; r < ring; ++r) { ev_in[r] = R.res.events[3 * r]; ev_ex[r] = R.res.events[3 * r + 1]; ev_out[r] = R.res.events[3 * r + 2]; }
+  for (long t = 0; t < tiles; ++t) {
+    const long len = std::min(T, N - t * T);
+    const int r = (int)(t % ring);
+    // BLAS: with a negative increment the vector runs backwards from the far end of its span
+    const long xoff = incx >= 0 ? t * T * ax : (N - t * T - len) * ax;
+    const long yoff = incy >= 0 ? t * T * ay : (N - t * T - len) * ay;
+    double* xs = x + xoff;
+    double* ys = y + yoff;
+    double* xd = rx ? (double*)R.pool.at(2 * r) : xs;
+    double* yd = ry ? (double*)R.pool.at(2 * r + 1) : ys;
+    const long long bx = ((long long)(len - 1) * ax + 1) * 8, by = ((long long)(len - 1) * ay + 1) * 8;
+    if (t >= ring) {  // the ring slot is free once its previous tenant has been consumed / written back
+      chk(pl_stream_wait_event(s_in, (write_y && ry) ? ev_out[r] : ev_ex[r]), "stream wait event");
+    }
+    if (rx) chk(pl_copy_async(xd, xs, bx, s_in), "fetch x tile");
+    if (ry) chk(pl_copy_async(yd, ys, by, s_in), "fetch y tile");
+    if (rx || ry) {
+      chk(pl_event_record(ev_in[r], s_in), "event record");
+      chk(pl_stream_wait_event(s_ex, ev_in[r]), "stream wait event");
+    }
+    op(t, xd, yd, len, s_ex);
+    chk(pl_event_record(ev_ex[r], s_ex), "event record");
+    if (write_y && ry) {
+      chk(pl_stream_wait_event(s_out, ev_ex[r]), "stream wait event");
+      chk(pl_copy_async(ys, yd, by, s_out), "write back y tile");
+      chk(pl_event_record(ev_out[r], s_out), "event record");
+    }
+  }
+  R.res.sync_all();
+}
+
+static void blas1_common_checks(const char* routine, long N, double* x, long incx, double* y, long incy, int* locx, int* locy) {
+  if (N < 0) error("PARALiA%s: negative N\n", routine);
+  if (N > 0 && (!x || !y)) error("PARALiA%s: null vector\n", routine);
+  if (incx == 0 || incy == 0) error("PARALiA%s: zero increment\n", routine);
+  *locx = *locy = 0;
+  if (N > 0) { chk(pl_ptr_location(x, locx), "pointer location"); chk(pl_ptr_location(y, locy), "pointer location"); }
+  if (*locx > 0 || *locy > 0) error("PARALiA%s: operand on device %d; only device 0 is driven\n", routine, std::max(*locx, *locy));
+}
+
+}  // namespace paralia
+
+using namespace paralia;
+
+// The C++ API keeps the reference's error behaviour: print and terminate (its error() never returns).
+#define PARALIA_TERMINATE_ON_ERROR(expr)                       \
+  try {                                                        \
+    return (expr);                                             \
+  } catch (const paralia_error& e) {                           \
+    fprintf(stderr, "ERROR -> %s", e.what());                  \
+    exit(1);                                                   \
+  }
+
+namespace paralia {
+ATC_p dgemm_impl(char TransA, char TransB, long M, long N, long K, double alpha, double* A, long ldA, double* B, long ldB,
+                 double beta, double* C, long ldC, ATC_p predef) {
+  return gemm_entry<double>(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef);
+}
+ATC_p sgemm_impl(char TransA, char TransB, long M, long N, long K, float alpha, float* A, long ldA, float* B, long ldB,
+                 float beta, float* C, long ldC, ATC_p predef) {
+  return gemm_entry<float>(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef);
+}
+
+ATC_p daxpy_impl(long N, double alpha, double* x, long incx, double* y, long incy, ATC_p predef) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  int locx, locy;
+  blas1_common_checks("Daxpy", N, x, incx, y, incy, &locx, &locy);
+  int prev_dev = 0;
+  chk(pl_get_device(&prev_dev), "get device");
+  if (prev_dev != 0) chk(pl_set_device(0), "set device");
+  struct Restore { int d; ~Restore() { if (d != 0) pl_set_device(d); } } restore{prev_dev};
+  if (N == 0) { ATC_p out = new ATC(); out->T = 0; out->active_unit_num = 1; out->active_unit_id_list[0] = 0; out->subkernel_num = 0; return out; }
+  ATC* atc = blas1_tune(R, "Daxpy", N, locx, locy, true, predef, 8 * (size_t)std::max(std::labs(incx), std::labs(incy)));
+  if (locx >= 0 && locy >= 0) {
+    R.res.ensure_streams(1);
+    chk(pl_daxpy(N, alpha, x, incx, y, incy, R.res.exec[0]), "daxpy launch");
+    chk(pl_stream_sync(R.res.exec[0]), "stream sync");
+  } else if (alpha != 0.0) {
+    const long T = atc->T;
+    blas1_stream(R, N, T, x, incx, locx, y, incy, locy, true, [&](long, double* xd, double* yd, long len, void* s) {
+      // inside a tile the span is walked forwards or backwards according to the sign of the increment
+      chk(pl_daxpy(len, alpha, xd, incx, yd, incy, s), "daxpy launch");
+    });
+  }
+  return atc_copy(atc);
+}
+
+ATC_p ddot_impl(long N, double* x, long incx, double* y, long incy, double* result, ATC_p predef) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  if (!result) error("PARALiADdot: result is null\n");
+  int locx, locy;
+  blas1_common_checks("Ddot", N, x, incx, y, incy, &locx, &locy);
+  int prev_dev = 0;
+  chk(pl_get_device(&prev_dev), "get device");
+  if (prev_dev != 0) chk(pl_set_device(0), "set device");
+  struct Restore { int d; ~Restore() { if (d != 0) pl_set_device(d); } } restore{prev_dev};
+  if (N == 0) { ATC_p out = new ATC(); out->T = 0; out->active_unit_num = 1; out->active_unit_id_list[0] = 0; out->subkernel_num = 0; return out; }
+  ATC* atc = blas1_tune(R, "Ddot", N, locx, locy, false, predef, 8 * (size_t)std::max(std::labs(incx), std::labs(incy)));
+  R.res.ensure_streams(1);
+  R.res.ensure_dot();
+  if (locx >= 0 && locy >= 0) {
+    chk(pl_ddot(N, x, incx, y, incy, R.res.dot_result, 0, R.res.dot_ws, R.res.exec[0]), "ddot launch");
+  } else {
+    const long T = atc->T;
+    // per-tile partials are folded into one device scalar in tile order (ddot.cpp:70,431 sums them on the host)
+    blas1_stream(R, N, T, x, incx, locx, y, incy, locy, false, [&](long t, double* xd, double* yd, long len, void* s) {
+      chk(pl_ddot(len, xd, incx, yd, incy, R.res.dot_result, t == 0 ? 0 : 1, R.res.dot_ws, s), "ddot launch");
+    });
+  }
+  chk(pl_copy_async(R.res.dot_host, R.res.dot_result, 8, R.res.exec[0]), "ddot result copy");
+  chk(pl_stream_sync(R.res.exec[0]), "stream sync");
+  *result += *R.res.dot_host;  // the reference accumulates into the caller's scalar (ddot.cpp:431)
+  return atc_copy(atc);
+}
+
+void cache_free_impl(short dev_id) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  if (dev_id != 0) return;  // the host "cache" of the reference (dev -1) holds nothing here
+  R.res.sync_all();
+  R.pool.release();
+}
+
+void runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  if (pmd_hits) *pmd_hits = R.pmd_hits;
+  if (pmd_misses) *pmd_misses = R.pmd_misses;
+  if (pool_bytes) *pool_bytes = R.pool.bytes();
+  if (pmd_entries) *pmd_entries = (long)R.pmd.size();
+}
+
+void runtime_reset() {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  R.pmd.clear();
+  R.pmd_hits = R.pmd_misses = 0;
+}
+}  // namespace paralia
+
+ATC_p PARALiADgemm(char TransA, char TransB, long int M, long int N, long int K, double alpha, double* A, long int ldA,
+                   double* B, long int ldB, double beta, double* C, long int ldC) {
+  PARALIA_TERMINATE_ON_ERROR(dgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, nullptr));
+}
+ATC_p PARALiADgemmControled(char TransA, char TransB, long int M, long int N, long int K, double alpha, double* A,
+                            long int ldA, double* B, long int ldB, double beta, double* C, long int ldC, ATC_p predef) {
+  PARALIA_TERMINATE_ON_ERROR(dgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef));
+}
+ATC_p PARALiASgemm(char TransA, char TransB, long int M, long int N, long int K, float alpha, float* A, long int ldA,
+                   float* B, long int ldB, float beta, float* C, long int ldC) {
+  PARALIA_TERMINATE_ON_ERROR(sgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, nullptr));
+}
+ATC_p PARALiASgemmControled(char TransA, char TransB, long int M, long int N, long int K, float alpha, float* A,
+                            long int ldA, float* B, long int ldB, float beta, float* C, long int ldC, ATC_p predef) {
+  PARALIA_TERMINATE_ON_ERROR(sgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef));
+}
+ATC_p PARALiADaxpy(long int N, double alpha, double* x, long int incx, double* y, long int incy) {
+  PARALIA_TERMINATE_ON_ERROR(daxpy_impl(N, alpha, x, incx, y, incy, nullptr));
+}
+ATC_p PARALiADaxpyControled(long int N, double alpha, double* x, long int incx, double* y, long int incy, ATC_p predef) {
+  PARALIA_TERMINATE_ON_ERROR(daxpy_impl(N, alpha, x, incx, y, incy, predef));
+}
+ATC_p PARALiADdot(long int N, double* x, long int incx, double* y, long int incy, double* result) {
+  PARALIA_TERMINATE_ON_ERROR(ddot_impl(N, x, incx, y, incy, result, nullptr));
+}
+ATC_p PARALiADdotControled(long int N, double* x, long int incx, double* y, long int incy, double* result, ATC_p predef) {
+  PARALIA_TERMINATE_ON_ERROR(ddot_impl(N, x, incx, y, incy, result, predef));
+}
+void PARALiADevCacheFree(short dev_id) {
+  try {
+    cache_free_impl(dev_id);
+  } catch (const paralia_error& e) {
+    fprintf(stderr, "ERROR -> %s", e.what());
+    exit(1);
+  }
+}

@@ -1,0 +1,59 @@
+"""The C ABI: the library loads, exports every symbol include/paralia_hip.h declares, and its argument checks
+answer with status codes before anything touches a GPU."""
+import ctypes as C
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "paralia_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:pl_|PARALiA_)[A-Za-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(pkg, L):
+    names = declared_symbols()
+    assert len(names) >= 55
+    raw = C.CDLL(pkg.LIB_PATH)
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert not missing, missing
+    # and the Python face declares a signature for each of them
+    from_binding = set(pkg.binding._SIGS)
+    assert set(names) <= from_binding, sorted(set(names) - from_binding)
+
+
+def test_cxx_api_is_exported(pkg):
+    import subprocess
+    out = subprocess.run(["nm", "-DC", pkg.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    for sym in ("PARALiADgemm(", "PARALiADgemmControled(", "PARALiASgemm(", "PARALiASgemmControled(", "PARALiADaxpy(",
+                "PARALiADaxpyControled(", "PARALiADdot(", "PARALiADdotControled(", "PARALiADevCacheFree(", "CoCoMalloc(",
+                "CoCoFree(", "CoCoMemcpy(", "CoCoSyncCheckErr(", "Dtest_equality(", "Stest_equality(", "csecond(",
+                "ATC::print_csv(", "ATC::autotune_problem("):
+        assert sym in out, sym
+
+
+def test_kernel_launchers_validate_before_launching(L):
+    # invalid arguments are refused on the host: no device is needed to see the status code
+    assert L.pl_dgemm_tile(b"X", b"N", 4, 4, 4, 1.0, None, 4, None, 4, 0.0, None, 4, None) == 1
+    assert L.pl_dgemm_tile(b"N", b"N", -1, 4, 4, 1.0, None, 4, None, 4, 0.0, None, 4, None) == 2
+    assert L.pl_dgemm_tile(b"N", b"N", 8, 4, 4, 1.0, None, 4, None, 4, 0.0, None, 8, None) == 3   # lda < M
+    assert L.pl_dgemm_tile(b"T", b"N", 8, 4, 16, 1.0, None, 8, None, 16, 0.0, None, 8, None) == 3  # lda < K when transposed
+    assert L.pl_sgemm_tile(b"N", b"T", 8, 4, 4, 1.0, None, 8, None, 2, 0.0, None, 8, None) == 3    # ldb < N when transposed
+    assert L.pl_dgemm_tile(b"N", b"N", 0, 4, 4, 1.0, None, 1, None, 4, 0.0, None, 1, None) == 0    # empty: nothing to do
+    assert L.pl_dgemm_tile(b"N", b"N", 4, 4, 4, 1.0, None, 4, None, 4, 0.0, None, 4, None) == 5    # null operands
+    assert L.pl_daxpy(0, 1.0, None, 1, None, 1, None) == 0
+    assert L.pl_daxpy(10, 0.0, None, 1, None, 1, None) == 0    # alpha == 0: quick return, y untouched
+    assert L.pl_daxpy(10, 1.0, None, 1, None, 1, None) == 5
+    assert L.pl_dgeadd_tile(8, 8, 1.0, None, 4, None, 8, None, 8, None) == 5
+    assert L.pl_ddot_workspace_doubles() >= 1024
+
+
+def test_csv_row_round_trip(pkg, L, tmp_path):
+    """The runner log row (reference testing.cpp:420-428): 'T,units,dev_token,cache, TransA,TransB,alpha,beta,M,N,K,
+    Aloc,Bloc,Cloc,Coutloc, t,pred_t,pred_J'."""
+    row = "%s, %c,%c,%.5lf,%.5lf,%zu,%zu,%zu,%d,%d,%d,%d, %e,%e,%e\n"
+    line = "2048,1,1,0, N,N,1.00000,0.00000,16384,16384,16384,-1,-1,-1,-1, 1.300000e-01,1.250000e-01,-1.000000e+00\n"
+    parts = [p.strip() for p in line.split(",")]
+    assert len(parts) == 18 and parts[0] == "2048" and parts[4] == "N" and float(parts[15]) == 0.13

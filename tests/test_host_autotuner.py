@@ -1,0 +1,158 @@
+"""The shipped autotuner (C++ inside libparalia.so, reached through its C probes; no GPU call is made) against
+hand-derived values and against the oracle on the same database numbers."""
+import ctypes as C
+import os
+import shutil
+
+import pytest
+
+from oracle_binding import make_table, orc_link, orc_problem
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+DB_SYNTH = os.path.join(HERE, "golden", "db_synth").encode()
+DB_V100 = os.path.join(HERE, "golden", "db_v100").encode()
+TILE = 1024 * 1024 * 8
+HOST3 = (C.c_int * 3)(-1, -1, -1)
+
+
+def loc3(a, b, c):
+    return (C.c_int * 3)(a, b, c)
+
+
+def test_heuristic_known_answers(L, orc):
+    sl = (C.c_double * 6)()
+    assert L.PARALiA_heuristic_tile(16384, 16384, 16384, sl) == 2048 and sl[0] == 0.00390625
+    assert L.PARALiA_heuristic_tile(4096, 4096, 4096, sl) == 2048 and sl[0] == 0.25
+    assert L.PARALiA_heuristic_tile(32768, 32768, 32768, sl) == 4096 and sl[0] == 0.00390625
+    assert L.PARALiA_heuristic_tile(40000, 40000, 2048, sl) == 2048
+    assert abs(sl[0] - (2.0 / 19 + 2.0 / 400)) < 1e-15
+
+
+@pytest.mark.parametrize("dims", [(16384, 16384, 16384), (40000, 40000, 2048), (289, 353, 307), (5000, 3000, 7000),
+                                  (8192, 1024, 4096)])
+def test_heuristic_matches_oracle_everywhere(L, orc, dims):
+    a, b = (C.c_double * 6)(), (C.c_double * 6)()
+    assert L.PARALiA_heuristic_tile(*dims, a) == orc.orc_optimize_tile(*dims, 1, b)
+    assert list(a) == list(b)
+    for T in (64, 100, 256, 1000, 2048, 2049, 4096, 5000):
+        if T > min(dims):
+            continue
+        assert L.PARALiA_T_slowdowns(*dims, T, a) == 0
+        orc.orc_get_T_slowdowns(*dims, 1, T, b)
+        assert list(a) == list(b)
+
+
+def test_models_by_hand(L):
+    """Same scenario as the oracle's hand-worked one: 4096^3, T = 1024, t_exec 1 ms, H2D 0.5 ms, D2H 0.25 ms per tile
+    (slowdowns 1.25 / 1.5 only matter to the bidirectional model)."""
+    pred = lambda mode, loc=HOST3, T=1024: L.PARALiA_model_predict(DB_SYNTH, b"Dgemm", mode, 4096, 4096, 4096, b"N", b"N", loc, T)
+    assert abs(pred(3) - 0.09725) < 1e-12
+    assert abs(pred(4) - 0.09725) < 1e-12
+    assert abs(pred(5) - 0.101975) < 1e-12
+    assert abs(pred(6) - 0.06575) < 1e-12
+    assert abs(pred(9) - 0.064) < 1e-12
+    assert abs(pred(10) - 0.096) < 1e-12
+    assert abs(pred(4, loc3(-1, -1, 0)) - 0.065) < 1e-12
+    assert abs(pred(4, loc3(-1, 0, 0)) - 0.064) < 1e-12
+    d = L.PARALiA_model_predict(DB_SYNTH, b"Daxpy", 5, 1 << 20, 1, 1, b"N", b"N", loc3(-1, -1, 0), 1 << 18)
+    assert abs(d - 1.21875e-3) < 1e-15
+
+
+def test_models_match_oracle_sweep(L, orc):
+    Ts = [512, 1024, 2048, 4096]
+    scale = {(b"N", b"N"): 1.0, (b"N", b"T"): 1.1, (b"T", b"N"): 1.2, (b"T", b"T"): 1.3}
+    for (ta, tb), s in scale.items():
+        tab, keep = make_table(Ts, [float("%e" % (1e-3 * s * (t / 1024.0) ** 3)) for t in Ts], (ta * 4).decode(), (tb * 4).decode())
+        for dims in ((4096, 4096, 4096), (8192, 4096, 2048), (5000, 6000, 7000)):
+            for locs in ((-1, -1, -1), (-1, -1, 0), (0, -1, -1), (-1, 0, 0), (0, 0, 0)):
+                p = orc_problem()
+                p.D1, p.D2, p.D3 = dims
+                p.dtype_sz, p.ta, p.tb = 8, ta, tb
+                for i in range(3):
+                    p.remote[i] = p.out_remote[i] = 1 if locs[i] < 0 else 0
+                p.h2d = orc_link(0.0, float("%.17e" % (0.5e-3 / TILE)), 1.25)
+                p.d2h = orc_link(0.0, float("%.17e" % (0.25e-3 / TILE)), 1.5)
+                p.exec = C.pointer(tab)
+                for mode in (3, 4, 5, 6, 9, 10):
+                    for T in (512, 1024, 2048, 3000):
+                        a = L.PARALiA_model_predict(DB_SYNTH, b"Dgemm", mode, *dims, ta, tb, loc3(*locs), T)
+                        b = orc.orc_predict_blas3(mode, p, T)
+                        assert abs(a - b) <= 1e-12 * max(1.0, abs(b)), (mode, T, dims, locs, ta, tb, a, b)
+
+
+def test_v100_rows_and_cubic_extrapolation(L):
+    """Real rows of the reference's V100 logs: an exact hit returns the logged time; a miss scales the nearest
+    lower entry with T^3 (GPUexec_lookup.cpp:118-128).  NO_OVERLAP on a device-resident problem is exec only."""
+    dev = loc3(0, 0, 0)
+    for T, t in ((2048, 2.556160e-03), (4096, 1.921535e-02), (8192, 1.578847e-01)):
+        got = L.PARALiA_model_predict(DB_V100, b"Dgemm", 10, T, T, T, b"N", b"N", dev, T)
+        assert abs(got - t) < 1e-15
+    got = L.PARALiA_model_predict(DB_V100, b"Dgemm", 3, 3000, 3000, 3000, b"N", b"N", dev, 3000)
+    assert abs(got - 2.556160e-03 * 27e9 / 2048 ** 3) < 1e-15  # one subkernel, nothing to transfer
+
+
+def test_missing_database_is_an_error(L, pkg, tmp_path):
+    assert L.PARALiA_model_predict(str(tmp_path).encode(), b"Dgemm", 6, 4096, 4096, 4096, b"N", b"N", HOST3, 1024) < 0
+    assert b"not generated" in L.PARALiA_last_error()
+    bad = tmp_path / "Processed"
+    bad.mkdir()
+    shutil.copy(os.path.join(DB_SYNTH.decode(), "Processed", "Dgemm_lookup-table_dev-0.log"), bad)
+    (bad / "Link-Stats_loc_dest-0_loc_src--1.log").write_text("Intercept: oops\n")
+    (bad / "Link-Stats_loc_dest--1_loc_src-0.log").write_text("Intercept: 0.0\nCoefficient: 1e-10\n")
+    assert L.PARALiA_model_predict(str(tmp_path).encode(), b"Dgemm", 6, 4096, 4096, 4096, b"N", b"N", HOST3, 1024) < 0
+    assert b"Problem in reading model" in L.PARALiA_last_error()
+
+
+def test_autotune_selectors(L, pkg, monkeypatch):
+    info = pkg.atc_info()
+    # model-driven search over the benchmarked tile sizes, pipeline model (default)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"pipeline-model" and info.has_db == 1
+    assert info.T in (512, 1024, 2048, 4096)
+    assert info.subkernel_num == (8192 // info.T) ** 3
+    assert info.pred_t > 0 and info.pipe_exec <= info.pred_t * 1.0000001
+    # the pick is the argmin of the simulated pipeline over the table
+    best = None
+    for T in (512, 1024, 2048, 4096):
+        one = pkg.atc_info()
+        assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, T, 0, C.byref(one)) == 0
+        assert one.selected_by == b"user" and one.T == T
+        if best is None or one.pred_t < best[1]:
+            best = (T, one.pred_t)
+    assert best[0] == info.T and abs(best[1] - info.pred_t) < 1e-12
+    # reference model-driven search (data-reuse model)
+    monkeypatch.setenv("PARALIA_T_SELECT", "reuse")
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"cocopelia-reuse"
+    # reference heuristic
+    monkeypatch.setenv("PARALIA_T_SELECT", "heuristic")
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"heuristic" and info.T == 2048 and info.slowdowns[0] == 0.00390625
+    assert info.subkernel_num == 512
+    # everything resident: nothing to tile
+    monkeypatch.delenv("PARALIA_T_SELECT")
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 4096, 2048, 1024, b"N", b"N", loc3(0, 0, 0), 0, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"resident" and info.subkernel_num == 1
+    # BLAS-1
+    assert L.PARALiA_autotune(DB_SYNTH, b"Daxpy", 1 << 24, 1, 1, b"N", b"N", loc3(-1, -1, 0), 0, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"cocopelia-bidirectional" and info.T in (1 << 16, 1 << 18, 1 << 20, 1 << 22)
+    assert info.subkernel_num == (1 << 24) // info.T
+    L.PARALiA_set_db_dir(None)
+
+
+def test_autotune_without_database_falls_back(L, pkg, tmp_path):
+    info = pkg.atc_info()
+    assert L.PARALiA_autotune(str(tmp_path).encode(), b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert info.has_db == 0 and info.selected_by == b"heuristic" and info.T == 2048
+    L.PARALiA_set_db_dir(None)
+
+
+def test_autotune_memory_limit(L, pkg):
+    info = pkg.atc_info()
+    # a pool of 3 blocks is the minimum (reference dgemm.cpp:41-42, 90-93); less is an error
+    blk = 2048 * 2048 * 8
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 0, 2048, 3 * blk, C.byref(info)) == 0
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 0, 2048, 2 * blk, C.byref(info)) != 0
+    assert b"less memory" in L.PARALiA_last_error()
+    L.PARALiA_set_db_dir(None)

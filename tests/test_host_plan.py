@@ -1,0 +1,208 @@
+"""Invariants of the static GEMM plan (tile order, beta schedule, block assignment, dependency edges), checked on
+the host, and a pure-Python replay of the plan on integer data against numpy."""
+import itertools
+
+import numpy as np
+import pytest
+
+FETCH_A, FETCH_B, FETCH_C, GEMM, REDUCE, WRITEBACK = range(6)
+BETA_ZERO, BETA_ONE, BETA_USER = 0, 1, 2
+H2D, D2H, EXEC0 = 0, 1, 2
+
+
+def grids(M, N, K, T):
+    c = lambda a: -(-a // T)
+    return c(M), c(N), (c(K) if K > 0 else 1)
+
+
+def check_plan(rows, stats, M, N, K, T, a_remote, b_remote, c_remote, beta_zero, pool_blocks, nq):
+    Mg, Ng, Kg = grids(M, N, K, T)
+    gemms = [r for r in rows if r["kind"] == GEMM]
+    # every subkernel fired exactly once
+    assert sorted((g["mi"], g["ni"], g["ki"]) for g in gemms) == sorted(itertools.product(range(Mg), range(Ng), range(Kg)))
+    assert stats[5] == Mg * Ng * Kg
+    chain = {}
+    for idx, r in enumerate(rows):
+        for w in r["waits"]:
+            assert 0 <= w < idx, "dependencies point backwards only"
+            assert rows[w]["stream"] != r["stream"], "same-stream order needs no event"
+        if r["kind"] == GEMM:
+            c = chain.setdefault((r["mi"], r["ni"]), [])
+            # first K-step of a C tile: beta' = 0 into the accumulator (remote C) or the caller's beta (resident C)
+            if not c:
+                assert r["beta_mode"] == (BETA_ZERO if c_remote else BETA_USER)
+            else:
+                assert r["beta_mode"] == BETA_ONE
+                assert r["stream"] == c[0]["stream"], "a C tile's K-chain stays on one exec queue"
+                assert r["block"] == c[0]["block"]
+            c.append(r)
+            assert EXEC0 <= r["stream"] < EXEC0 + nq
+            assert (r["a_block"] >= 0) == bool(a_remote) and (r["b_block"] >= 0) == bool(b_remote)
+            assert (r["block"] >= 0) == bool(c_remote)
+        if r["kind"] in (FETCH_A, FETCH_B, FETCH_C):
+            assert r["stream"] == H2D and 0 <= r["block"] < pool_blocks
+        if r["kind"] == WRITEBACK:
+            assert r["stream"] == D2H
+    assert all(len(c) == Kg for c in chain.values())
+    n_wb = sum(r["kind"] == WRITEBACK for r in rows)
+    n_red = sum(r["kind"] == REDUCE for r in rows)
+    assert n_wb == (Mg * Ng if c_remote else 0)
+    assert n_red == (Mg * Ng if (c_remote and not beta_zero) else 0)
+    assert stats[3] == n_red
+    assert stats[0] <= pool_blocks
+
+
+def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks):
+    """Execute the plan sequentially in plan order with numpy tiles; checks along the way that every block is read
+    only while it holds the tile the command expects (i.e. eviction never clobbers live data in plan order)."""
+    Mg, Ng, Kg = grids(M, N, K, T)
+    sl = lambda i, D: slice(i * T, min((i + 1) * T, D))
+    blocks = [None] * pool_blocks
+    out = C.copy()
+    for r in rows:
+        k = r["kind"]
+        if k == FETCH_A:
+            blocks[r["block"]] = ("A", r["mi"], r["ki"], A[sl(r["mi"], M), sl(r["ki"], K)].copy())
+        elif k == FETCH_B:
+            blocks[r["block"]] = ("B", r["ki"], r["ni"], B[sl(r["ki"], K), sl(r["ni"], N)].copy())
+        elif k == FETCH_C:
+            blocks[r["block"]] = ("S", r["mi"], r["ni"], C[sl(r["mi"], M), sl(r["ni"], N)].copy())
+        elif k == GEMM:
+            if r["a_block"] >= 0:
+                tag, i, j, a = blocks[r["a_block"]]
+                assert (tag, i, j) == ("A", r["mi"], r["ki"])
+            else:
+                a = A[sl(r["mi"], M), sl(r["ki"], K)]
+            if r["b_block"] >= 0:
+                tag, i, j, b = blocks[r["b_block"]]
+                assert (tag, i, j) == ("B", r["ki"], r["ni"])
+            else:
+                b = B[sl(r["ki"], K), sl(r["ni"], N)]
+            prod = alpha * (a @ b)
+            if r["block"] >= 0:
+                if r["beta_mode"] == BETA_ZERO:
+                    blocks[r["block"]] = ("ACC", r["mi"], r["ni"], prod)
+                else:
+                    tag, i, j, acc = blocks[r["block"]]
+                    assert (tag, i, j) == ("ACC", r["mi"], r["ni"]) and r["beta_mode"] == BETA_ONE
+                    blocks[r["block"]] = ("ACC", i, j, acc + prod)
+            else:
+                tgt = out[sl(r["mi"], M), sl(r["ni"], N)]
+                tgt[...] = prod + (beta if r["beta_mode"] == BETA_USER else 1.0) * tgt
+        elif k == REDUCE:
+            tag, i, j, acc = blocks[r["block"]]
+            stag, si, sj, src = blocks[r["a_block"]]
+            assert (tag, i, j) == ("ACC", r["mi"], r["ni"]) and (stag, si, sj) == ("S", r["mi"], r["ni"])
+            blocks[r["block"]] = ("ACC", i, j, beta * src + acc)
+        elif k == WRITEBACK:
+            tag, i, j, acc = blocks[r["block"]]
+            assert (tag, i, j) == ("ACC", r["mi"], r["ni"])
+            out[sl(r["mi"], M), sl(r["ni"], N)] = acc
+    return out
+
+
+ORDERS = [10000, 0, 1, 3, 10002, 10004]
+
+
+@pytest.mark.parametrize("order", ORDERS)
+@pytest.mark.parametrize("locs", [(1, 1, 1), (1, 1, 0), (0, 1, 1), (1, 0, 0), (0, 0, 1)])
+@pytest.mark.parametrize("beta_zero", [0, 1])
+def test_plan_invariants_and_replay(pkg, order, locs, beta_zero):
+    M, N, K, T = 90, 70, 110, 32
+    a_r, b_r, c_r = locs
+    rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
+    full = 1 + 3 * 4 + 4 * 3 + 2 * 3 * 3
+    check_plan(rows, stats, M, N, K, T, a_r, b_r, c_r, beta_zero, full, 2)
+    # everything fits: each remote tile is fetched exactly once, nothing is evicted
+    assert stats[1] == (3 * 4 if a_r else 0) and stats[2] == (4 * 3 if b_r else 0) and stats[4] == 0
+    rng = np.random.default_rng(order + 7 * beta_zero)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64)
+    B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C = rng.integers(-5, 6, (M, N)).astype(np.float64)
+    alpha, beta = 2.0, (0.0 if beta_zero else 3.0)
+    got = replay(rows, M, N, K, T, alpha, beta, A, B, C, full)
+    assert np.array_equal(got, alpha * (A @ B) + beta * C)
+
+
+@pytest.mark.parametrize("pool", [3, 4, 7, 12])
+@pytest.mark.parametrize("beta_zero", [0, 1])
+def test_plan_with_eviction(pkg, pool, beta_zero):
+    """A pool smaller than the working set: tiles are re-fetched, nothing live is clobbered, a writer of a recycled
+    block waits for every earlier user of that block."""
+    M, N, K, T = 100, 100, 100, 32
+    rows, stats = pkg.plan_rows(M, N, K, T, 1, 1, 1, beta_zero, 8, 2, pool, 10000)
+    check_plan(rows, stats, M, N, K, T, 1, 1, 1, beta_zero, pool, 2)
+    assert stats[4] > 0 and stats[1] + stats[2] > 2 * 16
+    rng = np.random.default_rng(pool)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64)
+    B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C = rng.integers(-5, 6, (M, N)).astype(np.float64)
+    beta = 0.0 if beta_zero else -2.0
+    assert np.array_equal(replay(rows, M, N, K, T, 1.0, beta, A, B, C, pool), A @ B + beta * C)
+    # asynchronous safety: every user of a block's previous tenant is ordered (transitively, through stream order
+    # and waits) before the command that overwrites the block
+    users = {}
+    order_before = [set() for _ in rows]
+    last_on_stream = {}
+    for i, r in enumerate(rows):
+        deps = set()
+        if r["stream"] in last_on_stream:
+            j = last_on_stream[r["stream"]]
+            deps |= order_before[j] | {j}
+        for w in r["waits"]:
+            deps |= order_before[w] | {w}
+        order_before[i] = deps
+        last_on_stream[r["stream"]] = i
+        writes = [r["block"]] if r["kind"] in (FETCH_A, FETCH_B, FETCH_C) or (r["kind"] == GEMM and r["beta_mode"] == BETA_ZERO) else []
+        for b in writes:
+            for u in users.get(b, []):
+                assert u in deps, "block %d overwritten by cmd %d before its user %d is known to be done" % (b, i, u)
+            users[b] = []
+        reads = []
+        if r["kind"] == GEMM:
+            reads = [x for x in (r["a_block"], r["b_block"], r["block"]) if x >= 0]
+        elif r["kind"] == REDUCE:
+            reads = [r["block"], r["a_block"]]
+        elif r["kind"] == WRITEBACK:
+            reads = [r["block"]]
+        for b in reads:
+            users.setdefault(b, []).append(i)
+
+
+def test_plan_too_small_pool_is_an_error(pkg):
+    with pytest.raises(pkg.ParaliaError, match="< 3 blocks"):
+        pkg.plan_rows(100, 100, 100, 32, 1, 1, 1, 0, 8, 2, 2, 10000)
+    # k-outer order keeps every C accumulator open: it cannot run in 5 blocks, the reference order can
+    with pytest.raises(pkg.ParaliaError, match="too small"):
+        pkg.plan_rows(100, 100, 100, 32, 1, 1, 1, 0, 8, 2, 5, 4)
+    pkg.plan_rows(100, 100, 100, 32, 1, 1, 1, 0, 8, 2, 5, 10000)
+
+
+def test_reference_order_is_index_order(pkg):
+    rows, _ = pkg.plan_rows(64, 96, 128, 32, 1, 1, 1, 1, 8, 2, 0, 10000)
+    got = [(r["mi"], r["ni"], r["ki"]) for r in rows if r["kind"] == GEMM]
+    assert got == list(itertools.product(range(2), range(3), range(4)))  # mi*Ng*Kg + ni*Kg + ki (dgemm.cpp:139-142)
+
+
+def test_pipeline_simulation(pkg, L):
+    import ctypes as C
+    busy = (C.c_double * 3)()
+    picked = C.c_int()
+    # 16384^3, T = 2048, tile costs 0.24 ms compute / 0.6 ms each way: compute-bound overall (123 ms of kernels,
+    # 77 ms of H2D, 38 ms of D2H); a good order hides nearly all transfers, the reference index order cannot hide
+    # the fetch of a whole K-chain per C tile at the start, pure k-outer leaves every write-back to the end.
+    args = (16384, 16384, 16384, 2048, 1, 1, 1, 1, 8, 2, 0)
+    st = (0.24e-3, 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.02e-3)
+    best = L.PARALiA_gemm_plan_simulate(*args, -1, *st, C.byref(picked), busy)
+    assert abs(busy[1] - 512 * 0.24e-3) < 1e-9 and abs(busy[0] - 128 * 0.6e-3) < 1e-9 and abs(busy[2] - 64 * 0.6e-3) < 1e-9
+    assert best >= busy[1] and best < busy[1] * 1.04
+    ref_order = L.PARALiA_gemm_plan_simulate(*args, 10000, *st, None, None)
+    k_outer = L.PARALiA_gemm_plan_simulate(*args, 8, *st, None, None)
+    assert best <= ref_order and best <= k_outer
+    assert k_outer > busy[1] + 0.5 * busy[2]          # write-backs pile up behind the last K step
+    serial = busy[0] + busy[1] + busy[2]
+    assert best < 0.6 * serial
+    # transfer-bound case (40000 x 40000 x 2048, beta != 0): the H2D stream is the critical resource
+    args5 = (40000, 40000, 2048, 2048, 1, 1, 1, 0, 8, 2, 0)
+    t5 = L.PARALiA_gemm_plan_simulate(*args5, -1, *st, C.byref(picked), busy)
+    assert busy[0] > busy[1] and t5 >= busy[0] and t5 < busy[0] * 1.05
