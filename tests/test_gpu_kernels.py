@@ -1,0 +1,247 @@
+"""Parity of the hand-written HIP kernels, called through the C ABI, with the CPU oracle and OpenBLAS.
+Bit-exact where the arithmetic is exact (integer-valued data, daxpy against the fused form), otherwise within the
+contract's tolerances: normwise relative error <= 1e-13 (fp64) / 1e-5 (fp32) for GEMM, |err| <= 1e-13 |x||y| for ddot,
+<= 1 ulp per element for daxpy."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_util import Buf, sync
+from oracle_binding import ptr, rand_f32, rand_f64
+
+pytestmark = pytest.mark.gpu
+TOL64, TOL32 = 1e-13, 1e-5
+
+
+def run_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc, a_off=0, b_off=0, c_off=0):
+    dA, dB, dC = Buf(pkg, A.size, dtype, 0).set(A), Buf(pkg, B.size, dtype, 0).set(B), Buf(pkg, C0.size, dtype, 0).set(C0)
+    fn = L.pl_dgemm_tile if dtype == np.float64 else L.pl_sgemm_tile
+    print("gemm", dtype.__name__, ta, tb, M, N, K, alpha, beta, lda, ldb, ldc, a_off, b_off, c_off, flush=True)
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), dA.at(a_off), lda, dB.at(b_off), ldb, float(beta), dC.at(c_off), ldc, None), "gemm tile")
+    sync(pkg)
+    return dC.get()
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(256, 256, 64), (289, 353, 307), (128, 128, 16), (1, 1, 1), (130, 5, 1000), (64, 700, 3)])
+def test_dgemm_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, dims):
+    M, N, K = dims
+    alpha, beta = 1.2, 1.1
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 2, M + 6  # even leading dimensions: the 16-byte vector path
+    A, B, C0 = rand_f64(lda * ca, 1), rand_f64(ldb * cb, 2), rand_f64(ldc * N, 3)
+    got = run_gemm(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    ref = C0.copy()
+    assert openblas.orc_openblas_dgemm(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(ref), ldc) == 0
+    d = abs(alpha) * orc.orc_fro_norm_f64(ptr(A), ra, ca, lda) * orc.orc_fro_norm_f64(ptr(B), rb, cb, ldb) + abs(beta) * orc.orc_fro_norm_f64(ptr(C0), M, N, ldc)
+    assert orc.orc_normwise_err_f64(ptr(got), ptr(ref), M, N, ldc, ldc, d) < TOL64
+    bf = C0.copy()
+    orc.orc_dgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(bf), ldc)
+    assert orc.orc_normwise_err_f64(ptr(got), ptr(bf), M, N, ldc, ldc, d) < TOL64
+    # padding between columns untouched
+    pad = np.ones(ldc * N, dtype=bool)
+    pad.reshape(N, ldc)[:, :M] = False
+    assert np.array_equal(got[pad], C0[pad])
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "T"), ("N", "T"), ("T", "N")])
+def test_dgemm_tile_unaligned_views(pkg, L, orc, ta, tb):
+    """Odd leading dimensions and operand pointers offset by one element: the element-load path."""
+    M, N, K = 200, 150, 77
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 3, rb + 1, M + 1
+    A, B, C0 = rand_f64(lda * ca + 1, 4), rand_f64(ldb * cb + 1, 5), rand_f64(ldc * N + 1, 6)
+    got = run_gemm(pkg, L, np.float64, ta, tb, M, N, K, -0.5, 2.0, A, lda, B, ldb, C0, ldc, 1, 1, 1)
+    bf = C0.copy()
+    orc.orc_dgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, -0.5, ptr(A[1:]), lda, ptr(B[1:]), ldb, 2.0, ptr(bf[1:]), ldc)
+    d = 0.5 * orc.orc_fro_norm_f64(ptr(A[1:]), ra, ca, lda) * orc.orc_fro_norm_f64(ptr(B[1:]), rb, cb, ldb) + 2.0 * orc.orc_fro_norm_f64(ptr(C0[1:]), M, N, ldc)
+    assert orc.orc_normwise_err_f64(ptr(got[1:]), ptr(bf[1:]), M, N, ldc, ldc, d) < TOL64
+    assert got[0] == C0[0]
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+def test_dgemm_tile_exact_on_integers(pkg, L, orc, ta, tb):
+    """Small-integer data: every product and partial sum is exact, so any summation order gives the same bits."""
+    M, N, K = 257, 131, 300
+    rng = np.random.default_rng(5)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    A = rng.integers(-8, 9, ra * ca).astype(np.float64)
+    B = rng.integers(-8, 9, rb * cb).astype(np.float64)
+    C0 = rng.integers(-8, 9, M * N).astype(np.float64)
+    for alpha, beta in ((2.0, 3.0), (1.0, 0.0), (-1.0, 1.0)):
+        got = run_gemm(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, A, ra, B, rb, C0, M)
+        ref = C0.copy()
+        orc.orc_dgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M)
+        assert np.array_equal(got, ref)
+
+
+def test_dgemm_tile_special_scalars(pkg, L):
+    M, N, K = 100, 90, 50
+    A, B, C0 = rand_f64(M * K, 1), rand_f64(K * N, 2), rand_f64(M * N, 3)
+    nan_c = np.full(M * N, np.nan)
+    got = run_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, A, M, B, K, nan_c, M)
+    assert not np.isnan(got).any()  # beta == 0 never reads C
+    nan_a = np.full(M * K, np.nan)
+    got = run_gemm(pkg, L, np.float64, "N", "N", M, N, K, 0.0, 0.5, nan_a, M, B, K, C0, M)
+    assert np.array_equal(got, 0.5 * C0)  # alpha == 0: A and B are not referenced
+    got = run_gemm(pkg, L, np.float64, "N", "N", M, N, 0, 1.0, 0.0, A, M, B, 1, C0, M)
+    assert np.array_equal(got, np.zeros(M * N))  # K == 0, beta == 0: C is cleared
+    got = run_gemm(pkg, L, np.float64, "N", "N", M, N, 0, 1.0, 1.0, A, M, B, 1, C0, M)
+    assert np.array_equal(got, C0)
+    # identity: C = alpha*B + beta*C0 with power-of-two scalars is exact
+    n = 160
+    I = np.eye(n).ravel()
+    Bn, Cn = rand_f64(n * n, 8), rand_f64(n * n, 9)
+    got = run_gemm(pkg, L, np.float64, "N", "N", n, n, n, 2.0, 0.25, I, n, Bn, n, Cn, n)
+    assert np.array_equal(got, 2.0 * Bn + 0.25 * Cn)
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(256, 256, 64), (289, 353, 307), (33, 1000, 129)])
+def test_sgemm_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, dims):
+    M, N, K = dims
+    alpha, beta = np.float32(1.0), np.float32(1.0)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 8, M + 4
+    A, B, C0 = rand_f32(lda * ca, 1), rand_f32(ldb * cb, 2), rand_f32(ldc * N, 3)
+    got = run_gemm(pkg, L, np.float32, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    ref = C0.copy()
+    assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(ref), ldc) == 0
+    d = orc.orc_fro_norm_f32(ptr(A), ra, ca, lda) * orc.orc_fro_norm_f32(ptr(B), rb, cb, ldb) + orc.orc_fro_norm_f32(ptr(C0), M, N, ldc)
+    assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, ldc, ldc, d) < TOL32
+    bf = C0.copy()
+    orc.orc_sgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(bf), ldc)
+    assert orc.orc_normwise_err_f32(ptr(got), ptr(bf), M, N, ldc, ldc, d) < TOL32
+
+
+def test_sgemm_tile_exact_and_unaligned(pkg, L, orc):
+    M, N, K = 150, 97, 210
+    rng = np.random.default_rng(6)
+    A = rng.integers(-4, 5, (M + 1) * K + 3).astype(np.float32)
+    B = rng.integers(-4, 5, (N + 3) * K + 3).astype(np.float32)
+    C0 = rng.integers(-4, 5, (M + 1) * N + 3).astype(np.float32)
+    got = run_gemm(pkg, L, np.float32, "N", "T", M, N, K, 1.0, 1.0, A, M + 1, B, N + 3, C0, M + 1, 3, 1, 2)
+    ref = C0.copy()
+    orc.orc_sgemm_bruteforce(b"N", b"T", M, N, K, 1.0, ptr(A[3:]), M + 1, ptr(B[1:]), N + 3, 1.0, ptr(ref[2:]), M + 1)
+    assert np.array_equal(got, ref)
+
+
+def scaled_ulp(a, b, alpha, x, y0):
+    scale = np.maximum(np.maximum(np.abs(alpha * x), np.abs(y0)), np.maximum(np.abs(a), np.abs(b)))
+    return float(np.max(np.abs(a - b) / np.spacing(scale)))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 1000, 100003, 1 << 22, (1 << 22) + 1])
+def test_daxpy(pkg, L, orc, openblas, n):
+    alpha = 0.7
+    x, y0 = rand_f64(n, 1), rand_f64(n, 2)
+    dx, dy = Buf(pkg, n, np.float64, 0).set(x), Buf(pkg, n, np.float64, 0).set(y0)
+    print("daxpy", n, flush=True)
+    pkg.check(L.pl_daxpy(n, alpha, dx.ptr, 1, dy.ptr, 1, None), "daxpy")
+    sync(pkg)
+    got = dy.get()
+    fused = y0.copy()
+    orc.orc_daxpy(n, alpha, ptr(x), 1, ptr(fused), 1)
+    assert np.array_equal(got, fused)  # the kernel computes fma(alpha, x, y): one rounding, bit for bit
+    ref = y0.copy()
+    assert openblas.orc_openblas_daxpy(n, alpha, ptr(x), 1, ptr(ref), 1) == 0
+    # contract: within 1 ulp per element of OpenBLAS (ulp of the larger operand: the sum may cancel)
+    assert orc.orc_max_ulp_f64(ptr(got), ptr(ref), n) <= 1 or scaled_ulp(got, ref, alpha, x, y0) <= 1.5
+
+
+def test_daxpy_strided_unaligned_and_alpha_zero(pkg, L, orc):
+    n = 5001
+    x, y0 = rand_f64(3 * n + 1, 3), rand_f64(2 * n + 1, 4)
+    dx, dy = Buf(pkg, x.size, np.float64, 0).set(x), Buf(pkg, y0.size, np.float64, 0).set(y0)
+    pkg.check(L.pl_daxpy(n, 1.25, dx.at(1), 3, dy.at(1), -2, None), "daxpy strided")
+    sync(pkg)
+    ref = y0.copy()
+    orc.orc_daxpy(n, 1.25, ptr(x[1:]), 3, ptr(ref[1:]), -2)
+    assert np.array_equal(dy.get(), ref)
+    dy.set(y0)
+    pkg.check(L.pl_daxpy(n, 1.0, dx.at(1), 1, dy.at(1), 1, None), "daxpy unaligned")  # 8-byte aligned only
+    sync(pkg)
+    ref = y0.copy()
+    orc.orc_daxpy(n, 1.0, ptr(x[1:]), 1, ptr(ref[1:]), 1)
+    assert np.array_equal(dy.get(), ref)
+    dy.set(y0)
+    pkg.check(L.pl_daxpy(n, 0.0, dx.ptr, 1, dy.ptr, 1, None), "daxpy alpha 0")
+    sync(pkg)
+    assert np.array_equal(dy.get(), y0)
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 4097, 1 << 20, (1 << 23) + 3])
+def test_ddot(pkg, L, orc, openblas, n):
+    x, y = rand_f64(n, 5), rand_f64(n, 6)
+    dx, dy = Buf(pkg, n, np.float64, 0).set(x), Buf(pkg, n, np.float64, 0).set(y)
+    ws = Buf(pkg, L.pl_ddot_workspace_doubles(), np.float64, 0)
+    res = Buf(pkg, 1, np.float64, 0).set(np.array([123.0]))
+    print("ddot", n, flush=True)
+    pkg.check(L.pl_ddot(n, dx.ptr, 1, dy.ptr, 1, res.ptr, 0, ws.ptr, None), "ddot")
+    sync(pkg)
+    got = res.get()[0]
+    exact = float(orc.orc_ddot_longdouble(n, ptr(x), 1, ptr(y), 1))
+    bound = 1e-13 * float(np.linalg.norm(x) * np.linalg.norm(y))
+    assert abs(got - exact) <= bound
+    ob = C.c_double()
+    assert openblas.orc_openblas_ddot(n, ptr(x), 1, ptr(y), 1, C.byref(ob)) == 0
+    assert abs(got - ob.value) <= bound
+    # accumulate flag adds to what is there; same input twice gives the same bits (fixed summation order)
+    pkg.check(L.pl_ddot(n, dx.ptr, 1, dy.ptr, 1, res.ptr, 1, ws.ptr, None), "ddot acc")
+    sync(pkg)
+    assert res.get()[0] == got + got
+    pkg.check(L.pl_ddot(n, dx.ptr, 1, dy.ptr, 1, res.ptr, 0, ws.ptr, None), "ddot again")
+    sync(pkg)
+    assert res.get()[0] == got
+
+
+def test_ddot_exact_and_strided(pkg, L, orc):
+    n = 123457
+    ones = np.ones(n)
+    d1 = Buf(pkg, n, np.float64, 0).set(ones)
+    ws = Buf(pkg, L.pl_ddot_workspace_doubles(), np.float64, 0)
+    res = Buf(pkg, 1, np.float64, 0)
+    pkg.check(L.pl_ddot(n, d1.ptr, 1, d1.ptr, 1, res.ptr, 0, ws.ptr, None), "ddot ones")
+    sync(pkg)
+    assert res.get()[0] == float(n)
+    m = 7001
+    x, y = rand_f64(2 * m + 1, 7), rand_f64(3 * m + 1, 8)
+    dx, dy = Buf(pkg, x.size, np.float64, 0).set(x), Buf(pkg, y.size, np.float64, 0).set(y)
+    pkg.check(L.pl_ddot(m, dx.at(1), 2, dy.at(1), -3, res.ptr, 0, ws.ptr, None), "ddot strided")
+    sync(pkg)
+    exact = float(orc.orc_ddot_longdouble(m, ptr(x[1:]), 2, ptr(y[1:]), -3))
+    assert abs(res.get()[0] - exact) <= 1e-13 * float(np.linalg.norm(x) * np.linalg.norm(y))
+    pkg.check(L.pl_ddot(0, dx.ptr, 1, dy.ptr, 1, res.ptr, 0, ws.ptr, None), "ddot empty")
+    sync(pkg)
+    assert res.get()[0] == 0.0
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_geadd(pkg, L, dtype):
+    M, N = 1001, 77
+    lds, lda, ldo = M + 1, M + 2, M + 3  # odd strides among them: mixed vector / element paths
+    rng = np.random.default_rng(9)
+    src = rng.integers(-50, 50, lds * N).astype(dtype)
+    acc = rng.integers(-50, 50, lda * N).astype(dtype)
+    out0 = rng.integers(-50, 50, ldo * N).astype(dtype)
+    ds, da, do = Buf(pkg, src.size, dtype, 0).set(src), Buf(pkg, acc.size, dtype, 0).set(acc), Buf(pkg, out0.size, dtype, 0).set(out0)
+    fn = L.pl_dgeadd_tile if dtype == np.float64 else L.pl_sgeadd_tile
+    pkg.check(fn(M, N, 3.0, ds.ptr, lds, da.ptr, lda, do.ptr, ldo, None), "geadd")
+    sync(pkg)
+    got = do.get().reshape(N, ldo)
+    ref = out0.copy().reshape(N, ldo)
+    ref[:, :M] = 3.0 * src.reshape(N, lds)[:, :M] + acc.reshape(N, lda)[:, :M]
+    assert np.array_equal(got, ref)
+    # in place (out aliases acc), even strides: the vector path
+    M2 = 1000
+    acc2 = rng.integers(-50, 50, M2 * N).astype(dtype)
+    src2 = rng.integers(-50, 50, M2 * N).astype(dtype)
+    da2, ds2 = Buf(pkg, acc2.size, dtype, 0).set(acc2), Buf(pkg, src2.size, dtype, 0).set(src2)
+    pkg.check(fn(M2, N, -2.0, ds2.ptr, M2, da2.ptr, M2, da2.ptr, M2, None), "geadd in place")
+    sync(pkg)
+    assert np.array_equal(da2.get(), -2.0 * src2 + acc2)

@@ -1,0 +1,287 @@
+"""Parity of the PARALiA routines (tiling, streaming, block pool, lazy write-back, metadata reuse) called through
+the C ABI, against OpenBLAS / the oracle on the same seeded inputs, for every operand placement."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_util import Buf, sync
+from oracle_binding import ptr, rand_f32, rand_f64
+
+pytestmark = pytest.mark.gpu
+TOL64, TOL32 = 1e-13, 1e-5
+
+
+def place(pkg, arr, loc):
+    return Buf(pkg, arr.size, arr.dtype, loc).set(arr)
+
+
+def call_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, bufA, lda, bufB, ldb, bufC, ldc, T=-1, cache_limit=0):
+    info = pkg.atc_info()
+    fn = L.PARALiA_dgemm if dtype == np.float64 else L.PARALiA_sgemm
+    print("PARALiA gemm", np.dtype(dtype).name, ta, tb, M, N, K, alpha, beta, "locs", bufA.loc, bufB.loc, bufC.loc, "T", T,
+          "limit", cache_limit, flush=True)
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), bufA.ptr, lda, bufB.ptr, ldb, float(beta), bufC.ptr, ldc, T,
+                 cache_limit, C.byref(info)), "PARALiA gemm")
+    return info
+
+
+def openblas_ref(openblas, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc):
+    ref = C0.copy()
+    fn = openblas.orc_openblas_dgemm if dtype == np.float64 else openblas.orc_openblas_sgemm
+    assert fn(ta.encode(), tb.encode(), M, N, K, float(alpha), ptr(A), lda, ptr(B), ldb, float(beta), ptr(ref), ldc) == 0
+    return ref
+
+
+def normwise(orc, dtype, got, ref, M, N, ldc, alpha, beta, A, ra, ca, lda, B, rb, cb, ldb, C0):
+    if dtype == np.float64:
+        d = abs(alpha) * orc.orc_fro_norm_f64(ptr(A), ra, ca, lda) * orc.orc_fro_norm_f64(ptr(B), rb, cb, ldb) + abs(beta) * orc.orc_fro_norm_f64(ptr(C0), M, N, ldc)
+        return orc.orc_normwise_err_f64(ptr(got), ptr(ref), M, N, ldc, ldc, d)
+    d = abs(alpha) * orc.orc_fro_norm_f32(ptr(A), ra, ca, lda) * orc.orc_fro_norm_f32(ptr(B), rb, cb, ldb) + abs(beta) * orc.orc_fro_norm_f32(ptr(C0), M, N, ldc)
+    return orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, ldc, ldc, d)
+
+
+LOCS = [(-1, -1, -1), (0, 0, 0), (-1, -1, 0), (0, -1, -1), (-1, 0, -1), (0, 0, -1), (-2, -2, -2), (-2, 0, -1)]
+
+
+@pytest.mark.parametrize("locs", LOCS)
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_dgemm_placements_and_transposes(pkg, L, orc, openblas, locs, ta, tb):
+    """The reference tester's 'weird' dimensions (dgemm_tester.cpp:133), its alpha/beta (:74-75) and sub-matrix views
+    with a leading dimension larger than the rows (:48,78); T = 128 gives 3 x 3 x 3 tiles with ragged edges."""
+    M, N, K = 289, 353, 307
+    alpha, beta = 1.23, 0.9876
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = 400, 400, 400
+    A, B, C0 = rand_f64(lda * ca, 42), rand_f64(ldb * cb, 43), rand_f64(ldc * N, 44)
+    bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, C0, locs[2])
+    info = call_gemm(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, bA, lda, bB, ldb, bC, ldc, T=128)
+    got = bC.get()
+    ref = openblas_ref(openblas, np.float64, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    assert normwise(orc, np.float64, got, ref, M, N, ldc, alpha, beta, A, ra, ca, lda, B, rb, cb, ldb, C0) < TOL64
+    tiled = C0.copy()
+    orc.orc_dgemm_tiled(128, 1 if locs[2] >= 0 else 0, ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(tiled), ldc)
+    assert normwise(orc, np.float64, got, tiled, M, N, ldc, alpha, beta, A, ra, ca, lda, B, rb, cb, ldb, C0) < TOL64
+    pad = np.ones(ldc * N, dtype=bool)
+    pad.reshape(N, ldc)[:, :M] = False
+    assert np.array_equal(got[pad], C0[pad])
+    assert info.T == 128 and info.selected_by == b"user" and info.subkernel_num == 27
+    assert np.array_equal(bA.get(), A) and np.array_equal(bB.get(), B)  # inputs are never written
+
+
+@pytest.mark.parametrize("T", [64, 100, 256, 512, 1000])
+@pytest.mark.parametrize("beta", [0.0, 3.0])
+def test_dgemm_tiled_exact_on_integers(pkg, L, orc, T, beta):
+    """Integer-valued operands in pinned host memory: the streamed, tiled result must equal the untiled one bit for
+    bit for every tile size, including T larger than K (tiles shallower than wide) and beta = 0 over NaN."""
+    M, N, K = 700, 520, 300
+    rng = np.random.default_rng(T)
+    A = rng.integers(-8, 9, M * K).astype(np.float64)
+    B = rng.integers(-8, 9, K * N).astype(np.float64)
+    C0 = rng.integers(-8, 9, M * N).astype(np.float64)
+    ref = C0.copy()
+    orc.orc_dgemm_bruteforce(b"N", b"N", M, N, K, 2.0, ptr(A), M, ptr(B), K, beta, ptr(ref), M)
+    start = np.full(M * N, np.nan) if beta == 0.0 else C0
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, start, -1)
+    info = call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 2.0, beta, bA, M, bB, K, bC, M, T=T)
+    assert info.T == min(T, max(M, N, K))  # a tile larger than every dimension is the whole problem
+    assert np.array_equal(bC.get(), ref)
+
+
+@pytest.mark.parametrize("blocks", [3, 4, 6, 11])
+def test_dgemm_block_pool_smaller_than_working_set(pkg, L, orc, openblas, blocks):
+    """cache_limit (the ...Controled knob) below the working set: tiles are evicted and fetched again; the result
+    does not change.  Fewer than 3 blocks is the reference's error (dgemm.cpp:41-42)."""
+    M = N = K = 640
+    T = 128
+    A, B, C0 = rand_f64(M * K, 1), rand_f64(K * N, 2), rand_f64(M * N, 3)
+    ref = openblas_ref(openblas, np.float64, "N", "T", M, N, K, 1.5, 0.5, A, M, B, N, C0, M)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    limit = blocks * T * T * 8
+    L.PARALiA_dev_cache_free(0)
+    info = call_gemm(pkg, L, np.float64, "N", "T", M, N, K, 1.5, 0.5, bA, M, bB, N, bC, M, T=T, cache_limit=limit)
+    assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.5, 0.5, A, M, K, M, B, N, K, N, C0) < TOL64
+    pool = C.c_longlong()
+    L.PARALiA_runtime_stats(None, None, C.byref(pool), None)
+    assert 0 < pool.value <= limit
+    L.PARALiA_dev_cache_free(0)
+    L.PARALiA_runtime_stats(None, None, C.byref(pool), None)
+    assert pool.value == 0
+
+
+def test_dgemm_too_little_memory_is_an_error(pkg, L):
+    M = N = K = 512
+    A = rand_f64(M * K, 1)
+    b = place(pkg, A, -1)
+    rc = L.PARALiA_dgemm(b"N", b"N", M, N, K, 1.0, b.ptr, M, b.ptr, K, 0.0, b.ptr, M, 128, 2 * 128 * 128 * 8, None)
+    assert rc != 0 and b"less memory" in L.PARALiA_last_error()
+    assert L.PARALiA_dgemm(b"N", b"X", M, N, K, 1.0, b.ptr, M, b.ptr, K, 0.0, b.ptr, M, -1, 0, None) != 0
+    assert b"transpose" in L.PARALiA_last_error()
+    assert L.PARALiA_dgemm(b"N", b"N", M, N, K, 1.0, b.ptr, M - 1, b.ptr, K, 0.0, b.ptr, M, -1, 0, None) != 0
+    assert b"leading dimension" in L.PARALiA_last_error()
+    assert L.PARALiA_dgemm(b"N", b"N", 0, N, K, 1.0, b.ptr, 1, b.ptr, K, 0.0, b.ptr, 1, -1, 0, None) == 0  # empty: nothing to do
+
+
+def test_dgemm_metadata_reuse(pkg, L, orc, openblas):
+    """A second call with the same shape and operand locations reuses the tuned problem (the reference's PMD cache,
+    dgemm.cpp:342-368) and still sees the new data."""
+    M, N, K, T = 384, 256, 320, 128
+    L.PARALiA_runtime_reset()
+    hits, misses = C.c_long(), C.c_long()
+    for seed in (1, 2, 3):
+        A, B, C0 = rand_f64(M * K, seed), rand_f64(K * N, seed + 10), rand_f64(M * N, seed + 20)
+        bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 1.0, bA, M, bB, K, bC, M, T=T)
+        ref = openblas_ref(openblas, np.float64, "N", "N", M, N, K, 1.0, 1.0, A, M, B, K, C0, M)
+        assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.0, 1.0, A, M, K, M, B, K, N, K, C0) < TOL64
+    L.PARALiA_runtime_stats(C.byref(hits), C.byref(misses), None, None)
+    assert misses.value == 1 and hits.value == 2
+
+
+def test_dgemm_alpha_zero_and_k_zero(pkg, L):
+    M, N = 300, 200
+    C0 = rand_f64(M * N, 5)
+    junk = np.full(16, np.nan)
+    bJ, bC = place(pkg, junk, -1), place(pkg, C0, -1)
+    call_gemm(pkg, L, np.float64, "N", "N", M, N, 50, 0.0, 0.5, bJ, M, bJ, 50, bC, M, T=128)
+    assert np.array_equal(bC.get(), 0.5 * C0)  # alpha == 0: A and B are not referenced
+    bC.set(C0)
+    call_gemm(pkg, L, np.float64, "N", "N", M, N, 0, 1.0, 2.0, bJ, M, bJ, 1, bC, M, T=128)
+    assert np.array_equal(bC.get(), 2.0 * C0)
+
+
+def test_dgemm_autotuned_call(pkg, L, orc, openblas):
+    """No preset: the autotuner picks T; config 1 of the benchmark set at a quarter of its size."""
+    M = N = K = 1024
+    alpha, beta = 1.2, 1.1
+    A, B, C0 = rand_f64(M * K, 0), rand_f64(K * N, 1), rand_f64(M * N, 2)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    info = call_gemm(pkg, L, np.float64, "N", "N", M, N, K, alpha, beta, bA, M, bB, K, bC, M)
+    assert 0 < info.T <= 1024 and info.subkernel_num >= 1
+    ref = openblas_ref(openblas, np.float64, "N", "N", M, N, K, alpha, beta, A, M, B, K, C0, M)
+    assert normwise(orc, np.float64, bC.get(), ref, M, N, M, alpha, beta, A, M, K, M, B, K, N, K, C0) < TOL64
+
+
+@pytest.mark.parametrize("locs", [(-1, -1, 0), (-1, -1, -1), (0, 0, 0)])
+def test_sgemm_mixed_locations(pkg, L, orc, openblas, locs):
+    """Shape of benchmark config 4 in small: fp32, transA = N, transB = T, alpha = beta = 1, A and B in pinned host
+    memory, C resident on the device."""
+    M, N, K, T = 520, 390, 450, 128
+    A, B, C0 = rand_f32(M * K, 1), rand_f32(N * K, 2), rand_f32(M * N, 3)
+    bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, C0, locs[2])
+    call_gemm(pkg, L, np.float32, "N", "T", M, N, K, 1.0, 1.0, bA, M, bB, N, bC, M, T=T)
+    ref = openblas_ref(openblas, np.float32, "N", "T", M, N, K, 1.0, 1.0, A, M, B, N, C0, M)
+    assert normwise(orc, np.float32, bC.get(), ref, M, N, M, 1.0, 1.0, A, M, K, M, B, N, K, N, C0) < TOL32
+
+
+def test_dgemm_large_checksum(pkg, L):
+    """4096^3 with host operands (benchmark config 1 on the GPU path): a full OpenBLAS product is replaced by the
+    size-independent identity (alpha*A*B + beta*C0) v = alpha*A*(B*v) + beta*(C0*v) for a random v, evaluated in
+    O(n^2) on the CPU."""
+    n = 4096
+    alpha, beta = 1.2, 1.1
+    A, B, C0 = rand_f64(n * n, 0), rand_f64(n * n, 1), rand_f64(n * n, 2)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    info = call_gemm(pkg, L, np.float64, "N", "N", n, n, n, alpha, beta, bA, n, bB, n, bC, n)
+    got = bC.get().reshape(n, n).T  # column-major
+    v = rand_f64(n, 3)
+    Am, Bm, Cm = A.reshape(n, n).T, B.reshape(n, n).T, C0.reshape(n, n).T
+    expect = alpha * (Am @ (Bm @ v)) + beta * (Cm @ v)
+    err = np.linalg.norm(got @ v - expect) / (abs(alpha) * np.linalg.norm(Am) * np.linalg.norm(Bm) * np.linalg.norm(v) + abs(beta) * np.linalg.norm(Cm) * np.linalg.norm(v))
+    assert err < TOL64
+    # and three random 64 x 64 panels against numpy in long double
+    rng = np.random.default_rng(0)
+    for _ in range(3):
+        i, j = rng.integers(0, n - 64, 2)
+        blk = alpha * (Am[i:i + 64, :].astype(np.longdouble) @ Bm[:, j:j + 64].astype(np.longdouble)) + beta * Cm[i:i + 64, j:j + 64]
+        d = np.linalg.norm((got[i:i + 64, j:j + 64] - blk).astype(np.float64))
+        assert d / (abs(alpha) * np.linalg.norm(Am[i:i + 64, :]) * np.linalg.norm(Bm[:, j:j + 64]) + abs(beta) * np.linalg.norm(Cm[i:i + 64, j:j + 64])) < TOL64
+
+
+def scaled_ulp(a, b, alpha, x, y0):
+    scale = np.maximum(np.maximum(np.abs(alpha * x), np.abs(y0)), np.maximum(np.abs(a), np.abs(b)))
+    return float(np.max(np.abs(a - b) / np.spacing(scale)))
+
+
+@pytest.mark.parametrize("locs", [(0, 0), (-1, -1), (-1, 0), (0, -1), (-2, -2)])
+@pytest.mark.parametrize("T", [-1, 1000, 1 << 16])
+def test_daxpy_routine(pkg, L, orc, openblas, locs, T):
+    n, alpha = (1 << 18) + 37, 0.7
+    x, y0 = rand_f64(n, 1), rand_f64(n, 2)
+    bx, by = place(pkg, x, locs[0]), place(pkg, y0, locs[1])
+    info = pkg.atc_info()
+    print("PARALiA daxpy", n, locs, T, flush=True)
+    pkg.check(L.PARALiA_daxpy(n, alpha, bx.ptr, 1, by.ptr, 1, T, C.byref(info)), "PARALiA_daxpy")
+    got = by.get()
+    fused = y0.copy()
+    orc.orc_daxpy(n, alpha, ptr(x), 1, ptr(fused), 1)
+    assert np.array_equal(got, fused)
+    ref = y0.copy()
+    assert openblas.orc_openblas_daxpy(n, alpha, ptr(x), 1, ptr(ref), 1) == 0
+    assert orc.orc_max_ulp_f64(ptr(got), ptr(ref), n) <= 1 or scaled_ulp(got, ref, alpha, x, y0) <= 1.5
+    assert np.array_equal(bx.get(), x)
+    if T > 0 and min(locs) < 0:
+        assert info.T == T and info.subkernel_num == -(-n // T)
+
+
+def test_daxpy_routine_strided_host(pkg, L, orc):
+    n = 40001
+    x, y0 = rand_f64(2 * n, 3), rand_f64(3 * n, 4)
+    for incx, incy in ((2, 3), (-2, 3), (2, -3), (1, -1)):
+        bx, by = place(pkg, x, -1), place(pkg, y0, -1)
+        pkg.check(L.PARALiA_daxpy(n, -1.5, bx.ptr, incx, by.ptr, incy, 7000, None), "PARALiA_daxpy strided")
+        ref = y0.copy()
+        orc.orc_daxpy(n, -1.5, ptr(x), incx, ptr(ref), incy)
+        assert np.array_equal(by.get(), ref), (incx, incy)
+
+
+@pytest.mark.parametrize("locs", [(0, 0), (-1, -1), (-1, 0), (-2, -1)])
+@pytest.mark.parametrize("T", [-1, 5000, 1 << 17])
+def test_ddot_routine(pkg, L, orc, openblas, locs, T):
+    n = (1 << 19) + 11
+    x, y = rand_f64(n, 5), rand_f64(n, 6)
+    bx, by = place(pkg, x, locs[0]), place(pkg, y, locs[1])
+    res = C.c_double(0.0)
+    print("PARALiA ddot", n, locs, T, flush=True)
+    pkg.check(L.PARALiA_ddot(n, bx.ptr, 1, by.ptr, 1, C.byref(res), T, None), "PARALiA_ddot")
+    exact = float(orc.orc_ddot_longdouble(n, ptr(x), 1, ptr(y), 1))
+    bound = 1e-13 * float(np.linalg.norm(x) * np.linalg.norm(y))
+    assert abs(res.value - exact) <= bound
+    ob = C.c_double()
+    assert openblas.orc_openblas_ddot(n, ptr(x), 1, ptr(y), 1, C.byref(ob)) == 0
+    assert abs(res.value - ob.value) <= bound
+    if T > 0:
+        tiled = C.c_double(0.0)
+        orc.orc_ddot_tiled(T, n, ptr(x), 1, ptr(y), 1, C.byref(tiled))
+        assert abs(res.value - tiled.value) <= bound
+    # the routine adds into *result, as the reference does (ddot.cpp:431)
+    first = res.value
+    pkg.check(L.PARALiA_ddot(n, bx.ptr, 1, by.ptr, 1, C.byref(res), T, None), "PARALiA_ddot again")
+    assert res.value == first + first
+
+
+def test_blas1_edge_cases(pkg, L):
+    x = rand_f64(16, 1)
+    bx = place(pkg, x, -1)
+    res = C.c_double(5.0)
+    assert L.PARALiA_ddot(0, bx.ptr, 1, bx.ptr, 1, C.byref(res), -1, None) == 0 and res.value == 5.0
+    assert L.PARALiA_daxpy(0, 1.0, bx.ptr, 1, bx.ptr, 1, -1, None) == 0
+    assert L.PARALiA_daxpy(4, 1.0, bx.ptr, 0, bx.ptr, 1, -1, None) != 0 and b"increment" in L.PARALiA_last_error()
+    assert L.PARALiA_daxpy(-1, 1.0, bx.ptr, 1, bx.ptr, 1, -1, None) != 0
+    assert L.PARALiA_ddot(4, bx.ptr, 1, bx.ptr, 1, None, -1, None) != 0
+    ones = place(pkg, np.ones(100003), -1)
+    res = C.c_double(0.0)
+    assert L.PARALiA_ddot(100003, ones.ptr, 1, ones.ptr, 1, C.byref(res), 1000, None) == 0 and res.value == 100003.0
+
+
+def test_vec_init_matches_oracle_generator(pkg, L):
+    """The drivers' seeded fill (CoCoVecInit) produces the oracle's stream wherever the buffer lives."""
+    n = 100000
+    for loc in (0, -1, -2):
+        b = Buf(pkg, n, np.float64, loc)
+        pkg.check(L.PARALiA_vec_init_f64(b.ptr, n, 42, loc), "vec init")
+        assert np.array_equal(b.get(), rand_f64(n, 42))
+    b = Buf(pkg, n, np.float32, 0)
+    pkg.check(L.PARALiA_vec_init_f32(b.ptr, n, 7, 0), "vec init f32")
+    assert np.array_equal(b.get(), rand_f32(n, 7))
