@@ -19,6 +19,12 @@
 #include <stdint.h>
 
 // Row index (MFMA i) of accumulator element r for lane group g = lane / 16 in the 16x16 fp64 result block.
+#ifndef PLK_F64_BK
+#define PLK_F64_BK 16
+#endif
+#ifndef PLK_WAVES_PER_EU
+#define PLK_WAVES_PER_EU 2
+#endif
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
 #endif
@@ -38,12 +44,13 @@ template <> struct Traits<double> {
   using vec_t = dvec2;
   using acc_t = double4_t;
   static constexpr int VEC = 2;      // elements per 16-byte vector
-  static constexpr int BK = 16;      // k-panel depth
+  static constexpr int BK = PLK_F64_BK;  // k-panel depth
   static constexpr int BLK = 16;     // MFMA block edge
   static constexpr int KSTEP = 4;    // k consumed per MFMA
   static constexpr int NACC = 4;     // accumulator elements per lane per block
   static constexpr int S_MN = 144;   // LDS row stride, [k][mn] layout (1152 B = 128 mod 256)
-  static constexpr int S_K = 18;     // LDS row stride, [mn][k] layout (144 B)
+  static constexpr int S_K = BK + 2; // LDS row stride, [mn][k] layout
+  static constexpr int NV = 128 * BK / VEC / 256;  // 16-byte vectors per thread per panel
   static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
@@ -61,6 +68,7 @@ template <> struct Traits<float> {
   static constexpr int NACC = 16;
   static constexpr int S_MN = 160;   // 640 B = 128 mod 256
   static constexpr int S_K = 36;     // 144 B
+  static constexpr int NV = 128 * BK / VEC / 256;
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -74,7 +82,7 @@ template <typename T, bool KMAJOR> struct Lds {
   static __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * Tr::S_K + k : k * Tr::S_MN + mn; }
 };
 
-// One thread's share of a 128 x BK panel: four 16-byte vectors.  "c" runs along the memory-contiguous
+// One thread's share of a 128 x BK panel: NV 16-byte vectors.  "c" runs along the memory-contiguous
 // dimension (mn for MN-major operands, k for K-major ones), "s" along the leading-dimension stride.
 template <typename T, bool KMAJOR> struct Slot {
   using Tr = Traits<T>;
@@ -88,11 +96,11 @@ template <typename T, bool KMAJOR> struct Slot {
 
 template <typename T, bool KMAJOR, bool GUARD>
 __device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int crem, int srem, bool vec_ok,
-                                      typename Traits<T>::vec_t (&regs)[4], int tid) {
+                                      typename Traits<T>::vec_t (&regs)[Traits<T>::NV], int tid) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < Tr::NV; ++i) {
     int c, s;
     Slot<T, KMAJOR>::coords(tid, i, c, s);
     const T* p = base + c + (long)s * ld;
@@ -117,11 +125,11 @@ __device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int c
 }
 
 template <typename T, bool KMAJOR>
-__device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[4], int tid) {
+__device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[Traits<T>::NV], int tid) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < Tr::NV; ++i) {
     int c, s;
     Slot<T, KMAJOR>::coords(tid, i, c, s);
     // the contiguous run is also contiguous in LDS for both layouts
@@ -149,7 +157,7 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
 template <typename T, bool AK, bool BKM>
-__global__ __launch_bounds__(NTHREADS, 2) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
+__global__ __launch_bounds__(NTHREADS, PLK_WAVES_PER_EU) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
                                                           long ldc, int gm, int gn, int vecA, int vecB) {
   using Tr = Traits<T>;
@@ -188,7 +196,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_kernel(int M, int N, int K, 
 
   const int nkt = (K + BK - 1) / BK;
   const int nfull = K / BK;
-  vec_t ra[4], rb[4];
+  vec_t ra[Tr::NV], rb[Tr::NV];
 
   auto fetch = [&](int kt) {
     const T* ap = Ab + kt * a_kstep;
@@ -215,6 +223,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_kernel(int M, int N, int K, 
     if (kt + 1 < nkt) fetch(kt + 1);
     const T* as = smem + cur * STAGE;
     const T* bs = as + ASZ;
+#ifdef PLK_SETPRIO
+    __builtin_amdgcn_s_setprio(PLK_SETPRIO);
+#endif
 #pragma unroll
     for (int ks = 0; ks < BK / Tr::KSTEP; ++ks) {
       T am[NB], bnv[NB];
@@ -228,6 +239,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_kernel(int M, int N, int K, 
 #pragma unroll
         for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[i], am[j], acc[i][j]);
     }
+#ifdef PLK_SETPRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
     if (kt + 1 < nkt) {
       lds_store<T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
       lds_store<T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
