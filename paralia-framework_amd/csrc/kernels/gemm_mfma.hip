@@ -79,7 +79,7 @@ template <typename T, bool KMAJOR> struct Lds {
   using Tr = Traits<T>;
   // elements of one staged panel (128 x BK plus padding)
   static constexpr int SIZE = KMAJOR ? 128 * Tr::S_K : Tr::BK * Tr::S_MN;
-  static __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * Tr::S_K + k : k * Tr::S_MN + mn; }
+  static constexpr __host__ __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * Tr::S_K + k : k * Tr::S_MN + mn; }
 };
 
 // One thread's share of a 128 x BK panel: NV 16-byte vectors.  "c" runs along the memory-contiguous
@@ -122,6 +122,21 @@ __device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int c
       regs[i] = v;
     }
   }
+}
+
+// Slot i only, unguarded: the pieces the pipelined loop spreads between MFMAs.
+template <typename T, bool KMAJOR>
+__device__ __forceinline__ void gload_one(const T* __restrict__ base, long ld, typename Traits<T>::vec_t& reg, int tid, int i) {
+  int c, s;
+  Slot<T, KMAJOR>::coords(tid, i, c, s);
+  reg = *reinterpret_cast<const typename Traits<T>::vec_t*>(base + c + (long)s * ld);
+}
+template <typename T, bool KMAJOR>
+__device__ __forceinline__ void lds_store_one(T* __restrict__ xs, const typename Traits<T>::vec_t& reg, int tid, int i) {
+  int c, s;
+  Slot<T, KMAJOR>::coords(tid, i, c, s);
+  const int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
+  *reinterpret_cast<typename Traits<T>::vec_t*>(xs + off) = reg;
 }
 
 template <typename T, bool KMAJOR>
@@ -211,42 +226,110 @@ __global__ __launch_bounds__(NTHREADS, PLK_WAVES_PER_EU) void gemm_kernel(int M,
     }
   };
 
-  if (nkt > 0) {
-    fetch(0);
+  const T* const lane_a = smem + Lds<T, AK>::at(kk, wm + idx);         // this lane's A operand of k-step 0, block 0
+  const T* const lane_b = smem + ASZ + Lds<T, BKM>::at(kk, wn + idx);  // this lane's B operand
+  constexpr int A_KS = Lds<T, AK>::at(Tr::KSTEP, 0), A_BL = Lds<T, AK>::at(0, BLK);    // strides per k-step / per block
+  constexpr int B_KS = Lds<T, BKM>::at(Tr::KSTEP, 0), B_BL = Lds<T, BKM>::at(0, BLK);
+  constexpr int KS = BK / Tr::KSTEP;
+
+  auto read_ops = [&](int buf, int ks, T (&am)[NB], T (&bnv)[NB]) {
+#pragma unroll
+    for (int j = 0; j < NB; ++j) am[j] = lane_a[buf * STAGE + ks * A_KS + j * A_BL];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) bnv[i] = lane_b[buf * STAGE + ks * B_KS + i * B_BL];
+  };
+  auto mfma_step = [&](const T (&am)[NB], const T (&bnv)[NB]) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[i], am[j], acc[i][j]);
+  };
+
+  if (fast && nkt > 0 && nfull == nkt) {
+    // Software-pipelined main loop (interior workgroup, K a multiple of the panel depth).  Per k-panel:
+    //   k-step 0     : store the prefetched panel kt+1 (registers -> LDS buffer cur^1), issue the global loads of
+    //                  panel kt+2, read the operands of k-step 1, multiply with the operands of k-step 0;
+    //   k-steps 1..  : read the operands of the next k-step while multiplying the current one;
+    //   last k-step  : barrier first (everyone is done reading buffer cur and writing buffer cur^1), read the
+    //                  operands of panel kt+1's first k-step, multiply the last operands of panel kt.
+    // So every LDS read, LDS write and global load is issued under the shadow of 16 (fp64) / 4 (fp32) MFMAs, and
+    // one barrier per panel sits where the MFMA queue still has a k-step of work behind it.  The loop body has
+    // no branches: past the end, the loads re-read the last panel and the stores fill a buffer nobody reads.
+    T am[2][NB], bnv[2][NB];
+    auto fetch_fast = [&](int kt) {
+      gload<T, AK, false>(Ab + kt * a_kstep, lda, 0, 0, true, ra, tid);
+      gload<T, BKM, false>(Bb + kt * b_kstep, ldb, 0, 0, true, rb, tid);
+    };
+    fetch_fast(0);
     lds_store<T, AK>(smem, ra, tid);
     lds_store<T, BKM>(smem + ASZ, rb, tid);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < nkt; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nkt) fetch(kt + 1);
-    const T* as = smem + cur * STAGE;
-    const T* bs = as + ASZ;
-#ifdef PLK_SETPRIO
-    __builtin_amdgcn_s_setprio(PLK_SETPRIO);
-#endif
+    fetch_fast(min(1, nkt - 1));
+    __syncthreads();
+    read_ops(0, 0, am[0], bnv[0]);
+    constexpr int NV = Tr::NV, SIDE = 4 * NV;              // 2*NV LDS stores, then 2*NV global loads
+    constexpr int PER_STEP = (SIDE + KS - 2) / (KS - 1);     // side instructions placed in each pre-barrier k-step
+    constexpr int MFMAS = NB * NB;
+    for (int kt = 0; kt < nkt; ++kt) {
+      const int cur = kt & 1;
+      T* const nxt_a = smem + (cur ^ 1) * STAGE;
+      T* const nxt_b = nxt_a + ASZ;
+      const int kt2 = min(kt + 2, nkt - 1);
+      const T* const ga = Ab + kt2 * a_kstep;
+      const T* const gb = Bb + kt2 * b_kstep;
 #pragma unroll
-    for (int ks = 0; ks < BK / Tr::KSTEP; ++ks) {
-      T am[NB], bnv[NB];
-      const int k = ks * Tr::KSTEP + kk;
+      for (int ks = 0; ks < KS - 1; ++ks) {
+        read_ops(cur, ks + 1, am[(ks + 1) & 1], bnv[(ks + 1) & 1]);
 #pragma unroll
-      for (int j = 0; j < NB; ++j) am[j] = as[Lds<T, AK>::at(k, wm + j * BLK + idx)];
+        for (int q = 0; q < PER_STEP; ++q) {
+          const int slot = ks * PER_STEP + q;
+          if (slot < NV) lds_store_one<T, AK>(nxt_a, ra[slot], tid, slot);
+          else if (slot < 2 * NV) lds_store_one<T, BKM>(nxt_b, rb[slot - NV], tid, slot - NV);
+          else if (slot < 3 * NV) gload_one<T, AK>(ga, lda, ra[slot - 2 * NV], tid, slot - 2 * NV);
+          else if (slot < SIDE) gload_one<T, BKM>(gb, ldb, rb[slot - 3 * NV], tid, slot - 3 * NV);
+        }
+        mfma_step(am[ks & 1], bnv[ks & 1]);
+        // issue order inside the k-step: operand reads first, then one side instruction after every few MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
 #pragma unroll
-      for (int i = 0; i < NB; ++i) bnv[i] = bs[Lds<T, BKM>::at(k, wn + i * BLK + idx)];
-#pragma unroll
-      for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[i], am[j], acc[i][j]);
+        for (int q = 0; q < PER_STEP; ++q) {
+          const int slot = ks * PER_STEP + q;
+          __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / PER_STEP > 0 ? MFMAS / PER_STEP : 1, 0);
+          if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();
+      read_ops(cur ^ 1, 0, am[KS & 1], bnv[KS & 1]);
+      mfma_step(am[(KS - 1) & 1], bnv[(KS - 1) & 1]);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-#ifdef PLK_SETPRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
-    if (kt + 1 < nkt) {
-      lds_store<T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
-      lds_store<T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
+  } else {
+    // General loop: edge workgroups, ragged K, unaligned operands.  Same double buffering, loads guarded.
+    if (nkt > 0) {
+      fetch(0);
+      lds_store<T, AK>(smem, ra, tid);
+      lds_store<T, BKM>(smem + ASZ, rb, tid);
     }
     __syncthreads();
+    for (int kt = 0; kt < nkt; ++kt) {
+      const int cur = kt & 1;
+      if (kt + 1 < nkt) fetch(kt + 1);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        T am[NB], bnv[NB];
+        read_ops(cur, ks, am, bnv);
+        mfma_step(am, bnv);
+      }
+      if (kt + 1 < nkt) {
+        lds_store<T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
+        lds_store<T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
+      }
+      __syncthreads();
+    }
   }
 
   // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk))
