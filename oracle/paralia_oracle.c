@@ -90,17 +90,19 @@ long long orc_max_ulp_f64(const double* a, const double* b, long long n) {
 }
 
 /* Own definition of "matching digits" (the reference's Dtest_equality is not in its tree): the smallest over
- * all elements of floor(-log10(relative difference)), capped at 16; the drivers demand >= 9
- * (dgemm_runner.cpp:99). */
+ * all elements of floor(-log10(|ref_i - x_i| / max(|ref_i|, |x_i|, rms(ref)))), capped at 16; the drivers demand
+ * >= 9 (dgemm_runner.cpp:99).  The rms term keeps elements that are small by cancellation on the vector's scale. */
 int orc_digits_equal(const double* ref, const double* x, long long n) {
+  long double ss = 0;
+  for (long long i = 0; i < n; ++i) ss += (long double)ref[i] * ref[i];
+  const double rms = n > 0 ? (double)sqrtl(ss / n) : 0.0;
   int worst = 16;
   for (long long i = 0; i < n; ++i) {
     double d = fabs(ref[i] - x[i]);
     if (d == 0) continue;
     if (isnan(d)) return 0;
-    double scale = fmax(fabs(ref[i]), fabs(x[i]));
-    double rel = d / scale;
-    int digits = (int)floor(-log10(rel));
+    double scale = fmax(fmax(fabs(ref[i]), fabs(x[i])), rms);
+    int digits = (int)floor(-log10(d / scale));
     if (digits < 0) digits = 0;
     if (digits < worst) worst = digits;
   }
@@ -425,7 +427,7 @@ double orc_predict_blas3(int mode, const orc_problem* p, long T) {
       one_over += gemm_in[i] * p->remote[i] * (d1 / T) * (d2 / T);
       if (t_recv > t_exec)
         for (int j = i + 1; j < 3; ++j)
-          if (gemm_in[i] * p->remote[i] && gemm_in[j] * p->remote[j]) {
+          if ((gemm_in[i] * p->remote[i]) != 0 && (gemm_in[j] * p->remote[j]) != 0) {
             /* the shared dimension of operands i and j: (A,B) share D3 = Dim2 of A; (A,C) share D1 = Dim1 of A;
              * (B,C) share D2 = Dim2 of B.  The reference tests Dim1[i] first, then Dim2[i]. */
             if (i == 0 && j == 2) two_over += d1 / T - 1;

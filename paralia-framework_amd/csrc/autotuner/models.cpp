@@ -132,7 +132,7 @@ double Modeler::predict(ModelType mode, long T) const {
         one_over += rin * (d1 / T) * (d2 / T);
         if (t_recv > t_exec)
           for (int j = i + 1; j < P.numT; ++j)
-            if (rin && P.in[j] * remote(P.loc[j], unit_id)) {
+            if (rin != 0 && (P.in[j] * remote(P.loc[j], unit_id)) != 0) {
               // tiles of operands i and j that can be fetched under one kernel share a dimension:
               // A-C share D1 (= Dim1 of A); A-B share D3 and B-C share D2 (= Dim2 of the first)
               two_over += ((i == 0 && j == 2) ? d1 : d2) / T - 1;

@@ -1,0 +1,326 @@
+// Deploy-time microbenchmarks and database builder for one MI355X.
+//
+//   paralia_deploy <db_dir> [--quick] [--only gemm|blas1|link]
+//
+// Measures (1) the tile GEMM kernels over square T for the four transpose combinations, fp64 and fp32,
+// (2) daxpy / ddot over vector lengths, (3) pinned-host <-> device 2-D tile copies in both directions and the
+// slowdown of each direction while the other is busy; writes the raw logs to <db_dir>/Benchmark-Results and the
+// tables the autotuner reads to <db_dir>/Processed.
+//
+// What it re-does from the reference: Database_builder/CuCuBLAS/src/dgemm_microbench.cu:26-230 (T sweep from
+// 256 in steps of 256, the step doubling once T >= 16*step, up to < 10000; alpha = 1.1234, beta = 1.2345;
+// stop when the 95% confidence half-width is within 5% of the mean and more than 10 samples were taken),
+// daxpy_microbench.cu / ddot_microbench.cu (sweep from 4096 in steps of 4096 with the same doubling),
+// transfer_link_microbench.cu:24-218 (square tiles with a host leading dimension of maxDim + 1, then the
+// overlap run), Python-DataManage/BenchToLookupTables.py.in:31-55 (flag columns prepended, sorted by T) and
+// LinkPreprocessing.py.in:44-61 (least-squares line bytes -> seconds, |intercept|, slowdown ratios).
+// File formats are unchanged so the tables are interchangeable with the reference's.
+// Kernel times are taken the way the scheduler runs the kernels: launches round-robin over its compute
+// streams, time per launch = wall time of a batch / launches in it.
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <sys/stat.h>
+#include <vector>
+
+#include "Autotuner.hpp"
+#include "backend_wrappers.hpp"
+#include "paralia_hip.h"
+
+#define DEPLOY_VERSION "2.0"
+#define MICRO_MIN_ITER 10
+#define MICRO_MAX_ITER 100
+
+static void must(int rc, const char* what) {
+  if (rc != 0) {
+    fprintf(stderr, "paralia_deploy: %s failed (%d): %s\n", what, rc, pl_last_error());
+    exit(1);
+  }
+}
+
+// two-sided 95% Student-t quantile
+static double t975(int df) {
+  static const double tab[] = {0,      12.706, 4.303, 3.182, 2.776, 2.571, 2.447, 2.365, 2.306, 2.262, 2.228,
+                               2.201,  2.179,  2.160, 2.145, 2.131, 2.120, 2.110, 2.101, 2.093, 2.086, 2.080,
+                               2.074,  2.069,  2.064, 2.060, 2.056, 2.052, 2.048, 2.045, 2.042};
+  if (df < 1) return 1e9;
+  if (df <= 30) return tab[df];
+  return 1.96 + 2.5 / df;
+}
+
+struct Sample { double mean = 0, margin = 0, bench_t = 0; long n = 0; };
+
+// Repeats run() until the 95% CI half-width is within 5% of the mean (n > MICRO_MIN_ITER) or MICRO_MAX_ITER.
+template <typename F> static Sample sample_until_stable(F&& run) {
+  std::vector<double> v;
+  Sample s;
+  const double t_start = csecond();
+  double sum = 0;
+  for (int i = 1; i <= MICRO_MAX_ITER; ++i) {
+    const double t = run();
+    v.push_back(t);
+    sum += t;
+    s.mean = sum / i;
+    s.n = i;
+    if (i < 2) continue;
+    double var = 0;
+    for (double x : v) var += (x - s.mean) * (x - s.mean);
+    const double sd = sqrt(var / i);
+    s.margin = t975(i - 1) * sd / sqrt((double)i);
+    if (i > MICRO_MIN_ITER && s.margin / s.mean * 100 <= 5) break;
+  }
+  s.bench_t = csecond() - t_start;
+  return s;
+}
+
+static std::vector<long> sweep(long start, long step, long limit, int double_at) {
+  std::vector<long> out;
+  for (long T = start; T < limit; T += step) {
+    if (T >= step * double_at) step *= 2;
+    out.push_back(T);
+  }
+  return out;
+}
+
+struct Row { char ta, tb; long T; Sample s; };
+
+static void mkdirs(const std::string& d) {
+  mkdir(d.c_str(), 0755);
+  mkdir((d + "/Benchmark-Results").c_str(), 0755);
+  mkdir((d + "/Processed").c_str(), 0755);
+}
+
+template <typename T>
+static void bench_gemm(const std::string& db, const char* func, bool quick, int queues) {
+  const long maxDim = quick ? 4352 : 10000;
+  std::vector<long> Ts = sweep(256, 256, maxDim, 16);
+  if (quick) {
+    std::vector<long> few;
+    for (long t : Ts) if (t == 512 || t == 1024 || t == 2048 || t == 3072 || t == 4096) few.push_back(t);
+    Ts = few;
+  }
+  const long ld = maxDim;
+  T *A, *B, *C;
+  A = (T*)CoCoMalloc(ld * ld * sizeof(T), 0, 0);
+  B = (T*)CoCoMalloc(ld * ld * sizeof(T), 0, 0);
+  C = (T*)CoCoMalloc(2 * ld * ld * sizeof(T), 0, 1);
+  CoCoVecInit(A, ld * ld, 42, 0);
+  CoCoVecInit(B, ld * ld, 43, 0);
+  CoCoVecInit(C, 2 * ld * ld, 44, 0);
+  std::vector<void*> st(queues);
+  for (auto& s : st) must(pl_stream_create(&s), "stream");
+  const T alpha = (T)1.1234, beta = (T)1.2345;
+  std::vector<Row> rows;
+  const char flags[2] = {'N', 'T'};
+  for (char ta : flags)
+    for (char tb : flags) {
+      char raw[1024];
+      snprintf(raw, sizeof raw, "%s/Benchmark-Results/hip%s_dev-0_TransA-%c_TransB-%c_%s.log", db.c_str(), func, ta, tb, DEPLOY_VERSION);
+      FILE* fp = fopen(raw, "w");
+      if (!fp) { fprintf(stderr, "cannot write %s\n", raw); exit(1); }
+      for (long Tt : Ts) {
+        auto launch = [&](int q) {
+          if (sizeof(T) == 8)
+            must(pl_dgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const double*)A, ld, (const double*)B, ld, beta, (double*)(C + (long)q * ld * ld), ld, st[q]), "gemm");
+          else
+            must(pl_sgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const float*)A, ld, (const float*)B, ld, beta, (float*)(C + (long)q * ld * ld), ld, st[q]), "gemm");
+        };
+        const int batch = 2 * queues;
+        auto run = [&]() {
+          const double t0 = csecond();
+          for (int i = 0; i < batch; ++i) launch(i % queues);
+          for (auto s : st) must(pl_stream_sync(s), "sync");
+          return (csecond() - t0) / batch;
+        };
+        run();  // warm-up
+        Row r{ta, tb, Tt, sample_until_stable(run)};
+        rows.push_back(r);
+        fprintf(fp, "%ld,%ld,%ld, %e,%e,%e,%e,%ld,%e\n", Tt, Tt, Tt, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
+        fprintf(stderr, "%s %c%c T=%ld: %.3f ms (%.1f GFLOP/s), margin %.2f%%, %ld samples\n", func, ta, tb, Tt, r.s.mean * 1e3,
+                2.0 * Tt * Tt * Tt / r.s.mean / 1e9, r.s.margin / r.s.mean * 100, r.s.n);
+      }
+      fclose(fp);
+    }
+  // Processed table: flag columns prepended, rows of all four files concatenated and sorted by T
+  std::stable_sort(rows.begin(), rows.end(), [](const Row& a, const Row& b) { return a.T < b.T; });
+  char out[1024];
+  snprintf(out, sizeof out, "%s/Processed/%s_lookup-table_dev-0.log", db.c_str(), func);
+  FILE* fp = fopen(out, "w");
+  if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  for (const Row& r : rows)
+    fprintf(fp, "%c,%c,%ld,%ld,%ld,%e,%e,%e,%e,%ld,%e\n", r.ta, r.tb, r.T, r.T, r.T, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
+  fclose(fp);
+  for (auto s : st) pl_stream_destroy(s);
+  CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
+}
+
+static void bench_blas1(const std::string& db, const char* func, bool quick) {
+  const long maxN = quick ? (1L << 24) + 1 : (1L << 27) + 1;
+  std::vector<long> Ns = sweep(4096, 4096, maxN, 16);
+  if (quick) {
+    std::vector<long> few;
+    for (long n : Ns) if ((n & (n - 1)) == 0 && n >= (1 << 16)) few.push_back(n);
+    Ns = few;
+  }
+  double* x = (double*)CoCoMalloc(maxN * 8, 0, 0);
+  double* y = (double*)CoCoMalloc(maxN * 8, 0, 1);
+  CoCoVecInit(x, maxN, 42, 0);
+  CoCoVecInit(y, maxN, 43, 0);
+  double* ws = (double*)CoCoMalloc((pl_ddot_workspace_doubles() + 1) * 8, 0, 1);
+  void* st;
+  must(pl_stream_create(&st), "stream");
+  const bool axpy = !strcmp(func, "Daxpy");
+  char raw[1024], out[1024];
+  snprintf(raw, sizeof raw, "%s/Benchmark-Results/hip%s_dev-0_%s.log", db.c_str(), func, DEPLOY_VERSION);
+  snprintf(out, sizeof out, "%s/Processed/%s_lookup-table_dev-0.log", db.c_str(), func);
+  FILE* fr = fopen(raw, "w");
+  FILE* fo = fopen(out, "w");
+  if (!fr || !fo) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  for (long N : Ns) {
+    const int batch = 4;
+    auto run = [&]() {
+      const double t0 = csecond();
+      for (int i = 0; i < batch; ++i) {
+        if (axpy) must(pl_daxpy(N, 1.1234, x, 1, y, 1, st), "daxpy");
+        else must(pl_ddot(N, x, 1, y, 1, ws + pl_ddot_workspace_doubles(), 0, ws, st), "ddot");
+      }
+      must(pl_stream_sync(st), "sync");
+      return (csecond() - t0) / batch;
+    };
+    run();
+    Sample s = sample_until_stable(run);
+    fprintf(fr, "%ld, %e,%e,%e,%e,%ld,%e\n", N, s.mean, -1.0, -1.0, s.margin, s.n, s.bench_t);
+    fprintf(fo, "%ld,%e,%e,%e,%e,%ld,%e\n", N, s.mean, -1.0, -1.0, s.margin, s.n, s.bench_t);
+    fprintf(stderr, "%s N=%ld: %.4f ms (%.1f GB/s)\n", func, N, s.mean * 1e3, (axpy ? 24.0 : 16.0) * N / s.mean / 1e9);
+  }
+  fclose(fr);
+  fclose(fo);
+  pl_stream_destroy(st);
+  CoCoFree(x, 0); CoCoFree(y, 0); CoCoFree(ws, 0);
+}
+
+static void bench_link(const std::string& db, bool quick) {
+  const long maxDim = quick ? 4352 : 10000;
+  std::vector<long> dims = sweep(256, 256, maxDim, 8);
+  const long ldh = maxDim + 1;
+  double* host = (double*)CoCoMalloc(ldh * maxDim * 8, -1, 1);
+  double* host2 = (double*)CoCoMalloc(ldh * maxDim * 8, -1, 1);
+  double* dev = (double*)CoCoMalloc(maxDim * maxDim * 8, 0, 1);
+  double* dev2 = (double*)CoCoMalloc(maxDim * maxDim * 8, 0, 1);
+  CoCoVecInit(host, ldh * maxDim, 42, -1);
+  void *s1, *s2;
+  must(pl_stream_create(&s1), "stream");
+  must(pl_stream_create(&s2), "stream");
+  struct Dir { int to, from; } dirs[2] = {{0, -1}, {-1, 0}};
+  for (const Dir& d : dirs) {
+    const bool h2d = d.to == 0;
+    char raw[1024];
+    snprintf(raw, sizeof raw, "%s/Benchmark-Results/hip_link_benchmark_loc_dest-%d_loc_src-%d_%s.log", db.c_str(), d.to, d.from, DEPLOY_VERSION);
+    FILE* fp = fopen(raw, "w");
+    if (!fp) { fprintf(stderr, "cannot write %s\n", raw); exit(1); }
+    auto copy = [&](long dim, void* st, bool forward, double* h, double* dv) {
+      if (forward) must(pl_copy2d_async(dv, dim, h, ldh, dim, dim, 8, st), "h2d copy");
+      else must(pl_copy2d_async(h, ldh, dv, dim, dim, dim, 8, st), "d2h copy");
+    };
+    double sx = 0, sy = 0, sxx = 0, sxy = 0;
+    long np = 0;
+    for (long dim : dims) {
+      const int batch = dim <= 1024 ? 8 : 2;
+      auto run = [&]() {
+        const double t0 = csecond();
+        for (int i = 0; i < batch; ++i) copy(dim, s1, h2d, host, dev);
+        must(pl_stream_sync(s1), "sync");
+        return (csecond() - t0) / batch;
+      };
+      run();
+      Sample s = sample_until_stable(run);
+      fprintf(fp, "%ld,%ld, %e,%e,%ld, %e\n", dim, dim, s.mean, s.margin, s.n, s.bench_t);
+      fprintf(stderr, "link %d<-%d dim=%ld: %.3f ms (%.1f GB/s)\n", d.to, d.from, dim, s.mean * 1e3, dim * dim * 8.0 / s.mean / 1e9);
+      const double b = (double)dim * dim * 8;
+      sx += b; sy += s.mean; sxx += b * b; sxy += b * s.mean;
+      ++np;
+    }
+    fclose(fp);
+    const double tb = (np * sxy - sx * sy) / (np * sxx - sx * sx);
+    const double ti = fabs((sy - tb * sx) / np);
+    // overlap: this direction alone vs. while the opposite direction streams tiles of the same size
+    const long dim = 2048;
+    const int reps = 10;
+    auto alone = [&]() {
+      const double t0 = csecond();
+      for (int i = 0; i < reps; ++i) copy(dim, s1, h2d, host, dev);
+      must(pl_stream_sync(s1), "sync");
+      return (csecond() - t0) / reps;
+    };
+    auto shared = [&]() {
+      for (int i = 0; i < 3 * reps; ++i) copy(dim, s2, !h2d, host2, dev2);  // keeps the other direction busy throughout
+      const double t0 = csecond();
+      for (int i = 0; i < reps; ++i) copy(dim, s1, h2d, host, dev);
+      must(pl_stream_sync(s1), "sync");
+      const double t = (csecond() - t0) / reps;
+      must(pl_stream_sync(s2), "sync");
+      return t;
+    };
+    alone();
+    const double bench0 = csecond();
+    double t_alone = 0, t_shared = 0;
+    for (int i = 0; i < 5; ++i) { t_alone += alone() / 5; t_shared += shared() / 5; }
+    snprintf(raw, sizeof raw, "%s/Benchmark-Results/hip_link_overlap_benchmark_loc_dest-%d_loc_src-%d_%s.log", db.c_str(), d.to, d.from, DEPLOY_VERSION);
+    fp = fopen(raw, "w");
+    if (!fp) { fprintf(stderr, "cannot write %s\n", raw); exit(1); }
+    fprintf(fp, "%d,%d, %e,%e,%d, %e\n", d.from, d.to, t_alone, t_shared, reps, csecond() - bench0);
+    fclose(fp);
+    char out[1024];
+    snprintf(out, sizeof out, "%s/Processed/Link-Stats_loc_dest-%d_loc_src-%d.log", db.c_str(), d.to, d.from);
+    fp = fopen(out, "w");
+    if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+    fprintf(fp, "Intercept: %.12e\nCoefficient: %.12e\n", ti, tb);
+    // the "other link" is the opposite direction: traffic from d.to to d.from
+    fprintf(fp, "Slowdown([%d]->[%d]): %.6f\n", d.to, d.from, t_shared / t_alone);
+    fclose(fp);
+    fprintf(stderr, "link %d<-%d: ti = %.3e s, tb = %.3e s/B (%.1f GB/s), slowdown under opposing traffic %.3f\n", d.to, d.from, ti, tb,
+            1e-9 / tb, t_shared / t_alone);
+  }
+  pl_stream_destroy(s1);
+  pl_stream_destroy(s2);
+  CoCoFree(host, -1); CoCoFree(host2, -1); CoCoFree(dev, 0); CoCoFree(dev2, 0);
+}
+
+int main(int argc, char** argv) {
+  if (argc < 2) {
+    fprintf(stderr, "usage: %s <db_dir> [--quick] [--only gemm|blas1|link]\n", argv[0]);
+    return 2;
+  }
+  const std::string db = argv[1];
+  bool quick = false;
+  std::string only;
+  for (int i = 2; i < argc; ++i) {
+    if (!strcmp(argv[i], "--quick")) quick = true;
+    else if (!strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
+  }
+  try {
+    mkdirs(db);
+    must(pl_set_device(0), "set device");
+    char name[256];
+    must(pl_device_name(0, name, sizeof name), "device name");
+    fprintf(stderr, "paralia_deploy: device 0 = %s, database -> %s%s\n", name, db.c_str(), quick ? " (quick sweep)" : "");
+    const char* q_env = getenv("PARALIA_EXEC_QUEUES");
+    const int queues = (q_env && atoi(q_env) > 0) ? std::min(atoi(q_env), 8) : 2;
+    if (only.empty() || only == "link") bench_link(db, quick);
+    if (only.empty() || only == "gemm") {
+      bench_gemm<double>(db, "Dgemm", quick, queues);
+      bench_gemm<float>(db, "Sgemm", quick, queues);
+    }
+    if (only.empty() || only == "blas1") {
+      bench_blas1(db, "Daxpy", quick);
+      bench_blas1(db, "Ddot", quick);
+    }
+  } catch (const paralia_error& e) {
+    fprintf(stderr, "ERROR -> %s\n", e.what());
+    return 1;
+  }
+  return 0;
+}

@@ -148,13 +148,19 @@ template <typename T> void CoCoVecInit(T* vec, long long length, int seed, short
 template void CoCoVecInit<double>(double*, long long, int, short);
 template void CoCoVecInit<float>(float*, long long, int, short);
 
+// Matching decimal digits of the worst element.  The difference of element i is taken relative to
+// max(|ref_i|, |x_i|, rms(ref)): an element that is small only because its terms cancelled is judged on the scale
+// of the vector, not on its own.
 template <typename T> static short test_equality(T* ref, T* x, long long n, int cap) {
+  long double ss = 0;
+  for (long long i = 0; i < n; ++i) ss += (long double)ref[i] * ref[i];
+  const double rms = n > 0 ? (double)sqrtl(ss / n) : 0.0;
   int worst = cap;
   for (long long i = 0; i < n; ++i) {
     const double d = fabs((double)ref[i] - (double)x[i]);
     if (d == 0) continue;
     if (std::isnan(d)) return 0;
-    const double scale = fmax(fabs((double)ref[i]), fabs((double)x[i]));
+    const double scale = fmax(fmax(fabs((double)ref[i]), fabs((double)x[i])), rms);
     int digits = (int)floor(-log10(d / scale));
     if (digits < 0) digits = 0;
     if (digits < worst) worst = digits;
