@@ -47,6 +47,9 @@ def main():
     ap.add_argument("--size", type=int, default=16384, help="M = N = K (default: the benchmark configuration)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-host", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="launch one daxpy (N=2^28: 4 GiB read, 2 GiB written) and one tile GEMM of --size, nothing else; "
+                         "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives one GPU; run with --gpus 1 (multi-GPU sharding is a design note only)")
@@ -71,6 +74,18 @@ def main():
         e = C.c_void_p()
         pkg.check(L.pl_event_create(C.byref(e), 1), "event")
         return e
+
+    if args.pmc_probe:
+        m = 1 << 28
+        dx, dy, dz = (Buf(pkg, max(m, n * n), np.float64, 0) for _ in range(3))
+        for b, seed in ((dx, 0), (dy, 1)):
+            pkg.check(L.PARALiA_vec_init_f64(b.ptr, b.n, seed, 0), "vec init")
+        pkg.check(L.pl_daxpy(m, 0.7, dx.ptr, 1, dz.ptr, 1, None), "daxpy")
+        pkg.check(L.pl_device_sync(), "sync")
+        pkg.check(L.pl_dgemm_tile(b"N", b"N", n, n, n, 1.0, dx.ptr, n, dy.ptr, n, 0.0, dz.ptr, n, None), "tile")
+        pkg.check(L.pl_device_sync(), "sync")
+        print(json.dumps({"pmc_probe": True, "daxpy_n": m, "gemm_n": n}))
+        return
 
     # ------------------------------------------------------------------ inputs (seeded, uniform [-1, 1))
     hA, hB, hC = (Buf(pkg, n * n, np.float64, -1) for _ in range(3))

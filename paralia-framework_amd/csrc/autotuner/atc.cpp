@@ -259,6 +259,10 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   const Modeler* m = atc->unit_modeler_list[0];
   paralia::StageTimes st;
   st.t_exec = m->exec->predict(T, d.TransA, d.TransB);
+  for (long i = 0; i < m->exec->lines(); ++i)
+    if (m->exec->TransA.empty() || (m->exec->TransA[i] == d.TransA && m->exec->TransB[i] == d.TransB))
+      if (st.exec_table.empty() || st.exec_table.back().first < m->exec->T[i])
+        st.exec_table.emplace_back(m->exec->T[i], m->exec->av_time[i]);
   const comm_data* h2d = m->link[idxize(-1)];
   const comm_data* d2h = m->revlink[idxize(-1)];
   st.h2d_ti = h2d->ti; st.h2d_tb = h2d->tb;
@@ -335,7 +339,15 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         try {
           paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
         } catch (const std::runtime_error&) { continue; }
-        if (r.t_total < best_t) { best_t = r.t_total; best_T = cand; }
+        // predictions of neighbouring T differ by less than the model's accuracy: the reference's penalty terms
+        // (ragged edges, too few or too many subkernels, Autotuner.cpp:571-603) break such near-ties
+        double score = r.t_total;
+        if (cand <= min_dim) {
+          double sl[6];
+          get_T_slowdowns(sl, (int)cand);
+          score *= 1.0 + 0.02 * sl[0];
+        }
+        if (score < best_t) { best_t = score; best_T = cand; }
       }
       if (best_T < 0) {
         // C narrower than every benchmarked tile: one tile across the short side, as square as that allows

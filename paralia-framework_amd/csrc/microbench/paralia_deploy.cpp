@@ -8,15 +8,17 @@
 // tables the autotuner reads to <db_dir>/Processed.
 //
 // What it re-does from the reference: Database_builder/CuCuBLAS/src/dgemm_microbench.cu:26-230 (T sweep from
-// 256 in steps of 256, the step doubling once T >= 16*step, up to < 10000; alpha = 1.1234, beta = 1.2345;
+// 256 in steps of 256, the step doubling once T >= 16*step, up to < 10000; alpha = 1.1234;
 // stop when the 95% confidence half-width is within 5% of the mean and more than 10 samples were taken),
 // daxpy_microbench.cu / ddot_microbench.cu (sweep from 4096 in steps of 4096 with the same doubling),
 // transfer_link_microbench.cu:24-218 (square tiles with a host leading dimension of maxDim + 1, then the
 // overlap run), Python-DataManage/BenchToLookupTables.py.in:31-55 (flag columns prepended, sorted by T) and
 // LinkPreprocessing.py.in:44-61 (least-squares line bytes -> seconds, |intercept|, slowdown ratios).
 // File formats are unchanged so the tables are interchangeable with the reference's.
-// Kernel times are taken the way the scheduler runs the kernels: launches round-robin over its compute
-// streams, time per launch = wall time of a batch / launches in it.
+// Kernel times are taken the way the scheduler runs the kernels: dense tiles (leading dimension = T, as in the
+// device block pool), beta = 1 (every K-step but the first accumulates), launches round-robin over its compute
+// streams, time per launch = wall time of a batch / launches in it.  (The reference benchmarks with the leading
+// dimension of the largest size and beta = 1.2345.)
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -102,7 +104,7 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
     for (long t : Ts) if (t == 512 || t == 1024 || t == 2048 || t == 3072 || t == 4096) few.push_back(t);
     Ts = few;
   }
-  const long ld = maxDim;
+  const long ld = maxDim;  // allocation edge; every measured tile is dense (its own T as leading dimension)
   T *A, *B, *C;
   A = (T*)CoCoMalloc(ld * ld * sizeof(T), 0, 0);
   B = (T*)CoCoMalloc(ld * ld * sizeof(T), 0, 0);
@@ -112,7 +114,7 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
   CoCoVecInit(C, 2 * ld * ld, 44, 0);
   std::vector<void*> st(queues);
   for (auto& s : st) must(pl_stream_create(&s), "stream");
-  const T alpha = (T)1.1234, beta = (T)1.2345;
+  const T alpha = (T)1.1234, beta = (T)1;
   std::vector<Row> rows;
   const char flags[2] = {'N', 'T'};
   for (char ta : flags)
@@ -124,11 +126,12 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
       for (long Tt : Ts) {
         auto launch = [&](int q) {
           if (sizeof(T) == 8)
-            must(pl_dgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const double*)A, ld, (const double*)B, ld, beta, (double*)(C + (long)q * ld * ld), ld, st[q]), "gemm");
+            must(pl_dgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const double*)A, Tt, (const double*)B, Tt, beta, (double*)(C + (long)q * ld * ld), Tt, st[q]), "gemm");
           else
-            must(pl_sgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const float*)A, ld, (const float*)B, ld, beta, (float*)(C + (long)q * ld * ld), ld, st[q]), "gemm");
+            must(pl_sgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const float*)A, Tt, (const float*)B, Tt, beta, (float*)(C + (long)q * ld * ld), Tt, st[q]), "gemm");
         };
-        const int batch = 2 * queues;
+        // long enough that the ramp at both ends of a batch does not weigh on the steady-state rate
+        const int batch = (Tt <= 2048 ? 16 : Tt <= 4096 ? 6 : 2) * queues;
         auto run = [&]() {
           const double t0 = csecond();
           for (int i = 0; i < batch; ++i) launch(i % queues);

@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <climits>
+#include <cmath>
 #include <deque>
 #include <stdexcept>
 #include <string>
@@ -263,9 +264,25 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
   return plan;
 }
 
+double StageTimes::exec_time(long T, long m, long n, long k) const {
+  const double vol = (double)m * n * (double)(k > 0 ? k : 1);
+  const double T3 = (double)T * T * T;
+  if (exec_table.empty() || vol >= T3) return t_exec * vol / T3;
+  // seconds per unit volume at the cube of equal volume, interpolated between the neighbouring table entries
+  const double edge = std::cbrt(vol);
+  auto rate = [](const std::pair<long, double>& e) { return e.second / ((double)e.first * e.first * e.first); };
+  if (edge <= exec_table.front().first) return rate(exec_table.front()) * vol * (exec_table.front().first / edge);
+  for (size_t i = 1; i < exec_table.size(); ++i)
+    if (edge <= exec_table[i].first) {
+      const double f = (edge - exec_table[i - 1].first) / (double)(exec_table[i].first - exec_table[i - 1].first);
+      return ((1 - f) * rate(exec_table[i - 1]) + f * rate(exec_table[i])) * vol;
+    }
+  return rate(exec_table.back()) * vol;
+}
+
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
   const GemmProblem& p = plan.p;
-  const double T2 = (double)p.T * p.T, T3 = T2 * p.T;
+  const double T2 = (double)p.T * p.T;
   std::vector<double> finish(plan.cmds.size(), 0.0);
   double h2d = 0, d2h = 0, exec = 0;
   double qclock[MAX_EXEC_QUEUES] = {0};
@@ -279,7 +296,7 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
       case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
       case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
       case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
-      case CMD_GEMM: dur = st.t_exec * ((double)p.tm(c.mi) * p.tn(c.ni) * std::max(1L, p.tk(c.ki))) / T3; break;
+      case CMD_GEMM: dur = st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(c.ki)); break;
       case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
       case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
     }

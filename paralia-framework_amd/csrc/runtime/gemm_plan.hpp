@@ -12,6 +12,7 @@
 #ifndef PARALIA_GEMM_PLAN_HPP
 #define PARALIA_GEMM_PLAN_HPP
 
+#include <utility>
 #include <vector>
 
 namespace paralia {
@@ -79,6 +80,10 @@ long gemm_full_block_num(const GemmProblem& p);
 // Stage costs of a full T x T (x T) tile; edge tiles scale with their area / volume.
 struct StageTimes {
   double t_exec = 0;                 // one T^3 subkernel
+  // Optional lookup (cube edge, seconds) sorted by edge: an m x n x k subkernel is priced at the flop rate of the
+  // cube of equal volume, so ragged edge tiles cost their (lower) small-kernel rate instead of a pro-rata share.
+  std::vector<std::pair<long, double>> exec_table;
+  double exec_time(long T, long m, long n, long k) const;
   double h2d_ti = 0, h2d_tb = 0;     // seconds, seconds per byte
   double d2h_ti = 0, d2h_tb = 0;
   double t_reduce = 0;               // one T^2 scale-add
