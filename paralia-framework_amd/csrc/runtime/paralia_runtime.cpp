@@ -61,9 +61,13 @@ struct Resources {
   double* dot_ws = nullptr;      // ddot partials
   double* dot_result = nullptr;  // device scalar
   double* dot_host = nullptr;    // pinned scalar
+  // HIP deals streams round-robin onto a few hardware queues (4 by default): streams created back to back land
+  // on different ones.  The copy streams and the default pair of compute streams are therefore created together on
+  // first use; a compute stream that shared a hardware queue with a copy stream would serialise behind the copies.
   void ensure_streams(int nq) {
     if (!h2d) chk(pl_stream_create(&h2d), "stream create");
     if (!d2h) chk(pl_stream_create(&d2h), "stream create");
+    nq = std::max(nq, 2);
     for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
   }
   void ensure_events(size_t n) {

@@ -112,15 +112,19 @@ def test_autotune_selectors(L, pkg, monkeypatch):
     assert info.T in (512, 1024, 2048, 4096)
     assert info.subkernel_num == (8192 // info.T) ** 3
     assert info.pred_t > 0 and info.pipe_exec <= info.pred_t * 1.0000001
-    # the pick is the argmin of the simulated pipeline over the table
+    # the pick is the argmin over the table of the simulated pipeline time, near-ties broken by the reference's
+    # penalty terms: score = pred_t * (1 + 0.02 * T_aggregate_sl)
     best = None
     for T in (512, 1024, 2048, 4096):
         one = pkg.atc_info()
         assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, T, 0, C.byref(one)) == 0
         assert one.selected_by == b"user" and one.T == T
-        if best is None or one.pred_t < best[1]:
-            best = (T, one.pred_t)
-    assert best[0] == info.T and abs(best[1] - info.pred_t) < 1e-12
+        sl = (C.c_double * 6)()
+        assert L.PARALiA_T_slowdowns(8192, 8192, 8192, T, sl) == 0
+        score = one.pred_t * (1.0 + 0.02 * sl[0])
+        if best is None or score < best[1]:
+            best = (T, score, one.pred_t)
+    assert best[0] == info.T and abs(best[2] - info.pred_t) < 1e-12
     # reference model-driven search (data-reuse model)
     monkeypatch.setenv("PARALIA_T_SELECT", "reuse")
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
