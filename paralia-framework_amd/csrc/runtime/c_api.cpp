@@ -18,6 +18,7 @@ ATC_p ddot_impl(long, double*, long, double*, long, double*, ATC_p);
 void cache_free_impl(short);
 void runtime_stats(long*, long*, long long*, long*);
 void runtime_reset();
+void stream_rotation(int*, int*);
 }  // namespace paralia
 paralia::StageTimes paralia_stage_times(const ATC* atc, long T);
 
@@ -105,6 +106,9 @@ int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_byte
 }
 int PARALiA_runtime_reset(void) {
   return guarded([&] { paralia::runtime_reset(); });
+}
+int PARALiA_stream_rotation(int* rotation, int* settled) {
+  return guarded([&] { paralia::stream_rotation(rotation, settled); });
 }
 int PARALiA_set_db_dir(const char* dir) {
   paralia_set_db_dir(dir);

@@ -61,14 +61,52 @@ struct Resources {
   double* dot_ws = nullptr;      // ddot partials
   double* dot_result = nullptr;  // device scalar
   double* dot_host = nullptr;    // pinned scalar
-  // HIP deals streams round-robin onto a few hardware queues (4 by default): streams created back to back land
-  // on different ones.  The copy streams and the default pair of compute streams are therefore created together on
-  // first use; a compute stream that shared a hardware queue with a copy stream would serialise behind the copies.
+  // HIP deals the streams of a process round-robin onto GPU_MAX_HW_QUEUES hardware queues (4 by default), in
+  // creation order and counting the default stream.  With 4 queues the four streams this scheduler keeps busy
+  // always sit on four different queues, yet which stream sits on which queue matters: of the four alignments
+  // one runs the streamed 16384^3 fp64 GEMM in 130 ms, the others in 148-169 ms.  The alignment depends on how
+  // many streams the application created before this library did, which cannot be queried.  So seven streams
+  // are created back to back, "rotation" r uses streams r .. r+3 as (H2D, D2H, compute 0, compute 1), and
+  // the first four large streamed GEMM calls each run under a different rotation; the fastest is kept
+  // (PARALIA_STREAM_ROTATION=r skips the trial).  With 8 or more hardware queues all rotations are equal.
+  void* ring[7] = {nullptr};
+  int rotation = 0;
+  int trials = 0;            // rotations tried so far; 4 = settled
+  double trial_rate[4] = {0, 0, 0, 0};
+  void set_rotation(int r) {
+    rotation = r;
+    h2d = ring[r];
+    d2h = ring[r + 1];
+    exec[0] = ring[r + 2];
+    exec[1] = ring[r + 3];
+  }
   void ensure_streams(int nq) {
-    if (!h2d) chk(pl_stream_create(&h2d), "stream create");
-    if (!d2h) chk(pl_stream_create(&d2h), "stream create");
-    nq = std::max(nq, 2);
+    if (!ring[0]) {
+      for (void*& s : ring) chk(pl_stream_create(&s), "stream create");
+      nexec = 2;
+      const char* env = getenv("PARALIA_STREAM_ROTATION");
+      if (env && atoi(env) >= 0 && atoi(env) < 4) {
+        set_rotation(atoi(env));
+        trials = 4;
+      } else {
+        set_rotation(0);
+      }
+    }
     for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
+  }
+  // Called around a large streamed GEMM: picks the rotation to try, then records seconds per flop.
+  void begin_trial() {
+    if (trials < 4) set_rotation(trials);
+  }
+  void end_trial(double seconds_per_flop) {
+    if (trials >= 4) return;
+    trial_rate[trials++] = seconds_per_flop;
+    if (trials == 4) {
+      int best = 0;
+      for (int r = 1; r < 4; ++r)
+        if (trial_rate[r] < trial_rate[best]) best = r;
+      set_rotation(best);
+    }
   }
   void ensure_events(size_t n) {
     while (events.size() < n) {
@@ -93,9 +131,8 @@ struct Resources {
     if (d2h) chk(pl_stream_sync(d2h), "stream sync");
   }
   void destroy() {
-    if (h2d) pl_stream_destroy(h2d);
-    if (d2h) pl_stream_destroy(d2h);
-    for (int q = 0; q < nexec; ++q) pl_stream_destroy(exec[q]);
+    for (void* s : ring) if (s) pl_stream_destroy(s);
+    for (int q = 2; q < nexec; ++q) pl_stream_destroy(exec[q]);
     for (void* e : events) pl_event_destroy(e);
     if (dot_ws) pl_free_device(dot_ws);
     if (dot_host) pl_free_pinned(dot_host);
@@ -347,7 +384,12 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   } else {
     const GemmPlan& plan = entry->plan;
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T));
+    R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
+    const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab;
+    if (trial) R.res.begin_trial();
+    const double t0 = csecond();
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC);
+    if (trial) R.res.end_trial((csecond() - t0) / (2.0 * M * N * (double)K));
   }
   return atc_copy(atc);
 }
@@ -533,6 +575,13 @@ void runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long
   if (pmd_misses) *pmd_misses = R.pmd_misses;
   if (pool_bytes) *pool_bytes = R.pool.bytes();
   if (pmd_entries) *pmd_entries = (long)R.pmd.size();
+}
+
+void stream_rotation(int* rotation, int* settled) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  if (rotation) *rotation = R.res.rotation;
+  if (settled) *settled = R.res.trials >= 4 ? 1 : 0;
 }
 
 void runtime_reset() {
