@@ -163,9 +163,13 @@ int PARALiA_autotune(const char* db_dir, const char* func, long D1, long D2, lon
 #define PL_PLAN_ROW (10 + PL_PLAN_MAX_WAITS)
 long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
                        int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]);
+/* makespan of one order (order_id >= 0) or of the best candidate (< 0) on the simulated H2D / compute / D2H pipeline;
+   h2d_sl, d2h_sl >= 1: how much slower a copy runs while the opposite direction is busy (the link model's sl,
+   CoModel.cpp:143-162) */
 double PARALiA_gemm_plan_simulate(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero,
                                   int elem, int exec_queues, long pool_blocks, int order_id, double t_exec, double h2d_ti,
-                                  double h2d_tb, double d2h_ti, double d2h_tb, double t_reduce, int* picked, double busy[3]);
+                                  double h2d_tb, double d2h_ti, double d2h_tb, double t_reduce, double h2d_sl, double d2h_sl, int* picked,
+                                  double busy[3]);
 
 #ifdef __cplusplus
 }

@@ -87,7 +87,7 @@ _SIGS = {
     "PARALiA_model_predict": (_d, [C.c_char_p, C.c_char_p, _i, _l, _l, _l, _c, _c, _pi, _l]),
     "PARALiA_autotune": (_i, [C.c_char_p, C.c_char_p, _l, _l, _l, _c, _c, _pi, _i, _l, _ll, C.POINTER(atc_info)]),
     "PARALiA_gemm_plan": (_l, [_l, _l, _l, _l, _i, _i, _i, _i, _i, _i, _l, _i, _pi, _l, C.POINTER(_l)]),
-    "PARALiA_gemm_plan_simulate": (_d, [_l, _l, _l, _l, _i, _i, _i, _i, _i, _i, _l, _i, _d, _d, _d, _d, _d, _d, _pi,
+    "PARALiA_gemm_plan_simulate": (_d, [_l, _l, _l, _l, _i, _i, _i, _i, _i, _i, _l, _i, _d, _d, _d, _d, _d, _d, _d, _d, _pi,
                                         C.POINTER(_d)]),
 }
 

@@ -267,6 +267,7 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   const comm_data* d2h = m->revlink[idxize(-1)];
   st.h2d_ti = h2d->ti; st.h2d_tb = h2d->tb;
   st.d2h_ti = d2h->ti; st.d2h_tb = d2h->tb;
+  st.h2d_sl = std::max(1.0, h2d->sl); st.d2h_sl = std::max(1.0, d2h->sl);
   st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
   return st;
 }

@@ -235,12 +235,14 @@ long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remot
 // Simulated makespan of one order (order_id >= 0) or of the best candidate (order_id < 0; *picked receives it).
 double PARALiA_gemm_plan_simulate(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero,
                                   int elem, int exec_queues, long pool_blocks, int order_id, double t_exec, double h2d_ti,
-                                  double h2d_tb, double d2h_ti, double d2h_tb, double t_reduce, int* picked, double busy[3]) {
+                                  double h2d_tb, double d2h_ti, double d2h_tb, double t_reduce, double h2d_sl, double d2h_sl, int* picked,
+                                  double busy[3]) {
   double out = -1;
   guarded([&] {
     paralia::GemmProblem gp = gp_of(M, N, K, T, a_remote, b_remote, c_remote, beta_zero, elem, exec_queues, pool_blocks);
     paralia::StageTimes st;
     st.t_exec = t_exec; st.h2d_ti = h2d_ti; st.h2d_tb = h2d_tb; st.d2h_ti = d2h_ti; st.d2h_tb = d2h_tb; st.t_reduce = t_reduce;
+    st.h2d_sl = h2d_sl; st.d2h_sl = d2h_sl;
     paralia::PipelineResult r;
     if (order_id >= 0) {
       r = paralia::simulate_plan(paralia::build_gemm_plan(gp, order_id), st);

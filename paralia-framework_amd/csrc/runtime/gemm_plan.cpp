@@ -280,42 +280,92 @@ double StageTimes::exec_time(long T, long m, long n, long k) const {
   return rate(exec_table.back()) * vol;
 }
 
+namespace {
+
+using Intervals = std::vector<std::pair<double, double>>;
+
+// Completion time of a copy that needs `work` seconds on an otherwise idle link and starts at s, when it runs sl
+// times slower while the opposite direction is busy.  `busy` is sorted and disjoint; `cursor` only moves forward
+// because the copies of one direction start in non-decreasing time order.
+double stretched_end(double s, double work, double sl, const Intervals& busy, size_t& cursor) {
+  if (sl <= 1.0 || busy.empty()) return s + work;
+  while (cursor < busy.size() && busy[cursor].second <= s) ++cursor;
+  double t = s;
+  for (size_t c = cursor; work > 0; ++c) {
+    if (c >= busy.size()) return t + work;
+    if (t < busy[c].first) {
+      const double idle = busy[c].first - t;
+      if (work <= idle) return t + work;
+      work -= idle;
+      t = busy[c].first;
+    }
+    const double span = busy[c].second - t;
+    if (work * sl <= span) return t + work * sl;
+    work -= span / sl;
+    t = busy[c].second;
+  }
+  return t;
+}
+
+void add_interval(Intervals& v, double a, double b) {
+  if (b <= a) return;
+  if (!v.empty() && a <= v.back().second) v.back().second = std::max(v.back().second, b);
+  else v.emplace_back(a, b);
+}
+
+}  // namespace
+
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
   const GemmProblem& p = plan.p;
   const double T2 = (double)p.T * p.T;
   std::vector<double> finish(plan.cmds.size(), 0.0);
-  double h2d = 0, d2h = 0, exec = 0;
-  double qclock[MAX_EXEC_QUEUES] = {0};
+  // The two copy directions share the host link: a copy is slower while the opposite direction is busy
+  // (the sl factor of the link model, CoModel.cpp:143-162).  The commands are walked in plan order, not in time
+  // order, so the opposite direction's busy intervals are taken from the previous pass; the first pass runs
+  // without slowdown and two more settle the schedule.
+  const bool contended = st.h2d_sl > 1.0 || st.d2h_sl > 1.0;
+  Intervals busy_h2d, busy_d2h;
   PipelineResult r;
-  for (size_t i = 0; i < plan.cmds.size(); ++i) {
-    const Cmd& c = plan.cmds[i];
-    double ready = 0;
-    for (int w = 0; w < c.nwait; ++w) ready = std::max(ready, finish[c.wait[w]]);
-    double dur = 0;
-    switch (c.kind) {
-      case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
-      case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
-      case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
-      case CMD_GEMM: dur = st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(c.ki)); break;
-      case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
-      case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+  for (int pass = 0; pass < (contended ? 3 : 1); ++pass) {
+    Intervals now_h2d, now_d2h;
+    size_t cur_h2d = 0, cur_d2h = 0;
+    double h2d = 0, d2h = 0, exec = 0;
+    double qclock[MAX_EXEC_QUEUES] = {0};
+    r = PipelineResult();
+    for (size_t i = 0; i < plan.cmds.size(); ++i) {
+      const Cmd& c = plan.cmds[i];
+      double ready = 0;
+      for (int w = 0; w < c.nwait; ++w) ready = std::max(ready, finish[c.wait[w]]);
+      double dur = 0;
+      switch (c.kind) {
+        case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
+        case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
+        case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+        case CMD_GEMM: dur = st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(c.ki)); break;
+        case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
+        case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+      }
+      if (c.stream == STREAM_H2D) {
+        const double s = std::max(ready, h2d);
+        finish[i] = h2d = stretched_end(s, dur, st.h2d_sl, busy_d2h, cur_d2h);
+        add_interval(now_h2d, s, h2d);
+        r.t_h2d += h2d - s;
+      } else if (c.stream == STREAM_D2H) {
+        const double s = std::max(ready, d2h);
+        finish[i] = d2h = stretched_end(s, dur, st.d2h_sl, busy_h2d, cur_h2d);
+        add_interval(now_d2h, s, d2h);
+        r.t_d2h += d2h - s;
+      } else {
+        // exec queues are in-order each and share the one compute resource
+        const int q = c.stream - STREAM_EXEC0;
+        const double s = std::max(std::max(ready, qclock[q]), exec);
+        finish[i] = qclock[q] = exec = s + dur;
+        r.t_exec += dur;
+      }
+      r.t_total = std::max(r.t_total, finish[i]);
     }
-    if (c.stream == STREAM_H2D) {
-      const double s = std::max(ready, h2d);
-      finish[i] = h2d = s + dur;
-      r.t_h2d += dur;
-    } else if (c.stream == STREAM_D2H) {
-      const double s = std::max(ready, d2h);
-      finish[i] = d2h = s + dur;
-      r.t_d2h += dur;
-    } else {
-      // exec queues are in-order each and share the one compute resource
-      const int q = c.stream - STREAM_EXEC0;
-      const double s = std::max(std::max(ready, qclock[q]), exec);
-      finish[i] = qclock[q] = exec = s + dur;
-      r.t_exec += dur;
-    }
-    r.t_total = std::max(r.t_total, finish[i]);
+    busy_h2d.swap(now_h2d);
+    busy_d2h.swap(now_d2h);
   }
   return r;
 }

@@ -86,6 +86,7 @@ struct StageTimes {
   double exec_time(long T, long m, long n, long k) const;
   double h2d_ti = 0, h2d_tb = 0;     // seconds, seconds per byte
   double d2h_ti = 0, d2h_tb = 0;
+  double h2d_sl = 1, d2h_sl = 1;     // how much slower a copy runs while the opposite direction is busy (>= 1)
   double t_reduce = 0;               // one T^2 scale-add
 };
 struct PipelineResult {

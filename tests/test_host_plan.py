@@ -192,7 +192,7 @@ def test_pipeline_simulation(pkg, L):
     # 77 ms of H2D, 38 ms of D2H); a good order hides nearly all transfers, the reference index order cannot hide
     # the fetch of a whole K-chain per C tile at the start, pure k-outer leaves every write-back to the end.
     args = (16384, 16384, 16384, 2048, 1, 1, 1, 1, 8, 2, 0)
-    st = (0.24e-3, 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.02e-3)
+    st = (0.24e-3, 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.02e-3, 1.0, 1.0)
     best = L.PARALiA_gemm_plan_simulate(*args, -1, *st, C.byref(picked), busy)
     assert abs(busy[1] - 512 * 0.24e-3) < 1e-9 and abs(busy[0] - 128 * 0.6e-3) < 1e-9 and abs(busy[2] - 64 * 0.6e-3) < 1e-9
     assert best >= busy[1] and best < busy[1] * 1.04
@@ -206,3 +206,28 @@ def test_pipeline_simulation(pkg, L):
     args5 = (40000, 40000, 2048, 2048, 1, 1, 1, 0, 8, 2, 0)
     t5 = L.PARALiA_gemm_plan_simulate(*args5, -1, *st, C.byref(picked), busy)
     assert busy[0] > busy[1] and t5 >= busy[0] and t5 < busy[0] * 1.05
+
+
+def test_pipeline_simulation_link_contention(pkg, L):
+    """Copies in opposite directions slow each other by the link model's sl factors.  Checked on cases whose answer
+    is known without running the simulator's own arithmetic: (1) sl = 1 changes nothing; (2) a D2H slowdown alone can
+    only lengthen the makespan and the D2H busy time, never the H2D busy time; (3) in the transfer-bound 40000 x 40000
+    x 2048 case the D2H stream is busy nearly the whole time, so the H2D busy time must land between the undisturbed
+    time and sl times it, and close to sl times it."""
+    import ctypes as C
+    busy0, busy1 = (C.c_double * 3)(), (C.c_double * 3)()
+    tb = 0.6e-3 / (2048 * 2048 * 8)
+    args5 = (40000, 40000, 2048, 2048, 1, 1, 1, 0, 8, 2, 0)
+    base = (0.24e-3, 0.0, tb, 0.0, tb, 0.02e-3)
+    t0 = L.PARALiA_gemm_plan_simulate(*args5, 10000, *base, 1.0, 1.0, None, busy0)
+    t_d = L.PARALiA_gemm_plan_simulate(*args5, 10000, *base, 1.0, 1.3, None, busy1)
+    assert t_d >= t0 and busy1[2] > busy0[2] * 1.05 and abs(busy1[0] - busy0[0]) < 1e-12
+    t_h = L.PARALiA_gemm_plan_simulate(*args5, 10000, *base, 1.2, 1.0, None, busy1)
+    assert busy0[0] * 1.12 < busy1[0] <= busy0[0] * 1.2 + 1e-9
+    assert t_h >= busy1[0] and t_h > t0 * 1.1
+    assert abs(busy1[2] - busy0[2]) < 1e-12
+    # compute-bound 16384^3 with beta = 0: transfers hide behind the kernels either way, the makespan barely moves
+    args3 = (16384, 16384, 16384, 2048, 1, 1, 1, 1, 8, 2, 0)
+    a = L.PARALiA_gemm_plan_simulate(*args3, 4, *base, 1.0, 1.0, None, None)
+    b = L.PARALiA_gemm_plan_simulate(*args3, 4, *base, 1.2, 1.2, None, None)
+    assert a <= b < a * 1.03
