@@ -1,0 +1,150 @@
+"""The benchmark configurations at their full sizes, through the C ABI.  A full CPU product would take minutes, so the
+GEMMs are checked with a size-independent identity evaluated in O(n^2) on the CPU,
+    (alpha*op(A)*op(B) + beta*C0) v  =  alpha*op(A)*(op(B)*v) + beta*(C0*v)      for a seeded random v,
+(one wrong tile, a dropped K step or a wrong beta on any tile moves it by orders of magnitude more than the tolerance)
+plus random 64 x 64 panels recomputed in long double.  The BLAS-1 cases are compared element by element with numpy."""
+import ctypes as C
+import time
+
+import numpy as np
+import pytest
+
+from gpu_util import Buf
+from oracle_binding import rand_f64
+
+pytestmark = pytest.mark.gpu
+TOL64, TOL32 = 1e-13, 1e-5
+
+
+def filled(pkg, L, n, dtype, seed, loc):
+    b = Buf(pkg, n, dtype, loc)
+    fn = L.PARALiA_vec_init_f64 if np.dtype(dtype) == np.float64 else L.PARALiA_vec_init_f32
+    pkg.check(fn(b.ptr, n, seed, loc), "vec_init")
+    return b
+
+
+def host(b):
+    return b.host_view() if b.loc < 0 else b.get()
+
+
+def colmajor(flat, rows, cols):
+    return flat.reshape(cols, rows).T
+
+
+def matvec64(Mx, v, chunk=4096):
+    """Mx @ v accumulated in fp64 whatever the dtype of Mx, converting one contiguous slab at a time."""
+    if Mx.dtype == np.float64:
+        return Mx @ v
+    out = np.zeros(Mx.shape[0])
+    if Mx.flags.c_contiguous:
+        for i in range(0, Mx.shape[0], chunk):
+            out[i:i + chunk] = Mx[i:i + chunk, :].astype(np.float64) @ v
+    else:
+        for j in range(0, Mx.shape[1], chunk):
+            out += Mx[:, j:j + chunk].astype(np.float64) @ v[j:j + chunk]
+    return out
+
+
+def fro(Mx, chunk=1 << 26):
+    flat = Mx.T.reshape(-1) if Mx.flags.f_contiguous else Mx.reshape(-1)   # views, never copies
+    return float(np.sqrt(sum(float(np.sum(np.square(flat[i:i + chunk], dtype=np.float64))) for i in range(0, flat.size, chunk))))
+
+
+def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL64, panels=3):
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    t0 = time.time()
+    bA, bB, bC = filled(pkg, L, ra * ca, dtype, 42, locs[0]), filled(pkg, L, rb * cb, dtype, 43, locs[1]), filled(pkg, L, M * N, dtype, 44, locs[2])
+    C0 = host(bC).copy() if beta != 0.0 else None
+    info = pkg.atc_info()
+    fn = L.PARALiA_dgemm if np.dtype(dtype) == np.float64 else L.PARALiA_sgemm
+    print(f"full-size gemm {np.dtype(dtype).name} {ta}{tb} {M}x{N}x{K} alpha={alpha} beta={beta} locs={locs} T={T} (init {time.time() - t0:.1f}s)", flush=True)
+    t0 = time.time()
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), bA.ptr, ra, bB.ptr, rb, float(beta), bC.ptr, M, T, 0, C.byref(info)), "gemm")
+    print(f"  first call {1e3 * (time.time() - t0):.1f} ms, T={info.T} ({info.selected_by.decode()}), order {info.order_id}, "
+          f"{info.subkernel_num} subkernels, predicted {1e3 * info.pred_t:.1f} ms", flush=True)
+    got = colmajor(host(bC), M, N)
+    A, B = colmajor(host(bA), ra, ca), colmajor(host(bB), rb, cb)
+    opA = A if ta == "N" else A.T
+    opB = B if tb == "N" else B.T
+    v = rand_f64(N, 7)
+    expect = alpha * matvec64(opA, matvec64(opB, v))
+    nA, nB, nv = fro(A), fro(B), float(np.linalg.norm(v))
+    denom = abs(alpha) * nA * nB * nv
+    if C0 is not None:
+        C0m = colmajor(C0, M, N)
+        expect = expect + beta * matvec64(C0m, v)
+        denom += abs(beta) * fro(C0m) * nv
+    err = float(np.linalg.norm(matvec64(got, v) - expect)) / denom
+    print(f"  checksum identity error {err:.3e}", flush=True)
+    assert err < tol
+    rng = np.random.default_rng(1)
+    for _ in range(panels):
+        i, j = int(rng.integers(0, M - 64)), int(rng.integers(0, N - 64))
+        blk = alpha * (opA[i:i + 64, :].astype(np.longdouble) @ opB[:, j:j + 64].astype(np.longdouble))
+        d = abs(alpha) * float(np.linalg.norm(opA[i:i + 64, :].astype(np.float64))) * float(np.linalg.norm(opB[:, j:j + 64].astype(np.float64)))
+        if C0 is not None:
+            blk = blk + beta * C0m[i:i + 64, j:j + 64].astype(np.longdouble)
+            d += abs(beta) * float(np.linalg.norm(C0m[i:i + 64, j:j + 64].astype(np.float64)))
+        assert float(np.linalg.norm((got[i:i + 64, j:j + 64] - blk).astype(np.float64))) / d < tol
+    for b in (bA, bB, bC):
+        b.free()
+    return info
+
+
+@pytest.mark.timeout(600)
+def test_dgemm_16384_host_operands(pkg, L):
+    """dgemm 16384^3, alpha = 1, beta = 0, all operands in pinned host memory, T picked by the autotuner."""
+    info = check_gemm(pkg, L, np.float64, "N", "N", 16384, 16384, 16384, 1.0, 0.0, (-1, -1, -1))
+    assert info.subkernel_num == (16384 // info.T) ** 3
+
+
+@pytest.mark.timeout(600)
+def test_sgemm_32768_mixed_locations(pkg, L):
+    """sgemm 32768^3, transA = N, transB = T, alpha = beta = 1, A and B in pinned host memory, C on the device."""
+    check_gemm(pkg, L, np.float32, "N", "T", 32768, 32768, 32768, 1.0, 1.0, (-1, -1, 0), tol=TOL32, panels=2)
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("T", [-1, 8192])
+def test_dgemm_40000x40000x2048_read_modify_write(pkg, L, T):
+    """dgemm 40000 x 40000 x 2048, alpha = 1.5, beta = 0.5, everything on the host: ragged last tiles (40000 =
+    19 * 2048 + 1088), C fetched, combined on the device and written back; T = 8192 makes tiles deeper than K."""
+    check_gemm(pkg, L, np.float64, "N", "N", 40000, 40000, 2048, 1.5, 0.5, (-1, -1, -1), T=T, panels=2)
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("loc", [0, -1])
+def test_daxpy_ddot_2p28(pkg, L, orc, openblas, loc):
+    """daxpy and ddot at N = 2^28 (2 GiB per vector), alpha = 0.7, unit strides, both vectors on the device or both in
+    pinned host memory, against OpenBLAS on the same vectors: ddot within 1e-13 * |x| * |y|, daxpy within 1 ulp."""
+    n, alpha = 1 << 28, 0.7
+    bx, by = filled(pkg, L, n, np.float64, 11, loc), filled(pkg, L, n, np.float64, 12, loc)
+    x, y0 = host(bx).copy(), host(by).copy()
+    print(f"full-size daxpy/ddot N=2^28 loc={loc}", flush=True)
+    ref = C.c_double(0.0)
+    assert openblas.orc_openblas_ddot(n, x.ctypes.data, 1, y0.ctypes.data, 1, C.byref(ref)) == 0
+    bound = 1e-13 * float(np.linalg.norm(x)) * float(np.linalg.norm(y0))
+    res = C.c_double(1.25)
+    pkg.check(L.PARALiA_ddot(n, bx.ptr, 1, by.ptr, 1, C.byref(res), -1, None), "ddot")
+    print(f"  ddot {res.value - 1.25!r} vs OpenBLAS {ref.value!r} (bound {bound:.2e})", flush=True)
+    assert abs((res.value - 1.25) - ref.value) <= bound      # the product is added to what *result held
+    m = 1 << 20                                               # a prefix against long double
+    exact = float(np.dot(x[:m].astype(np.longdouble), y0[:m].astype(np.longdouble)))
+    r2 = C.c_double(0.0)
+    pkg.check(L.PARALiA_ddot(m, bx.ptr, 1, by.ptr, 1, C.byref(r2), -1, None), "ddot prefix")
+    assert abs(r2.value - exact) <= 1e-13 * float(np.linalg.norm(x[:m])) * float(np.linalg.norm(y0[:m]))
+    pkg.check(L.PARALiA_daxpy(n, alpha, bx.ptr, 1, by.ptr, 1, -1, None), "daxpy")
+    got = host(by)
+    expect = y0.copy()
+    assert openblas.orc_openblas_daxpy(n, alpha, x.ctypes.data, 1, expect.ctypes.data, 1) == 0
+    worst = int(orc.orc_max_ulp_f64(got.ctypes.data, expect.ctypes.data, n))
+    print(f"  daxpy worst distance from OpenBLAS: {worst} ulp", flush=True)
+    if worst > 1:
+        # OpenBLAS kernels without a fused multiply-add round alpha*x first: then the distance is bounded on the scale
+        # of the larger operand instead (1.5 units: half for alpha*x, half for each final rounding)
+        scale = np.maximum(np.maximum(np.abs(alpha * x), np.abs(y0)), np.maximum(np.abs(got), np.abs(expect)))
+        assert float(np.max(np.abs(got - expect) / np.spacing(scale))) <= 1.5
+    assert np.array_equal(host(bx), x)
+    bx.free()
+    by.free()
