@@ -27,6 +27,12 @@ ATC_p PARALiASgemmControled(char TransA, char TransB, long int M, long int N, lo
                             long int ldA, float* B, long int ldB, float beta, float* C, long int ldC,
                             ATC_p predef_control_values);
 /// y <- alpha * x + y  (daxpy.cpp:200)
+/// y = alpha * op(A) * x + beta * y with A column-major M x N (PARALiA.hpp:48-53 of the reference, dgemv.cpp:288):
+/// x has N elements for TransA = 'N' and M for 'T', y the other count.
+ATC_p PARALiADgemv(char TransA, long int M, long int N, double alpha, double* A, long int ldA, double* x, long int incx,
+                   double beta, double* y, long int incy);
+ATC_p PARALiADgemvControled(char TransA, long int M, long int N, double alpha, double* A, long int ldA, double* x,
+                            long int incx, double beta, double* y, long int incy, ATC_p predef_control_values);
 ATC_p PARALiADaxpy(long int N, double alpha, double* x, long int incx, double* y, long int incy);
 ATC_p PARALiADaxpyControled(long int N, double alpha, double* x, long int incx, double* y, long int incy,
                             ATC_p predef_control_values);
@@ -45,6 +51,10 @@ inline ATC_p PARALiA_dgemm(char TransA, char TransB, long int M, long int N, lon
 inline ATC_p PARALiA_sgemm(char TransA, char TransB, long int M, long int N, long int K, float alpha, float* A,
                            long int ldA, float* B, long int ldB, float beta, float* C, long int ldC) {
   return PARALiASgemm(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC);
+}
+inline ATC_p PARALiA_dgemv(char TransA, long int M, long int N, double alpha, double* A, long int ldA, double* x,
+                           long int incx, double beta, double* y, long int incy) {
+  return PARALiADgemv(TransA, M, N, alpha, A, ldA, x, incx, beta, y, incy);
 }
 inline ATC_p PARALiA_daxpy(long int N, double alpha, double* x, long int incx, double* y, long int incy) {
   return PARALiADaxpy(N, alpha, x, incx, y, incy);

@@ -48,6 +48,7 @@ inline long long gemm_flops(long M, long N, long K) { return (long long)M * K * 
 inline long long gemm_memory(long M, long N, long K, long A_loc, long B_loc, long C_loc, short dsize) {
   return ((long long)M * K * A_loc + (long long)K * N * B_loc + (long long)M * N * C_loc) * dsize;
 }
+inline long long gemv_flops(long M, long N) { return (long long)M * (2 * N + 1); }  // by analogy with gemm_flops (the reference's own is un-vendored)
 inline long long axpy_flops(long N) { return 2LL * N; }
 inline long long dot_flops(long N) { return 2LL * N; }
 

@@ -100,6 +100,15 @@ long pl_ddot_workspace_doubles(void);
 int pl_ddot(long n, const double* x, long incx, const double* y, long incy, double* result, int accumulate,
             double* workspace, void* stream);
 
+/* y <- alpha*op(A)*x + beta*y, A column-major M x N; replaces cublasDgemv on a tile or on a whole device-resident
+ * matrix (gemv_backend_in<double>, dgemv.cpp:41-118).  All pointers are device pointers; workspace holds
+ * pl_dgemv_workspace_doubles(trans, M, N) doubles (partial sums of the reduction chunks; the chunking, and with it the
+ * summation order, depends only on the shape, the parity of M and lda, and the 16-byte alignment of A).  BLAS quick returns: M == 0, N == 0, or alpha == 0 with
+ * beta == 1 leave y untouched; beta == 0 never reads y. */
+long long pl_dgemv_workspace_doubles(char trans, long M, long N);
+int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
+             double* y, long incy, double* workspace, void* stream);
+
 /* ---- routines: plain-C faces of Library_scheduler/include/PARALiA.hpp:33-72 ----
  * Operands may be host (pinned or pageable) or device pointers; the library detects which.  Calls return
  * after the result has reached the caller's buffer.  T > 0 / cache_limit > 0 preset the tile size and the
@@ -129,6 +138,10 @@ int PARALiA_sgemm(char TransA, char TransB, long M, long N, long K, float alpha,
 int PARALiA_daxpy(long N, double alpha, double* x, long incx, double* y, long incy, long T, pl_atc_info* info);
 /* PARALiADdot / PARALiADdotControled (ddot.cpp:201): the dot product is ADDED to *result (ddot.cpp:431) */
 int PARALiA_ddot(long N, double* x, long incx, double* y, long incy, double* result, long T, pl_atc_info* info);
+/* PARALiADgemv / PARALiADgemvControled (dgemv.cpp:288,720, PARALiA.hpp:48-53): y <- alpha*op(A)*x + beta*y; x has N
+ * ('N') or M ('T') elements, y the other count */
+int PARALiA_dgemv(char TransA, long M, long N, double alpha, double* A, long ldA, double* x, long incx, double beta, double* y,
+                  long incy, long T, long long cache_limit, pl_atc_info* info);
 /* PARALiADevCacheFree (Subkernel.cpp:488) */
 int PARALiA_dev_cache_free(int dev_id);
 /* metadata-cache and pool counters (PMD_cache, dgemm.cpp:342-368); reset drops the cached problems */

@@ -259,6 +259,54 @@ long double orc_ddot_longdouble(long n, const double* x, long incx, const double
 #define ORC_TILE_MAX 4096              /* :164 */
 #define ORC_TILE_MAX_SLOWDOWN 0.1      /* :165 */
 
+/* ------------------------------------------------------------------------------------------------ BLAS-2 */
+/* y = alpha*op(A)*x + beta*y, long double accumulation, one rounding per element; BLAS conventions: quick return for
+ * M == 0 or N == 0, beta == 0 never reads y, negative increments walk the vector backwards. */
+void orc_dgemv_bruteforce(char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                          double beta, double* y, long incy) {
+  if (M <= 0 || N <= 0) return;
+  const int t = is_t(ta);
+  const long lx = t ? M : N, ly = t ? N : M;
+  const double* xs = first_c(x, lx, incx);
+  double* ys = first_m(y, ly, incy);
+  for (long i = 0; i < ly; ++i) {
+    long double acc = 0.0L;
+    if (alpha != 0.0) /* BLAS: A and x are not referenced when alpha == 0 */
+      for (long j = 0; j < lx; ++j) acc += (long double)(t ? A[j + i * lda] : A[i + j * lda]) * (long double)xs[j * incx];
+    const long double prev = beta == 0.0 ? 0.0L : (long double)beta * (long double)ys[i * incy];
+    ys[i * incy] = (double)((long double)alpha * acc + prev);
+  }
+}
+
+/* The reference's schedule (dgemv.cpp:41-118, 121-126): A cut into T x T tiles, subkernel mi*Ng + ni multiplies the x
+ * tile of its reduction index into the y tile of its output index, the first subkernel of a y tile applies the
+ * caller's beta and later ones accumulate with beta = 1.  Each tile product is an ordinary double-precision gemv
+ * (fma accumulation in index order), as one cublasDgemv call per tile would be.  Returns the number of subkernels. */
+long orc_dgemv_tiled(long T, char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                     double beta, double* y, long incy) {
+  if (M <= 0 || N <= 0 || T <= 0) return 0;
+  const int t = is_t(ta);
+  const long lx = t ? M : N, ly = t ? N : M;
+  const double* xs = first_c(x, lx, incx);
+  double* ys = first_m(y, ly, incy);
+  const long Mg = (M + T - 1) / T, Ng = (N + T - 1) / T;
+  for (long mi = 0; mi < Mg; ++mi)
+    for (long ni = 0; ni < Ng; ++ni) {
+      const long tm = mi == Mg - 1 ? M - mi * T : T, tn = ni == Ng - 1 ? N - ni * T : T;
+      const double* At = A + mi * T + ni * T * lda;
+      const long xi = t ? mi : ni, yi = t ? ni : mi, xl = t ? tm : tn, yl = t ? tn : tm;
+      const int first = (t ? mi : ni) == 0;
+      const double b = first ? beta : 1.0;
+      for (long i = 0; i < yl; ++i) {
+        double acc = 0.0;
+        for (long j = 0; j < xl; ++j) acc = fma(t ? At[j + i * lda] : At[i + j * lda], xs[(xi * T + j) * incx], acc);
+        double* yp = ys + (yi * T + i) * incy;
+        *yp = b == 0.0 ? alpha * acc : fma(alpha, acc, b * *yp);
+      }
+    }
+  return Mg * Ng;
+}
+
 static long cdiv(long a, long b) { return a / b + ((a % b) ? 1 : 0); }
 
 long orc_sk_num_blas3(long D1, long D2, long D3, long T) { return cdiv(D1, T) * cdiv(D2, T) * cdiv(D3, T); }
@@ -459,6 +507,39 @@ double orc_predict_blas1_bidirectional(const orc_problem* p, int numT, const int
   return fmax(t_exec, t_over) * ker_over + fmax(t_exec, numTout * t_send) + numTin * t_recv + numTout * t_send;
 }
 
+double orc_predict_blas2(int mode, const orc_problem* p, long T) {
+  /* ModelLvl2.cpp:89-132 (full overlap), :133-176 (zero overlap), :194-259 (bidirectional).  Operand sizes as the
+   * reference declares them (CoCoModel_gemv_init, :66-71): A is D1 x D2, x D1 x 1, y D2 x 1; in = {1,1,1}, out = {0,0,1}.
+   * The bidirectional model prices one tile transfer as T elements and overlaps D1/T - 1 kernels. */
+  static const int in[3] = {1, 1, 1}, out[3] = {0, 0, 1};
+  const orc_link local = {0.0, 0.0, 1.0};
+  if (mode == ORC_FULL_OVERLAP || mode == ORC_NO_OVERLAP) {
+    long maxT = p->exec->T[0];
+    for (int i = 0; i < p->exec->lines; ++i) if (p->exec->T[i] > maxT) maxT = p->exec->T[i];
+    const long Tbig = orc_exec_nearest_T(p->exec, (long)fmin((double)maxT, fmin((double)p->D1, (double)p->D2)));
+    const double t_exec = (p->D1 * 1.0 / Tbig * p->D2 * 1.0 / Tbig) * orc_exec_predict(p->exec, Tbig, p->ta, 'N');
+    double t_recv = 0, t_send = 0;
+    for (int i = 0; i < 3; ++i) {
+      const double d1 = (i == 2) ? (double)p->D2 : (double)p->D1, d2 = (i == 0) ? (double)p->D2 : 1.0;
+      t_recv += in[i] * orc_t_com_predict(p->remote[i] ? &p->h2d : &local, d1 * d2 * p->dtype_sz);
+      t_send += out[i] * orc_t_com_predict(p->out_remote[i] ? &p->h2d : &local, d1 * d2 * p->dtype_sz);
+    }
+    return mode == ORC_FULL_OVERLAP ? fmax(t_exec, fmax(t_recv, t_send)) : t_exec + t_recv + t_send;
+  }
+  if (mode != ORC_BIDIRECTIONAL) return -1.0;
+  const double t_exec = orc_exec_predict(p->exec, T, p->ta, 'N');
+  if (t_exec < 0) return -1.0;
+  const int host = mv_is_host(p, 3);
+  const double bytes = (double)T * p->dtype_sz;
+  const double t_recv = orc_t_com_predict(host ? &p->h2d : &local, bytes);
+  const double t_send = orc_t_com_predict(host ? &p->d2h : &local, bytes);
+  int numTin = 0, numTout = 0;
+  for (int i = 0; i < 3; ++i) { numTin += in[i] * p->remote[i]; numTout += out[i] * p->remote[i]; }
+  const double ker_over = (1.0 * p->D1 / T) - 1;
+  const double t_over = orc_t_com_bid_predict(host ? &p->h2d : &local, host ? &p->d2h : &local, bytes * numTin, bytes * numTout);
+  return fmax(t_exec, t_over) * ker_over + fmax(t_exec, numTout * t_send) + numTin * t_recv + numTout * t_send;
+}
+
 long orc_optimize_tile_model(int mode, const orc_problem* p, double* pred_t) { /* Model_functions.cpp:195-244 */
   long minT = p->exec->T[0];
   for (int i = 0; i < p->exec->lines; ++i)
@@ -485,7 +566,7 @@ long orc_optimize_tile_model(int mode, const orc_problem* p, double* pred_t) { /
 static void* g_blas = NULL;
 static char g_blas_path[1024] = "";
 static int g_ilp64 = 0;
-static void *g_dgemm, *g_sgemm, *g_daxpy, *g_ddot, *g_cfg, *g_setthr, *g_getthr;
+static void *g_dgemm, *g_sgemm, *g_dgemv, *g_daxpy, *g_ddot, *g_cfg, *g_setthr, *g_getthr;
 
 static int try_open(const char* path) {
   void* h = dlopen(path, RTLD_NOW | RTLD_LOCAL);
@@ -500,6 +581,7 @@ static int try_open(const char* path) {
       if (!f) continue;
       g_dgemm = f;
       snprintf(name, sizeof name, "%ssgemm%s", pre[pr], suf[s]); g_sgemm = dlsym(h, name);
+      snprintf(name, sizeof name, "%sdgemv%s", pre[pr], suf[s]); g_dgemv = dlsym(h, name);
       snprintf(name, sizeof name, "%sdaxpy%s", pre[pr], suf[s]); g_daxpy = dlsym(h, name);
       snprintf(name, sizeof name, "%sddot%s", pre[pr], suf[s]); g_ddot = dlsym(h, name);
       const char* op = pr ? "scipy_openblas_" : "openblas_";
@@ -570,6 +652,18 @@ int orc_openblas_sgemm(char ta, char tb, long M, long N, long K, float alpha, co
   else
     ((void (*)(int, int, int, int, int, int, float, const float*, int, const float*, int, float, float*, int))g_sgemm)(
         COL_MAJOR, a, b, (int)M, (int)N, (int)K, alpha, A, (int)lda, B, (int)ldb, beta, C, (int)ldc);
+  return 0;
+}
+int orc_openblas_dgemv(char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                       double beta, double* y, long incy) {
+  if (!g_blas || !g_dgemv) return 1;
+  const int a = is_t(ta) ? TRANS : NO_TRANS;
+  if (g_ilp64)
+    ((void (*)(int, int, int64_t, int64_t, double, const double*, int64_t, const double*, int64_t, double, double*,
+               int64_t))g_dgemv)(COL_MAJOR, a, M, N, alpha, A, lda, x, incx, beta, y, incy);
+  else
+    ((void (*)(int, int, int, int, double, const double*, int, const double*, int, double, double*, int))g_dgemv)(
+        COL_MAJOR, a, (int)M, (int)N, alpha, A, (int)lda, x, (int)incx, beta, y, (int)incy);
   return 0;
 }
 int orc_openblas_daxpy(long n, double alpha, const double* x, long incx, double* y, long incy) {

@@ -10,6 +10,9 @@
  *                             alpha = 0, beta = 0 with NaN C); exact small-integer data
  *   orc_*gemm_tiled           equality with the brute force on integer-valued data for every T; T-invariance
  *   orc_daxpy / orc_ddot_*    OpenBLAS cblas_daxpy/ddot; exact cases (power-of-two alpha, x = y = 1)
+ *   orc_dgemv_bruteforce /    OpenBLAS cblas_dgemv; closed forms (identity, all-ones, alpha = 0, beta = 0 over NaN);
+ *   orc_dgemv_tiled           exact small-integer data for every T and both transposes; gemv as a one-column gemm
+ *   orc_predict_blas2         hand-evaluated closed forms on synthetic (t_exec, ti, tb, sl)
  *   orc_get_T_slowdowns /     hand-derived values: 16384^3 -> T 2048 (sl 0.00390625, 512 subkernels),
  *   orc_optimize_tile         4096^3 -> 2048 (sl 0.25), 32768^3 -> 4096, 40000x40000x2048 -> 2048
  *   orc_t_com_* / orc_predict_* hand-evaluated closed forms on synthetic (t_exec, ti, tb, sl)
@@ -62,6 +65,13 @@ long orc_daxpy_tiled(long T, long n, double alpha, const double* x, long incx, d
 long orc_ddot_tiled(long T, long n, const double* x, long incx, const double* y, long incy, double* result);
 long double orc_ddot_longdouble(long n, const double* x, long incx, const double* y, long incy);
 
+/* ---- BLAS-2 (dgemv.cpp:41-126) ---- */
+void orc_dgemv_bruteforce(char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                          double beta, double* y, long incy); /* long double accumulation */
+/* T x T tiles in index order mi*Ng + ni, beta on the first subkernel of a y tile, 1 afterwards */
+long orc_dgemv_tiled(long T, char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                     double beta, double* y, long incy);
+
 /* ---- tile-size heuristic (Autotuner.cpp:571-655; constants CMakeLists.txt:157-165) ---- */
 long orc_sk_num_blas3(long D1, long D2, long D3, long T);                     /* ModelLvl3.cpp GetSKNumBLAS3 */
 void orc_get_T_slowdowns(long D1, long D2, long D3, int active_unit_num, long T, double sl[6]);
@@ -101,6 +111,7 @@ typedef struct {
 } orc_problem;
 double orc_predict_blas3(int mode, const orc_problem* p, long T);
 double orc_predict_blas1_bidirectional(const orc_problem* p, int numT, const int* in, const int* out, long T);
+double orc_predict_blas2(int mode, const orc_problem* p, long T); /* ModelLvl2.cpp:89-259; D1 = M, D2 = N */
 /* argmin over the T values present in the lookup table, T <= min dim (Model_functions.cpp:195-244) */
 long orc_optimize_tile_model(int mode, const orc_problem* p, double* pred_t);
 
@@ -113,6 +124,8 @@ int orc_openblas_dgemm(char ta, char tb, long M, long N, long K, double alpha, c
                        const double* B, long ldb, double beta, double* C, long ldc);
 int orc_openblas_sgemm(char ta, char tb, long M, long N, long K, float alpha, const float* A, long lda, const float* B,
                        long ldb, float beta, float* C, long ldc);
+int orc_openblas_dgemv(char ta, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                       double beta, double* y, long incy);
 int orc_openblas_daxpy(long n, double alpha, const double* x, long incx, double* y, long incy);
 int orc_openblas_ddot(long n, const double* x, long incx, const double* y, long incy, double* out);
 

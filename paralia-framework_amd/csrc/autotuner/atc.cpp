@@ -147,6 +147,7 @@ void ATC::set_T_slowdowns(double* sl) {
 static long sk_num_of(const ProblemDesc& P, long T) {
   auto cdiv = [](long a, long b) { return a / b + ((a % b) ? 1 : 0); };
   if (P.problem == BLAS3) return cdiv(P.D1, T) * cdiv(P.D2, T) * cdiv(P.D3, T);
+  if (P.problem == BLAS2) return cdiv(P.D1, T) * cdiv(P.D2, T);
   return cdiv(P.D1, T);
 }
 
@@ -277,6 +278,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
   problem = desc;
   problem.func = routine_name;
   if (!strcmp(routine_name, "Dgemm") || !strcmp(routine_name, "Sgemm")) problem.problem = BLAS3;
+  else if (!strcmp(routine_name, "Dgemv")) problem.problem = BLAS2;
   else if (!strcmp(routine_name, "Daxpy") || !strcmp(routine_name, "Ddot")) problem.problem = BLAS1;
   else error("ATC::autotune_problem: routine %s not integrated\n", routine_name);
 
@@ -321,7 +323,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     } else if (!has_db || selector == "heuristic") {
       optimize_tile();
       T_selected_by = "heuristic";
-    } else if (selector == "reuse") {
+    } else if (selector == "reuse" || selector == "cocopelia") {
       optimize_tile_CoCoPeLia(0, COCOPELIA_REUSE);
       T_selected_by = "cocopelia-reuse";
     } else {
@@ -379,6 +381,72 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     pred_t_pesimistic = r.t_h2d + r.t_exec + r.t_d2h;
     update_sk_num(gp.subkernels());
     distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
+  } else if (problem.problem == BLAS2) {
+    // dgemv streams every A tile over the link exactly once and the kernels are three orders of magnitude faster
+    // than the copies, so the call is a two-stage pipeline (tile copies, tile kernels) with the vectors riding
+    // along.  Each benchmarked T is priced by walking that pipeline in the subkernel order mi * Ng + ni
+    // (dgemv.cpp:57-60); the reference's own BLAS-2 model (ModelLvl2.cpp:194-259) is available as
+    // PARALIA_T_SELECT=cocopelia.
+    const long M = problem.D1, N = problem.D2;
+    const long max_dim = std::max(M, N);
+    const bool a_remote = remote(problem.loc[0], 0) != 0;
+    const bool is_n = problem.TransA == 'N';
+    auto cdiv = [](long a, long b) { return a / b + ((a % b) ? 1 : 0); };
+    auto estimate = [&](long cand) -> double {
+      const Modeler* m = unit_modeler_list[0];
+      const comm_data* h2d = m->link[idxize(-1)];
+      const comm_data* d2h = m->revlink[idxize(-1)];
+      const double t_exec = m->exec->predict(cand, problem.TransA);
+      const long len_x = is_n ? N : M, len_y = is_n ? M : N;
+      double copy_end = 0, exec_end = 0;
+      if (remote(problem.loc[1], 0)) copy_end += t_com_predict(h2d, (double)len_x * problem.dtype_sz);
+      if (remote(problem.loc[2], 0) && !problem.beta_is_zero) copy_end += t_com_predict(h2d, (double)len_y * problem.dtype_sz);
+      exec_end = copy_end;
+      for (long mi = 0; mi < cdiv(M, cand); ++mi)
+        for (long ni = 0; ni < cdiv(N, cand); ++ni) {
+          const double tm = (double)std::min(cand, M - mi * cand), tn = (double)std::min(cand, N - ni * cand);
+          if (a_remote) copy_end += t_com_predict(h2d, tm * tn * problem.dtype_sz);
+          exec_end = std::max(exec_end, copy_end) + t_exec * (tm * tn) / ((double)cand * cand);
+        }
+      if (remote(problem.loc[2], 0)) exec_end += t_com_predict(d2h, (double)len_y * problem.dtype_sz);
+      return exec_end;
+    };
+    if (T > 0) {
+      if (T > max_dim) T = max_dim;
+      T_selected_by = "user";
+    } else if (!a_remote) {
+      T = max_dim;  // A already in HBM: one launch over the caller's matrix
+      T_selected_by = "resident";
+    } else if (!has_db) {
+      T = std::min(max_dim, 4096L);  // 128 MiB tiles: the link runs at its asymptotic rate
+      T_selected_by = "heuristic";
+    } else if (selector == "cocopelia" || selector == "reuse") {
+      optimize_tile_CoCoPeLia(0, COCOPELIA_BIDIRECTIONAL);
+      T_selected_by = "cocopelia-bidirectional";
+    } else {
+      const Modeler* m = unit_modeler_list[0];
+      long best_T = -1, prev = -1;
+      double best_t = DBL_MAX;
+      for (long i = 0; i < m->exec->lines(); i++) {
+        const long cand = m->exec->T[i];
+        if (cand == prev || cand > max_dim) continue;
+        prev = cand;
+        if (problem.pool_budget_bytes > 0 && 4LL * cand * cand * problem.dtype_sz > problem.pool_budget_bytes) continue;
+        const double t = estimate(cand);
+        if (t < best_t) { best_t = t; best_T = cand; }
+      }
+      if (best_T < 0) {
+        T = std::min(max_dim, m->exec->MinT());
+        T_selected_by = "heuristic";
+      } else {
+        T = best_T;
+        T_selected_by = "pipeline-model";
+      }
+    }
+    if (T <= 0) error("ATC::autotune_problem: T = %ld after tuning\n", T);
+    if (has_db) pred_t = estimate(T);
+    update_sk_num(sk_num_of(problem, T));
+    distribute_subkernels((int)cdiv(M, T), (int)cdiv(N, T), 1);
   } else {
     const long N = problem.D1;
     if (T > 0) {

@@ -153,10 +153,12 @@ double GPUexecModel::predict(long Tq, char ta, char tb) const {
 }
 
 // BLAS-3 line: TransA,TransB,M,N,K,t,W,J,err,n,bench   (GPUexec_lookup.cpp:79-82)
+// BLAS-2 line: TransA,M,N,t,W,J,err,n,bench            (GPUexec_lookup.cpp:196-198)
 // BLAS-1 line: T,t,W,J,err,n,bench                     (GPUexec_lookup.cpp:311)
 GPUexecModel* GPUexecModel_init(const std::string& db_dir, int dev_id, const char* func) {
   ProblemType problem;
   if (!strcmp(func, "Dgemm") || !strcmp(func, "Sgemm")) problem = BLAS3;
+  else if (!strcmp(func, "Dgemv")) problem = BLAS2;
   else if (!strcmp(func, "Daxpy") || !strcmp(func, "Ddot")) problem = BLAS1;
   else error("GPUexecModel_init: Invalid/Not implemented func %s\n", func);
   char filename[1024];
@@ -182,6 +184,15 @@ GPUexecModel* GPUexecModel_init(const std::string& db_dir, int dev_id, const cha
       }
       m->TransA.push_back(ta);
       m->TransB.push_back(tb);
+    } else if (problem == BLAS2) {
+      char ta;
+      if (sscanf(line, "%c,%ld,%ld,%lf,%lf,%lf,%lf,%ld,%lf", &ta, &Tv, &d2, &t, &W, &J, &err, &n, &bench) != 9) {
+        fclose(fp);
+        delete m;
+        error("GPUexecModel_init: Problem in reading model (%s line %d)\n", filename, lineno);
+      }
+      m->TransA.push_back(ta);
+      m->TransB.push_back('N');  // no second flag: lookups pass the default
     } else {
       if (sscanf(line, "%ld,%lf,%lf,%lf,%lf,%ld,%lf", &Tv, &t, &W, &J, &err, &n, &bench) != 7) {
         fclose(fp);

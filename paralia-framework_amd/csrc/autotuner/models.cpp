@@ -1,7 +1,8 @@
 // Modeler: per-unit bundle of link models + exec lookup, and the CoCoPeLia overlap predictions.
 // Arithmetic follows the reference's Autotuner/src/ModelLvl3.cpp:20-73 (full overlap), :239-284 (no overlap),
 // :287-346 (baseline), :348-408 (data location), :410-474 (bidirectional), :476-551 (reuse) and
-// ModelLvl1.cpp:262-326 (BLAS-1 bidirectional), reduced to one GPU plus the host.
+// ModelLvl1.cpp:262-326 (BLAS-1 bidirectional), ModelLvl2.cpp:89-259 (BLAS-2: full / zero overlap and bidirectional),
+// reduced to one GPU plus the host.
 #include <cmath>
 #include <cstring>
 
@@ -30,26 +31,35 @@ Modeler::~Modeler() {
 }
 
 long Modeler::getMinT() const {
-  if (P.problem == BLAS3) return std::max(exec->MinT(), 1024L);  // MinAllowedTBLAS3
+  if (P.problem == BLAS3 || P.problem == BLAS2) return std::max(exec->MinT(), 1024L);  // MinAllowedTBLAS3 / BLAS2
   return exec->MinT();
 }
 long Modeler::getMaxT() const {
   if (P.problem == BLAS3) return std::min(std::min(P.D1, P.D2), P.D3);
+  if (P.problem == BLAS2) return std::min(P.D1, P.D2);  // MaxAllowedTBLAS2
   return P.D1;
 }
 long Modeler::getSKNum(long T) const {
   auto cdiv = [](long a, long b) { return a / b + ((a % b) ? 1 : 0); };
   if (P.problem == BLAS3) return cdiv(P.D1, T) * cdiv(P.D2, T) * cdiv(P.D3, T);
+  if (P.problem == BLAS2) return cdiv(P.D1, T) * cdiv(P.D2, T);  // GetSKNumBLAS2
   return cdiv(P.D1, T);
 }
 long Modeler::getFlops() const {
   if (P.problem == BLAS3) return gemm_flops(P.D1, P.D2, P.D3);
+  if (P.problem == BLAS2) return gemv_flops(P.D1, P.D2);
   return axpy_flops(P.D1);
 }
 
 namespace {
 // Dim1 x Dim2 of operand i: A is D1 x D3, B is D3 x D2, C is D1 x D2 (CoCoModel_gemm_init); vectors are D1 x 1.
 void dims_of(const ProblemDesc& P, int i, double* d1, double* d2) {
+  if (P.problem == BLAS2) {
+    // CoCoModel_gemv_init (ModelLvl2.cpp:66-71): A is D1 x D2, "x" D1 x 1, "y" D2 x 1 whatever TransA says
+    *d1 = (i == 2) ? (double)P.D2 : (double)P.D1;
+    *d2 = (i == 0) ? (double)P.D2 : 1;
+    return;
+  }
   if (P.problem != BLAS3) { *d1 = (double)P.D1; *d2 = 1; return; }
   *d1 = (i == 1) ? (double)P.D3 : (double)P.D1;
   *d2 = (i == 0) ? (double)P.D3 : (double)P.D2;
@@ -68,6 +78,38 @@ double Modeler::predict(ModelType mode, long T) const {
   if (P.problem == BLAS1) {
     if (mode != COCOPELIA_BIDIRECTIONAL) error("Modeler::predict: BLAS-1 supports only COCOPELIA_BIDIRECTIONAL\n");
     const double t_exec = exec->predict(T);
+    if (t_exec < 0) return -1.0;
+    const double bytes = (double)T * P.dtype_sz;
+    const double t_recv = t_com_predict(recv_m, bytes), t_send = t_com_predict(send_m, bytes);
+    int numTin = 0, numTout = 0;
+    for (int i = 0; i < P.numT; ++i) {
+      numTin += P.in[i] * remote(P.loc[i], unit_id);
+      numTout += P.out[i] * remote(P.loc[i], unit_id);
+    }
+    const double ker_over = (1.0 * P.D1 / T) - 1;
+    const double t_over = t_com_bid_predict(recv_m, send_m, bytes * numTin, bytes * numTout);
+    return fmax(t_exec, t_over) * ker_over + fmax(t_exec, numTout * t_send) + numTin * t_recv + numTout * t_send;
+  }
+
+  if (P.problem == BLAS2) {
+    if (mode == FULL_OVERLAP || mode == NO_OVERLAP) {
+      const long Tbig = exec->NearestT((long)fmin((double)exec->MaxT(), fmin((double)P.D1, (double)P.D2)));
+      const double t_exec = (P.D1 * 1.0 / Tbig * P.D2 * 1.0 / Tbig) * exec->predict(Tbig, P.TransA);
+      if (t_exec < 0) return -1.0;
+      double t_recv = 0, t_send = 0;
+      for (int i = 0; i < P.numT; ++i) {
+        double d1, d2;
+        dims_of(P, i, &d1, &d2);
+        t_recv += P.in[i] * t_com_predict(link[idxize(P.loc[i])], d1 * d2 * P.dtype_sz);
+        t_send += P.out[i] * t_com_predict(link[idxize(P.out_loc[i])], d1 * d2 * P.dtype_sz);
+      }
+      return mode == FULL_OVERLAP ? fmax(t_exec, fmax(t_recv, t_send)) : t_exec + t_recv + t_send;
+    }
+    if (mode != COCOPELIA_BIDIRECTIONAL) error("Modeler::predict: BLAS-2 supports FULL_OVERLAP, NO_OVERLAP and COCOPELIA_BIDIRECTIONAL\n");
+    // ModelLvl2.cpp:194-259.  The reference prices a BLAS-2 tile transfer as T elements (a vector tile), not the
+    // T x T matrix tile that actually moves, and counts D1/T kernels; kept as it is, which is why this runtime
+    // picks T for dgemv with its own streaming estimate (ATC::autotune_problem) and reports this one on request.
+    const double t_exec = exec->predict(T, P.TransA);
     if (t_exec < 0) return -1.0;
     const double bytes = (double)T * P.dtype_sz;
     const double t_recv = t_com_predict(recv_m, bytes), t_send = t_com_predict(send_m, bytes);

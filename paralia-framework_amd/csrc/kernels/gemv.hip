@@ -1,0 +1,218 @@
+// fp64 matrix-vector product for gfx950:  y = alpha * op(A) * x + beta * y,  A column-major M x N, leading dimension lda.
+//
+// Stands where the reference calls cublasDgemv on one tile (gemv_backend_in<double>, Library_scheduler
+// dgemv.cpp:41-118; cuBLASDgemvWrap in Benchmarking/CuCuBLAS/src/PARALia/dgemv_runner.cpp).  The routine streams A
+// once (8*M*N bytes) and is bound by HBM, so both kernels are laid out for coalesced 16-byte loads and enough
+// independent loads in flight, not for the matrix cores:
+//   op = N  lanes run down the rows (a wave reads 1 KiB of one column per load), the four waves of a workgroup take
+//           every fourth column of a column chunk and are combined through LDS;
+//   op = T  a wave owns four adjacent columns and walks down their rows, sharing each x load between the four dot
+//           products, then reduces with wavefront shuffles.
+// Long reductions are split into chunks (grid.y) so that about GEMV_TARGET_WGS workgroups are in flight whatever the
+// shape; every chunk writes its partial sums to a workspace and a small second kernel adds them in chunk order and
+// applies alpha and beta.  The summation order therefore depends only on (op, M, N), never on timing.
+#include <hip/hip_runtime.h>
+
+#include "paralia_hip.h"
+
+namespace plk {
+
+typedef double dvec2 __attribute__((ext_vector_type(2)));
+
+constexpr int GEMV_WG = 256;
+constexpr long GEMV_TARGET_WGS = 2048;
+constexpr long GEMV_N_MIN_COLS = 64;    // columns per chunk at least (16 per wave)
+constexpr long GEMV_T_MIN_ROWS = 2048;  // rows per chunk at least
+
+struct GemvShape {
+  long blocks_x;  // row blocks (N) or column groups (T)
+  long chunks;    // grid.y
+  long per_chunk; // columns (N) or rows (T) per chunk
+  int vec;        // rows per lane in one load: 2 when 16-byte loads are possible, else 1
+  long len_y;
+};
+
+// Pure function of the arguments: the workspace size and the summation order follow from it.
+__host__ inline GemvShape gemv_shape(bool trans, long M, long N, long lda, const void* A) {
+  GemvShape s;
+  s.vec = (M % 2 == 0 && lda % 2 == 0 && ((unsigned long long)A % 16) == 0) ? 2 : 1;
+  if (!trans) {
+    s.len_y = M;
+    s.blocks_x = (M + 64 * s.vec - 1) / (64 * s.vec);
+    long want = (GEMV_TARGET_WGS + s.blocks_x - 1) / s.blocks_x;
+    long most = N / GEMV_N_MIN_COLS > 0 ? N / GEMV_N_MIN_COLS : 1;
+    s.chunks = want < most ? want : most;
+    if (s.chunks < 1) s.chunks = 1;
+    s.per_chunk = (N + s.chunks - 1) / s.chunks;
+    s.per_chunk = (s.per_chunk + 3) / 4 * 4;
+    s.chunks = (N + s.per_chunk - 1) / s.per_chunk;
+  } else {
+    s.len_y = N;
+    s.blocks_x = (N + 15) / 16;
+    long want = (GEMV_TARGET_WGS + s.blocks_x - 1) / s.blocks_x;
+    long most = M / GEMV_T_MIN_ROWS > 0 ? M / GEMV_T_MIN_ROWS : 1;
+    s.chunks = want < most ? want : most;
+    if (s.chunks < 1) s.chunks = 1;
+    s.per_chunk = (M + s.chunks - 1) / s.chunks;
+    s.per_chunk = (s.per_chunk + 127) / 128 * 128;
+    s.chunks = (M + s.per_chunk - 1) / s.per_chunk;
+  }
+  if (s.chunks < 1) s.chunks = 1;
+  return s;
+}
+
+template <int VEC> struct RowVec;
+template <> struct RowVec<2> {
+  typedef dvec2 type;
+  static __device__ __forceinline__ dvec2 load(const double* p) { return __builtin_nontemporal_load((const dvec2*)p); }
+  static __device__ __forceinline__ void fma_into(double* acc, dvec2 a, double xv) { acc[0] = fma(a.x, xv, acc[0]); acc[1] = fma(a.y, xv, acc[1]); }
+  static __device__ __forceinline__ double dot_into(double acc, dvec2 a, const double* xv) { return fma(a.y, xv[1], fma(a.x, xv[0], acc)); }
+};
+template <> struct RowVec<1> {
+  typedef double type;
+  static __device__ __forceinline__ double load(const double* p) { return __builtin_nontemporal_load(p); }
+  static __device__ __forceinline__ void fma_into(double* acc, double a, double xv) { acc[0] = fma(a, xv, acc[0]); }
+  static __device__ __forceinline__ double dot_into(double acc, double a, const double* xv) { return fma(a, xv[0], acc); }
+};
+
+// partial[chunk * M + m] = sum over the chunk's columns n of A[m, n] * x[n]
+template <int VEC>
+__global__ __launch_bounds__(GEMV_WG) void gemv_n_kernel(long M, long N, const double* __restrict__ A, long lda,
+                                                         const double* __restrict__ x, long incx, double* __restrict__ partial,
+                                                         long cols_per_chunk) {
+  __shared__ double red[4][64 * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long row0 = ((long)blockIdx.x * 64 + lane) * VEC;
+  const long c0 = (long)blockIdx.y * cols_per_chunk;
+  const long c1 = c0 + cols_per_chunk < N ? c0 + cols_per_chunk : N;
+  double acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = 0.0;
+  if (row0 < M) {  // VEC == 2 is only chosen for even M, so row0 + 1 < M as well
+    const double* col = A + row0;
+    long n = c0 + wave;
+    for (; n + 12 < c1; n += 16) {
+      typename RowVec<VEC>::type a0 = RowVec<VEC>::load(col + n * lda);
+      typename RowVec<VEC>::type a1 = RowVec<VEC>::load(col + (n + 4) * lda);
+      typename RowVec<VEC>::type a2 = RowVec<VEC>::load(col + (n + 8) * lda);
+      typename RowVec<VEC>::type a3 = RowVec<VEC>::load(col + (n + 12) * lda);
+      const double x0 = x[n * incx], x1 = x[(n + 4) * incx], x2 = x[(n + 8) * incx], x3 = x[(n + 12) * incx];
+      RowVec<VEC>::fma_into(acc, a0, x0);
+      RowVec<VEC>::fma_into(acc, a1, x1);
+      RowVec<VEC>::fma_into(acc, a2, x2);
+      RowVec<VEC>::fma_into(acc, a3, x3);
+    }
+    for (; n < c1; n += 4) RowVec<VEC>::fma_into(acc, RowVec<VEC>::load(col + n * lda), x[n * incx]);
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) red[wave][lane * VEC + v] = acc[v];
+  __syncthreads();
+  if (wave == 0 && row0 < M) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const int i = lane * VEC + v;
+      partial[(long)blockIdx.y * M + row0 + v] = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
+    }
+  }
+}
+
+// partial[chunk * N + n] = sum over the chunk's rows m of A[m, n] * x[m]
+template <int VEC>
+__global__ __launch_bounds__(GEMV_WG) void gemv_t_kernel(long M, long N, const double* __restrict__ A, long lda,
+                                                         const double* __restrict__ x, long incx, double* __restrict__ partial,
+                                                         long rows_per_chunk) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long col0 = ((long)blockIdx.x * 4 + wave) * 4;
+  if (col0 >= N) return;
+  const int ncols = N - col0 < 4 ? (int)(N - col0) : 4;
+  const long r0 = (long)blockIdx.y * rows_per_chunk;
+  const long r1 = r0 + rows_per_chunk < M ? r0 + rows_per_chunk : M;
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  const double* base = A + col0 * lda;
+  if (ncols == 4) {
+    for (long m = r0 + (long)lane * VEC; m < r1; m += 64 * VEC) {  // VEC == 2: M and the chunk size are even
+      double xv[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) xv[v] = x[(m + v) * incx];
+      typename RowVec<VEC>::type a[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) a[c] = RowVec<VEC>::load(base + c * lda + m);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] = RowVec<VEC>::dot_into(acc[c], a[c], xv);
+    }
+  } else {
+    for (long m = r0 + lane; m < r1; m += 64) {
+      const double xv = x[m * incx];
+      for (int c = 0; c < ncols; ++c) acc[c] = fma(base[c * lda + m], xv, acc[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    for (int off = 32; off > 0; off >>= 1) acc[c] += __shfl_down(acc[c], off, 64);
+  if (lane == 0)
+    for (int c = 0; c < ncols; ++c) partial[(long)blockIdx.y * N + col0 + c] = acc[c];
+}
+
+// y[i] = alpha * (partial[0][i] + partial[1][i] + ...) + beta * y[i]; beta == 0 never reads y (NaN-safe, as in BLAS)
+__global__ __launch_bounds__(GEMV_WG) void gemv_final_kernel(long len, long chunks, const double* __restrict__ partial, double alpha,
+                                                             double beta, double* __restrict__ y, long incy) {
+  const long i = (long)blockIdx.x * GEMV_WG + threadIdx.x;
+  if (i >= len) return;
+  double s = 0.0;
+  for (long c = 0; c < chunks; ++c) s += partial[c * len + i];
+  double* yp = y + i * incy;
+  *yp = beta == 0.0 ? alpha * s : fma(alpha, s, beta * *yp);
+}
+
+}  // namespace plk
+
+extern "C" {
+
+long long pl_dgemv_workspace_doubles(char trans, long M, long N) {
+  if (M <= 0 || N <= 0) return 0;
+  const bool t = !(trans == 'N' || trans == 'n');
+  // the chunk count depends on which load width the launch will pick (parity of M and lda, alignment of A):
+  // take the larger of the two
+  const plk::GemvShape wide = plk::gemv_shape(t, M + (M & 1), N, 2, nullptr);
+  const plk::GemvShape narrow = plk::gemv_shape(t, M, N, 1, nullptr);
+  const long chunks = wide.chunks > narrow.chunks ? wide.chunks : narrow.chunks;
+  return (long long)chunks * (wide.len_y + 1);
+}
+
+int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
+             double* y, long incy, double* workspace, void* stream) {
+  using namespace plk;
+  const bool is_n = trans == 'N' || trans == 'n';
+  const bool is_t = trans == 'T' || trans == 't' || trans == 'C' || trans == 'c';
+  if (!is_n && !is_t) return PL_ERR_TRANS;
+  if (M < 0 || N < 0) return PL_ERR_DIM;
+  if (lda < (M > 1 ? M : 1)) return PL_ERR_LD;
+  if (incx == 0 || incy == 0) return PL_ERR_LD;
+  if (M == 0 || N == 0 || (alpha == 0.0 && beta == 1.0)) return 0;  // BLAS quick return: y untouched
+  if (!A || !x || !y) return PL_ERR_NULL;
+  hipStream_t st = (hipStream_t)stream;
+  const long len_x = is_n ? N : M, len_y = is_n ? M : N;
+  // BLAS: with a negative increment the vector runs backwards from the far end of its span
+  const double* xs = incx > 0 ? x : x - (len_x - 1) * incx;
+  double* ys = incy > 0 ? y : y - (len_y - 1) * incy;
+  const unsigned fin_blocks = (unsigned)((len_y + GEMV_WG - 1) / GEMV_WG);
+  if (alpha == 0.0) {
+    hipLaunchKernelGGL(gemv_final_kernel, dim3(fin_blocks), dim3(GEMV_WG), 0, st, len_y, 0L, (const double*)nullptr, 0.0, beta, ys, incy);
+    return hipGetLastError() == hipSuccess ? 0 : PL_ERR_HIP;
+  }
+  if (!workspace) return PL_ERR_NULL;
+  const GemvShape s = gemv_shape(is_t, M, N, lda, A);
+  if (s.blocks_x > 0x7fffffffL || s.chunks > 65535) return PL_ERR_DIM;
+  const dim3 grid((unsigned)s.blocks_x, (unsigned)s.chunks);
+  if (is_n) {
+    if (s.vec == 2) hipLaunchKernelGGL(gemv_n_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
+    else hipLaunchKernelGGL(gemv_n_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
+  } else {
+    if (s.vec == 2) hipLaunchKernelGGL(gemv_t_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
+    else hipLaunchKernelGGL(gemv_t_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
+  }
+  hipLaunchKernelGGL(gemv_final_kernel, dim3(fin_blocks), dim3(GEMV_WG), 0, st, len_y, s.chunks, (const double*)workspace, alpha, beta, ys, incy);
+  return hipGetLastError() == hipSuccess ? 0 : PL_ERR_HIP;
+}
+
+}  // extern "C"

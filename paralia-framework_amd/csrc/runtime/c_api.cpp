@@ -13,6 +13,7 @@
 namespace paralia {
 ATC_p dgemm_impl(char, char, long, long, long, double, double*, long, double*, long, double, double*, long, ATC_p);
 ATC_p sgemm_impl(char, char, long, long, long, float, float*, long, float*, long, float, float*, long, ATC_p);
+ATC_p dgemv_impl(char, long, long, double, double*, long, double*, long, double, double*, long, ATC_p);
 ATC_p daxpy_impl(long, double, double*, long, double*, long, ATC_p);
 ATC_p ddot_impl(long, double*, long, double*, long, double*, ATC_p);
 void cache_free_impl(short);
@@ -81,6 +82,14 @@ int PARALiA_sgemm(char TransA, char TransB, long M, long N, long K, float alpha,
   return guarded([&] {
     std::unique_ptr<ATC> predef(make_predef(T, cache_limit));
     std::unique_ptr<ATC> out(paralia::sgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef.get()));
+    fill_info(info, out.get());
+  });
+}
+int PARALiA_dgemv(char TransA, long M, long N, double alpha, double* A, long ldA, double* x, long incx, double beta, double* y,
+                  long incy, long T, long long cache_limit, pl_atc_info* info) {
+  return guarded([&] {
+    std::unique_ptr<ATC> predef(make_predef(T, cache_limit));
+    std::unique_ptr<ATC> out(paralia::dgemv_impl(TransA, M, N, alpha, A, ldA, x, incx, beta, y, incy, predef.get()));
     fill_info(info, out.get());
   });
 }
@@ -161,8 +170,9 @@ static ProblemDesc desc_of(const char* func, long D1, long D2, long D3, char ta,
   ProblemDesc d;
   d.func = func;
   const bool l1 = !strcmp(func, "Daxpy") || !strcmp(func, "Ddot");
-  d.problem = l1 ? BLAS1 : BLAS3;
-  d.D1 = D1; d.D2 = l1 ? 1 : D2; d.D3 = l1 ? 1 : D3;
+  const bool l2 = !strcmp(func, "Dgemv");
+  d.problem = l1 ? BLAS1 : l2 ? BLAS2 : BLAS3;
+  d.D1 = D1; d.D2 = l1 ? 1 : D2; d.D3 = (l1 || l2) ? 1 : D3;
   d.TransA = ta; d.TransB = tb;
   d.dtype_sz = !strcmp(func, "Sgemm") ? 4 : 8;
   d.numT = l1 ? 2 : 3;

@@ -124,6 +124,20 @@ struct Resources {
     chk(pl_malloc_pinned(&p, 64), "ddot host scalar");
     dot_host = (double*)p;
   }
+  // growable device scratch of dgemv: staged copies of host-resident x and y, and the kernels' partial sums
+  struct Scratch {
+    void* p = nullptr;
+    long long cap = 0;
+    void* ensure(long long bytes) {
+      if (bytes <= cap) return p;
+      if (p) chk(pl_free_device(p), "scratch free");
+      p = nullptr; cap = 0;
+      chk(pl_malloc_device(&p, bytes), "scratch allocation");
+      cap = bytes;
+      return p;
+    }
+    void release() { if (p) pl_free_device(p); p = nullptr; cap = 0; }
+  } gemv_x, gemv_y, gemv_ws;
   void* stream(int id) const { return id == STREAM_H2D ? h2d : id == STREAM_D2H ? d2h : exec[id - STREAM_EXEC0]; }
   void sync_all() {
     if (h2d) chk(pl_stream_sync(h2d), "stream sync");
@@ -136,6 +150,7 @@ struct Resources {
     for (void* e : events) pl_event_destroy(e);
     if (dot_ws) pl_free_device(dot_ws);
     if (dot_host) pl_free_pinned(dot_host);
+    gemv_x.release(); gemv_y.release(); gemv_ws.release();
     *this = Resources();
   }
 };
@@ -560,6 +575,153 @@ ATC_p ddot_impl(long N, double* x, long incx, double* y, long incy, double* resu
   return atc_copy(atc);
 }
 
+// ------------------------------------------------------------------------------------------ BLAS-2
+// PARALiADgemv (dgemv.cpp:288-718).  One GPU: a device-resident A is one launch; a host-resident A is cut into
+// T x T tiles (subkernel mi * Ng + ni, dgemv.cpp:57-60) that cross the link once each through a small ring of device
+// blocks while the kernel of the previous tile runs; x and y are staged whole (they are M + N elements against
+// M * N of A).  The first subkernel of a y tile applies the caller's beta, later ones accumulate (WR_first /
+// DgemvUpdateDevice, dgemv.cpp:121-126).
+ATC_p dgemv_impl(char TransA, long M, long N, double alpha, double* A, long ldA, double* x, long incx, double beta, double* y,
+                 long incy, ATC_p predef) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  const char ta = (char)toupper(TransA);
+  if (ta != 'N' && ta != 'T') error("PARALiADgemv: invalid transpose flag '%c' (only N and T)\n", TransA);
+  if (M < 0 || N < 0) error("PARALiADgemv: negative dimension (%ld, %ld)\n", M, N);
+  if (ldA < std::max(1L, M)) error("PARALiADgemv: leading dimension %ld smaller than %ld rows\n", ldA, M);
+  if (incx == 0 || incy == 0) error("PARALiADgemv: zero increment\n");
+  auto empty = [] { ATC_p out = new ATC(); out->T = 0; out->active_unit_num = 1; out->active_unit_id_list[0] = 0; out->subkernel_num = 0; return out; };
+  if (M == 0 || N == 0) return empty();  // BLAS quick return: y is not touched
+  if (!A || !x || !y) error("PARALiADgemv: null operand\n");
+  int locA = 0, locx = 0, locy = 0;
+  chk(pl_ptr_location(A, &locA), "pointer location");
+  chk(pl_ptr_location(x, &locx), "pointer location");
+  chk(pl_ptr_location(y, &locy), "pointer location");
+  if (locA > 0 || locx > 0 || locy > 0) error("PARALiADgemv: operand on device %d; only device 0 is driven\n", std::max(locA, std::max(locx, locy)));
+  int prev_dev = 0;
+  chk(pl_get_device(&prev_dev), "get device");
+  if (prev_dev != 0) chk(pl_set_device(0), "set device");
+  struct Restore { int d; ~Restore() { if (d != 0) pl_set_device(d); } } restore{prev_dev};
+
+  const long len_x = ta == 'N' ? N : M, len_y = ta == 'N' ? M : N;
+  const long ax = std::labs(incx), ay = std::labs(incy);
+  const bool beta_zero = beta == 0.0;
+
+  // ---- tuned problem (metadata cache)
+  PMDKey key;
+  key.routine = "Dgemv"; key.ta = ta; key.D1 = M; key.D2 = N; key.D3 = 1;
+  key.loc[0] = host_or_dev(locA); key.loc[1] = host_or_dev(locx); key.loc[2] = host_or_dev(locy);
+  key.beta_zero = beta_zero;
+  key.predef_T = predef ? predef->T : -1;
+  key.cache_limit = predef ? predef->cache_limit : 0;
+  ATC* atc = nullptr;
+  for (auto& e : R.pmd)
+    if (e->key == key) { ++R.pmd_hits; atc = e->atc.get(); break; }
+  if (!atc) {
+    ++R.pmd_misses;
+    std::unique_ptr<PMDEntry> ne(new PMDEntry());
+    ne->key = key;
+    ne->atc.reset(new ATC());
+    atc = ne->atc.get();
+    if (predef) {
+      atc->T = predef->T; atc->cache_limit = predef->cache_limit; atc->active_unit_num = predef->active_unit_num;
+      for (int d = 0; d < LOC_NUM; d++) atc->active_unit_id_list[d] = predef->active_unit_id_list[d];
+    }
+    ProblemDesc d;
+    d.func = "Dgemv"; d.problem = BLAS2; d.D1 = M; d.D2 = N; d.D3 = 1; d.TransA = ta; d.dtype_sz = 8; d.numT = 3;
+    d.in[0] = d.in[1] = d.in[2] = 1;
+    d.out[0] = d.out[1] = 0; d.out[2] = 1;
+    for (int i = 0; i < 3; ++i) d.loc[i] = d.out_loc[i] = key.loc[i];
+    d.beta_is_zero = beta_zero;
+    d.pool_budget_bytes = key.loc[0] < 0 ? pool_budget(key.cache_limit, R.pool.bytes()) : 0;
+    atc->autotune_problem("Dgemv", d);
+    if (key.loc[0] < 0) {
+      // dgemv.cpp:389-390: one 2-D block (and two 1-D blocks) is the least the routine can run with
+      const long long tile = (long long)std::min(atc->T, M) * std::min(atc->T, N) * 8 + 256;
+      if (d.pool_budget_bytes < tile) error("PARALiADgemv: Problem cannot run with less memory than %lld\n", tile);
+    }
+    if ((int)R.pmd.size() >= PROBLEM_MD_CACHE) R.pmd.erase(R.pmd.begin());
+    R.pmd.push_back(std::move(ne));
+    atc = R.pmd.back()->atc.get();
+  }
+  if (alpha == 0.0 && beta == 1.0) return atc_copy(atc);  // BLAS quick return
+
+  R.res.ensure_streams(1);
+  void* s_in = R.res.h2d; void* s_ex = R.res.exec[0]; void* s_out = R.res.d2h;
+  R.res.ensure_events(16);
+
+  // ---- vectors: staged whole; a strided vector moves as its contiguous span (gaps included, so that the
+  // write-back of y restores what lies between its elements)
+  const long long span_x = ((long long)(len_x - 1) * ax + 1) * 8, span_y = ((long long)(len_y - 1) * ay + 1) * 8;
+  double* xd = x;
+  double* yd = y;
+  void* ev_vec = R.res.events[0];
+  bool staged = false;
+  if (locx < 0 && alpha != 0.0) {
+    xd = (double*)R.res.gemv_x.ensure(span_x);
+    chk(pl_copy_async(xd, x, span_x, s_in), "fetch x");
+    staged = true;
+  }
+  if (locy < 0) {
+    yd = (double*)R.res.gemv_y.ensure(span_y);
+    if (!beta_zero || ay != 1) { chk(pl_copy_async(yd, y, span_y, s_in), "fetch y"); staged = true; }
+  }
+  if (staged) {
+    chk(pl_event_record(ev_vec, s_in), "event record");
+    chk(pl_stream_wait_event(s_ex, ev_vec), "stream wait event");
+  }
+
+  const long T = atc->T;
+  if (locA >= 0 || alpha == 0.0) {
+    double* ws = nullptr;
+    if (alpha != 0.0) ws = (double*)R.res.gemv_ws.ensure(std::max(8LL, pl_dgemv_workspace_doubles(ta, M, N) * 8));
+    chk(pl_dgemv(ta, M, N, alpha, A, ldA, xd, incx, beta, yd, incy, ws, s_ex), "dgemv launch");
+  } else {
+    const long Mg = (M + T - 1) / T, Ng = (N + T - 1) / T;
+    const long tiles = Mg * Ng;
+    const long long blk = ((long long)std::min(T, M) * std::min(T, N) * 8 + 255) / 256 * 256;  // slots keep A's alignment
+    long long budget = pool_budget(atc->cache_limit, R.pool.bytes());
+    const int ring = (int)std::max<long long>(1, std::min<long long>(std::min<long>(tiles, 4), budget / blk));
+    R.pool.ensure(ring, blk);
+    // every tile has at most max(T, ...) outputs per chunk: size the workspace for the largest tile shape
+    long long ws_doubles = 8;
+    for (long mi : {0L, Mg - 1})
+      for (long ni : {0L, Ng - 1}) {
+        const long tm = std::min(T, M - mi * T), tn = std::min(T, N - ni * T);
+        ws_doubles = std::max(ws_doubles, pl_dgemv_workspace_doubles(ta, tm, tn));
+      }
+    double* ws = (double*)R.res.gemv_ws.ensure(ws_doubles * 8);
+    for (long t = 0; t < tiles; ++t) {
+      const long mi = t / Ng, ni = t % Ng;
+      const long tm = std::min(T, M - mi * T), tn = std::min(T, N - ni * T);
+      const int r = (int)(t % ring);
+      void* ev_in = R.res.events[1 + 2 * r];
+      void* ev_ex = R.res.events[2 + 2 * r];
+      double* Ad = (double*)R.pool.at(r);
+      if (t >= ring) chk(pl_stream_wait_event(s_in, ev_ex), "stream wait event");  // the slot's previous tile was consumed
+      chk(pl_copy2d_async(Ad, tm, A + mi * T + ni * T * ldA, ldA, tm, tn, 8, s_in), "fetch A tile");
+      chk(pl_event_record(ev_in, s_in), "event record");
+      chk(pl_stream_wait_event(s_ex, ev_in), "stream wait event");
+      // tile (mi, ni) multiplies the x tile of its reduction index into the y tile of its output index
+      const long xi = ta == 'N' ? ni : mi, yi = ta == 'N' ? mi : ni;
+      const long xlen = ta == 'N' ? tn : tm, ylen = ta == 'N' ? tm : tn;
+      const long xoff = incx >= 0 ? xi * T * ax : (len_x - xi * T - xlen) * ax;
+      const long yoff = incy >= 0 ? yi * T * ay : (len_y - yi * T - ylen) * ay;
+      const bool first = (ta == 'N' ? ni : mi) == 0;
+      chk(pl_dgemv(ta, tm, tn, alpha, Ad, tm, xd + xoff, incx, first ? beta : 1.0, yd + yoff, incy, ws, s_ex), "dgemv tile launch");
+      chk(pl_event_record(ev_ex, s_ex), "event record");
+    }
+  }
+  if (locy < 0) {
+    void* ev_done = R.res.events[15];
+    chk(pl_event_record(ev_done, s_ex), "event record");
+    chk(pl_stream_wait_event(s_out, ev_done), "stream wait event");
+    chk(pl_copy_async(y, yd, span_y, s_out), "write back y");
+  }
+  R.res.sync_all();
+  return atc_copy(atc);
+}
+
 void cache_free_impl(short dev_id) {
   Runtime& R = rt();
   std::lock_guard<std::mutex> lk(R.mu);
@@ -607,6 +769,14 @@ ATC_p PARALiASgemm(char TransA, char TransB, long int M, long int N, long int K,
 ATC_p PARALiASgemmControled(char TransA, char TransB, long int M, long int N, long int K, float alpha, float* A,
                             long int ldA, float* B, long int ldB, float beta, float* C, long int ldC, ATC_p predef) {
   PARALIA_TERMINATE_ON_ERROR(sgemm_impl(TransA, TransB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, predef));
+}
+ATC_p PARALiADgemv(char TransA, long int M, long int N, double alpha, double* A, long int ldA, double* x, long int incx,
+                   double beta, double* y, long int incy) {
+  PARALIA_TERMINATE_ON_ERROR(dgemv_impl(TransA, M, N, alpha, A, ldA, x, incx, beta, y, incy, nullptr));
+}
+ATC_p PARALiADgemvControled(char TransA, long int M, long int N, double alpha, double* A, long int ldA, double* x,
+                            long int incx, double beta, double* y, long int incy, ATC_p predef) {
+  PARALIA_TERMINATE_ON_ERROR(dgemv_impl(TransA, M, N, alpha, A, ldA, x, incx, beta, y, incy, predef));
 }
 ATC_p PARALiADaxpy(long int N, double alpha, double* x, long int incx, double* y, long int incy) {
   PARALIA_TERMINATE_ON_ERROR(daxpy_impl(N, alpha, x, incx, y, incy, nullptr));

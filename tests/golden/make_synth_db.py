@@ -2,9 +2,11 @@
 
 File formats are the reference's (Autotuner/src/GPUexec_lookup.cpp:79-82,311; CoModel.cpp:32-55):
   <Func>_lookup-table_dev-0.log   BLAS-3: TransA,TransB,M,N,K,t,W,J,err,n,bench   BLAS-1: T,t,W,J,err,n,bench
+                                  BLAS-2 (GPUexec_lookup.cpp:196-198): TransA,M,N,t,W,J,err,n,bench
   Link-Stats_loc_dest-<to>_loc_src-<from>.log   Intercept / Coefficient / Slowdown([src]->[dst]) lines
 Numbers are round on purpose so that tests can state expected predictions by hand:
-  Dgemm NN tile time 1e-3 s at T=1024 scaling with T^3; H2D 0.5e-3 s and D2H 0.25e-3 s per 1024^2 fp64 tile.
+  Dgemm NN tile time 1e-3 s at T=1024 scaling with T^3; H2D 0.5e-3 s and D2H 0.25e-3 s per 1024^2 fp64 tile;
+  Dgemv N tile time 2e-5 s at T=1024 scaling with T^2 (T: 1.25 times that).
 Also writes db_v100/, three real rows of the reference's own V100 logs re-cut into the Processed layout.
 Run from the repository root: python tests/golden/make_synth_db.py
 """
@@ -34,6 +36,12 @@ def synth():
             t = 0.5e-3 * s * (T / 1024.0) ** 3
             rows.append("%s,%s,%d,%d,%d,%e,%e,%e,%e,%d,%e" % (ta, tb, T, T, T, t, 0.0, 0.0, t * 0.01, 100, 1.0))
     write(os.path.join(d, "Sgemm_lookup-table_dev-0.log"), "\n".join(rows) + "\n")
+    rows = []
+    for T in (512, 1024, 2048, 4096):
+        for ta, sc in (("N", 1.0), ("T", 1.25)):
+            t = 2e-5 * sc * (T / 1024.0) ** 2
+            rows.append("%s,%d,%d,%e,%e,%e,%e,%d,%e" % (ta, T, T, t, 0.0, 0.0, t * 0.01, 100, 1.0))
+    write(os.path.join(d, "Dgemv_lookup-table_dev-0.log"), "\n".join(rows) + "\n")
     for func, per in (("Daxpy", 1e-4), ("Ddot", 0.8e-4)):
         rows = []
         for T in (1 << 16, 1 << 18, 1 << 20, 1 << 22):

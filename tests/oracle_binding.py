@@ -42,6 +42,8 @@ _SIGS = {
     "orc_sgemm_bruteforce": (None, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l]),
     "orc_dgemm_tiled": (_l, [_l, _i, _c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l]),
     "orc_sgemm_tiled": (_l, [_l, _i, _c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l]),
+    "orc_dgemv_bruteforce": (None, [_c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l]),
+    "orc_dgemv_tiled": (_l, [_l, _c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l]),
     "orc_daxpy": (None, [_l, _d, _vp, _l, _vp, _l]),
     "orc_daxpy_mul_add": (None, [_l, _d, _vp, _l, _vp, _l]),
     "orc_daxpy_tiled": (_l, [_l, _l, _d, _vp, _l, _vp, _l]),
@@ -59,6 +61,7 @@ _SIGS = {
     "orc_exec_predict": (_d, [C.POINTER(orc_exec_table), _l, _c, _c]),
     "orc_predict_blas3": (_d, [_i, C.POINTER(orc_problem), _l]),
     "orc_predict_blas1_bidirectional": (_d, [C.POINTER(orc_problem), _i, C.POINTER(_i), C.POINTER(_i), _l]),
+    "orc_predict_blas2": (_d, [_i, C.POINTER(orc_problem), _l]),
     "orc_optimize_tile_model": (_l, [_i, C.POINTER(orc_problem), _pd]),
     "orc_openblas_open": (_i, [C.c_char_p]),
     "orc_openblas_path": (C.c_char_p, []),
@@ -66,6 +69,7 @@ _SIGS = {
     "orc_openblas_threads": (_i, [_i]),
     "orc_openblas_dgemm": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l]),
     "orc_openblas_sgemm": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l]),
+    "orc_openblas_dgemv": (_i, [_c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l]),
     "orc_openblas_daxpy": (_i, [_l, _d, _vp, _l, _vp, _l]),
     "orc_openblas_ddot": (_i, [_l, _vp, _l, _vp, _l, _pd]),
 }

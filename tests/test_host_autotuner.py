@@ -160,3 +160,54 @@ def test_autotune_memory_limit(L, pkg):
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 0, 2048, 2 * blk, C.byref(info)) != 0
     assert b"less memory" in L.PARALiA_last_error()
     L.PARALiA_set_db_dir(None)
+
+
+def test_blas2_models_by_hand_and_against_oracle(L, orc):
+    """Dgemv through the shipped Modeler: the hand-worked values of the oracle's test, then a sweep against the oracle
+    on the synthetic table (N: 20 us at T = 1024 scaling with T^2; T: 1.25 times that; slowdowns 1.25 / 1.5)."""
+    pred = lambda mode, loc=HOST3, T=1024, ta=b"N": L.PARALiA_model_predict(DB_SYNTH, b"Dgemv", mode, 4096, 4096, 1, ta, b"N", loc, T)
+    assert abs(pred(5) - 8.1708984375e-5) < 1e-18
+    assert abs(pred(9) - 8.00390625e-3) < 1e-15
+    assert abs(pred(10) - 8.325859375e-3) < 1e-15
+    Ts = [512, 1024, 2048, 4096]
+    for ta, sc in ((b"N", 1.0), (b"T", 1.25)):
+        tab, keep = make_table(Ts, [float("%e" % (2e-5 * sc * (t / 1024.0) ** 2)) for t in Ts], ta.decode() * 4, "NNNN")
+        for dims in ((4096, 4096), (8192, 2048), (5000, 7000)):
+            for locs in ((-1, -1, -1), (-1, 0, 0), (0, -1, -1), (0, 0, 0)):
+                p = orc_problem()
+                p.D1, p.D2, p.D3, p.dtype_sz, p.ta, p.tb = dims[0], dims[1], 1, 8, ta, b"N"
+                for i in range(3):
+                    p.remote[i] = p.out_remote[i] = 1 if locs[i] < 0 else 0
+                p.h2d = orc_link(0.0, float("%.17e" % (0.5e-3 / TILE)), 1.25)
+                p.d2h = orc_link(0.0, float("%.17e" % (0.25e-3 / TILE)), 1.5)
+                p.exec = C.pointer(tab)
+                for mode in (5, 9, 10):
+                    for T in (512, 1024, 3000):
+                        a = L.PARALiA_model_predict(DB_SYNTH, b"Dgemv", mode, dims[0], dims[1], 1, ta, b"N", loc3(*locs), T)
+                        b = orc.orc_predict_blas2(mode, p, T)
+                        assert abs(a - b) <= 1e-12 * max(1.0, abs(b)), (mode, T, dims, locs, ta, a, b)
+
+
+def test_dgemv_autotune(L, pkg, monkeypatch):
+    """Tile choice for dgemv.  With the synthetic zero-latency link every T moves the same bytes, so the smallest
+    benchmarked tile wins (only the last kernel is exposed): 8192 x 8192 on the host ->
+    x and y in 2 * 3.90625 us, 256 tiles of 512^2 in 32 ms, last kernel 5 us, y back in 1.953125 us."""
+    info = pkg.atc_info()
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 8192, 8192, 1, b"N", b"N", HOST3, 0, -1, 0, C.byref(info)) == 0
+    assert info.T == 512 and info.selected_by == b"pipeline-model" and info.subkernel_num == 256
+    assert abs(info.pred_t - 0.032014765625) < 1e-12
+    # beta == 0: y is not fetched
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 8192, 8192, 1, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert abs(info.pred_t - (0.032014765625 - 3.90625e-6)) < 1e-12
+    # A resident on the device: one launch, T labels the call
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 8192, 4096, 1, b"T", b"N", loc3(0, -1, -1), 0, -1, 0, C.byref(info)) == 0
+    assert info.T == 8192 and info.selected_by == b"resident" and info.subkernel_num == 1
+    # a preset tile is kept (clamped to the larger dimension), ragged grid 3 x 2
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 5000, 3000, 1, b"N", b"N", HOST3, 0, 2048, 0, C.byref(info)) == 0
+    assert info.T == 2048 and info.selected_by == b"user" and info.subkernel_num == 6
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 5000, 3000, 1, b"N", b"N", HOST3, 0, 1 << 20, 0, C.byref(info)) == 0
+    assert info.T == 5000 and info.subkernel_num == 1
+    # a memory budget too small for four 4096^2 tiles rules that candidate out; the reference's own selector on request
+    monkeypatch.setenv("PARALIA_T_SELECT", "cocopelia")
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 8192, 8192, 1, b"N", b"N", HOST3, 0, -1, 0, C.byref(info)) == 0
+    assert info.selected_by == b"cocopelia-bidirectional" and info.T in (1024, 2048, 4096)
