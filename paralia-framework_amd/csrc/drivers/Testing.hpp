@@ -73,6 +73,33 @@ inline void ParseInputLvl1(const int argc, const char* argv[], ATC_p* predef, do
           *alpha, (size_t)*D1, (size_t)*inc1, (size_t)*inc2, *loc1, *loc2, *outloc1, *outloc2);
 }
 
+/// argv of the BLAS-2 drivers (testing.cpp:215-271):
+///   active_unit_num dev_ids_token T cache_limit TransA alpha beta D1 D2 inc1 inc2 loc1 loc2 loc3 outloc
+inline void ParseInputLvl2(const int argc, const char* argv[], ATC_p* predef, char* TransA, double* alpha, double* beta,
+                           long int* D1, long int* D2, long int* inc1, long int* inc2, short* loc1, short* loc2, short* loc3,
+                           short* outloc) {
+  if (argc != 16)
+    error("Incorrect input arguments. Usage: ./correct_run\n\tactive_unit_num(auto if <0)\n\tdev_ids(form example: 0101 for devices 0,2 - "
+          "ignore if active_unit_num < 0)\n\tT(auto if <=0)\n\tcache_max_size(auto if <0)\n\tTransA alpha beta D1 D2 inc1 inc2 loc1 loc2 loc3 "
+          "outloc \n");
+  *predef = parse_control("ParseInputLvl2", argv);
+  *TransA = argv[5][0];
+  *alpha = atof(argv[6]);
+  *beta = atof(argv[7]);
+  *D1 = atol(argv[8]);
+  *D2 = atol(argv[9]);
+  *inc1 = atol(argv[10]);
+  *inc2 = atol(argv[11]);
+  *loc1 = atoi(argv[12]);
+  *loc2 = atoi(argv[13]);
+  *loc3 = atoi(argv[14]);
+  *outloc = atoi(argv[15]);
+  fprintf(stderr, "ParseInputLvl2: ");
+  if (*predef) (*predef)->print();
+  fprintf(stderr, "Routine values:\n\tTransA: %c\n\talpha: %lf, beta: %lf\n\tD1: %zu, D2: %zu, inc1: %zu, inc2: %zu\n\tloc1: %d, loc2: %d, "
+          "loc3: %d, outloc: %d\n", *TransA, *alpha, *beta, (size_t)*D1, (size_t)*D2, (size_t)*inc1, (size_t)*inc2, *loc1, *loc2, *loc3, *outloc);
+}
+
 inline void ParseInputLvl3(const int argc, const char* argv[], ATC_p* predef, char* TransA, char* TransB, double* alpha,
                            double* beta, long int* D1, long int* D2, long int* D3, short* loc1, short* loc2, short* loc3,
                            short* outloc) {
@@ -111,6 +138,18 @@ inline void StoreLogLvl1(const char* filename, ATC_p ctl, double alpha, long int
   fclose(fp);
 }
 
+/// "T,units,dev_token,cache, TransA,alpha,beta,D1,D2,inc1,inc2,loc1,loc2,loc3,outloc, t,pred_t,pred_J" (testing.cpp:414)
+inline void StoreLogLvl2(const char* filename, ATC_p ctl, char TransA, double alpha, double beta, long int D1, long int D2,
+                         long int inc1, long int inc2, short loc1, short loc2, short loc3, short outloc, double timer, double pred_t,
+                         double pred_J) {
+  FILE* fp = fopen(filename, "a");
+  if (!fp) error("report_results: LogFile failed to open");
+  const char* control_str = ctl ? ctl->print_csv() : "-1,-1,-1,-1";
+  fprintf(fp, "%s, %c,%.5lf,%.5lf,%zu,%zu,%zu,%zu,%d,%d,%d,%d, %e,%e,%e\n", control_str, TransA, alpha, beta, (size_t)D1, (size_t)D2,
+          (size_t)inc1, (size_t)inc2, loc1, loc2, loc3, outloc, timer, pred_t, pred_J);
+  fclose(fp);
+}
+
 /// "T,units,dev_token,cache, TransA,TransB,alpha,beta,D1,D2,D3,loc1,loc2,loc3,outloc, t,pred_t,pred_J" (testing.cpp:424)
 inline void StoreLogLvl3(const char* filename, ATC_p ctl, char TransA, char TransB, double alpha, double beta, long int D1,
                          long int D2, long int D3, short loc1, short loc2, short loc3, short outloc, double timer, double pred_t,
@@ -129,7 +168,7 @@ inline void StoreLogLvl3(const char* filename, ATC_p ctl, char TransA, char Tran
 struct OpenBlas {
   void* h = nullptr;
   bool ilp64 = false;
-  void *dgemm = nullptr, *sgemm = nullptr, *daxpy = nullptr, *ddot = nullptr, *cfg = nullptr, *setthr = nullptr;
+  void *dgemm = nullptr, *sgemm = nullptr, *dgemv = nullptr, *daxpy = nullptr, *ddot = nullptr, *cfg = nullptr, *setthr = nullptr;
   std::string path;
   bool try_open(const char* p) {
     void* hh = dlopen(p, RTLD_NOW | RTLD_LOCAL);
@@ -143,6 +182,7 @@ struct OpenBlas {
         if (!f) continue;
         dgemm = f;
         sgemm = dlsym(hh, (base + "sgemm" + tail).c_str());
+        dgemv = dlsym(hh, (base + "dgemv" + tail).c_str());
         daxpy = dlsym(hh, (base + "daxpy" + tail).c_str());
         ddot = dlsym(hh, (base + "ddot" + tail).c_str());
         const std::string ob = q ? "scipy_openblas_" : "openblas_";
@@ -188,6 +228,12 @@ struct OpenBlas {
     const int a = (ta == 'T') ? 112 : 111, b = (tb == 'T') ? 112 : 111;
     if (ilp64) ((void (*)(int, int, int, int64_t, int64_t, int64_t, float, const float*, int64_t, const float*, int64_t, float, float*, int64_t))sgemm)(102, a, b, M, N, K, al, A, lda, B, ldb, be, C, ldc);
     else ((void (*)(int, int, int, int, int, int, float, const float*, int, const float*, int, float, float*, int))sgemm)(102, a, b, (int)M, (int)N, (int)K, al, A, (int)lda, B, (int)ldb, be, C, (int)ldc);
+  }
+  void Dgemv(char ta, long M, long N, double al, const double* A, long lda, const double* x, long incx, double be, double* y,
+             long incy) const {
+    const int a = (ta == 'T') ? 112 : 111;
+    if (ilp64) ((void (*)(int, int, int64_t, int64_t, double, const double*, int64_t, const double*, int64_t, double, double*, int64_t))dgemv)(102, a, M, N, al, A, lda, x, incx, be, y, incy);
+    else ((void (*)(int, int, int, int, double, const double*, int, const double*, int, double, double*, int))dgemv)(102, a, (int)M, (int)N, al, A, (int)lda, x, (int)incx, be, y, (int)incy);
   }
   void Daxpy(long n, double al, const double* x, long incx, double* y, long incy) const {
     if (ilp64) ((void (*)(int64_t, double, const double*, int64_t, double*, int64_t))daxpy)(n, al, x, incx, y, incy);

@@ -1,15 +1,17 @@
 // Deploy-time microbenchmarks and database builder for one MI355X.
 //
-//   paralia_deploy <db_dir> [--quick] [--only gemm|blas1|link]
+//   paralia_deploy <db_dir> [--quick] [--only gemm|gemv|blas1|link]
 //
 // Measures (1) the tile GEMM kernels over square T for the four transpose combinations, fp64 and fp32,
-// (2) daxpy / ddot over vector lengths, (3) pinned-host <-> device 2-D tile copies in both directions and the
+// (2) daxpy / ddot over vector lengths and dgemv over square T for both transposes, (3) pinned-host <-> device 2-D tile copies in both directions and the
 // slowdown of each direction while the other is busy; writes the raw logs to <db_dir>/Benchmark-Results and the
 // tables the autotuner reads to <db_dir>/Processed.
 //
 // What it re-does from the reference: Database_builder/CuCuBLAS/src/dgemm_microbench.cu:26-230 (T sweep from
 // 256 in steps of 256, the step doubling once T >= 16*step, up to < 10000; alpha = 1.1234;
 // stop when the 95% confidence half-width is within 5% of the mean and more than 10 samples were taken),
+// dgemv_microbench.cu:26-250 (the same T sweep, MIN/STEP/MAX_DIM_BLAS2 of microbenchmarks.hpp:31-33; table line
+// TransA,M,N,t,W,J,err,n,bench as GPUexec_lookup.cpp:196-198 reads it),
 // daxpy_microbench.cu / ddot_microbench.cu (sweep from 4096 in steps of 4096 with the same doubling),
 // transfer_link_microbench.cu:24-218 (square tiles with a host leading dimension of maxDim + 1, then the
 // overlap run), Python-DataManage/BenchToLookupTables.py.in:31-55 (flag columns prepended, sorted by T) and
@@ -160,6 +162,61 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
   CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
 }
 
+static void bench_gemv(const std::string& db, bool quick) {
+  const long maxDim = quick ? 4352 : 10000;
+  std::vector<long> Ts = sweep(256, 256, maxDim, 16);
+  if (quick) {
+    std::vector<long> few;
+    for (long t : Ts) if (t == 512 || t == 1024 || t == 2048 || t == 4096) few.push_back(t);
+    Ts = few;
+  }
+  double* A = (double*)CoCoMalloc(maxDim * maxDim * sizeof(double), 0, 0);
+  double* x = (double*)CoCoMalloc(maxDim * sizeof(double), 0, 0);
+  double* y = (double*)CoCoMalloc(maxDim * sizeof(double), 0, 1);
+  CoCoVecInit(A, maxDim * maxDim, 42, 0);
+  CoCoVecInit(x, maxDim, 43, 0);
+  CoCoVecInit(y, maxDim, 44, 0);
+  long long ws_doubles = 8;
+  for (long Tt : Ts) ws_doubles = std::max(ws_doubles, std::max(pl_dgemv_workspace_doubles('N', Tt, Tt), pl_dgemv_workspace_doubles('T', Tt, Tt)));
+  double* ws = (double*)CoCoMalloc(ws_doubles * 8, 0, 1);
+  void* st;
+  must(pl_stream_create(&st), "stream");
+  std::vector<Row> rows;
+  for (char ta : {'N', 'T'}) {
+    char raw[1024];
+    snprintf(raw, sizeof raw, "%s/Benchmark-Results/hipDgemv_dev-0_TransA-%c_%s.log", db.c_str(), ta, DEPLOY_VERSION);
+    FILE* fp = fopen(raw, "w");
+    if (!fp) { fprintf(stderr, "cannot write %s\n", raw); exit(1); }
+    for (long Tt : Ts) {
+      const int batch = Tt <= 2048 ? 16 : 4;
+      auto run = [&]() {
+        const double t0 = csecond();
+        // dense tile, beta = 1: the way the scheduler runs every subkernel but the first of a y tile
+        for (int i = 0; i < batch; ++i) must(pl_dgemv(ta, Tt, Tt, 1.1234, A, Tt, x, 1, 1.0, y, 1, ws, st), "dgemv");
+        must(pl_stream_sync(st), "sync");
+        return (csecond() - t0) / batch;
+      };
+      run();
+      Row r{ta, 'N', Tt, sample_until_stable(run)};
+      rows.push_back(r);
+      fprintf(fp, "%ld,%ld, %e,%e,%e,%e,%ld,%e\n", Tt, Tt, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
+      fprintf(stderr, "Dgemv %c T=%ld: %.4f ms (%.1f GB/s), margin %.2f%%, %ld samples\n", ta, Tt, r.s.mean * 1e3,
+              8.0 * Tt * Tt / r.s.mean / 1e9, r.s.margin / r.s.mean * 100, r.s.n);
+    }
+    fclose(fp);
+  }
+  std::stable_sort(rows.begin(), rows.end(), [](const Row& a, const Row& b) { return a.T < b.T; });
+  char out[1024];
+  snprintf(out, sizeof out, "%s/Processed/Dgemv_lookup-table_dev-0.log", db.c_str());
+  FILE* fp = fopen(out, "w");
+  if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  for (const Row& r : rows)
+    fprintf(fp, "%c,%ld,%ld,%e,%e,%e,%e,%ld,%e\n", r.ta, r.T, r.T, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
+  fclose(fp);
+  pl_stream_destroy(st);
+  CoCoFree(A, 0); CoCoFree(x, 0); CoCoFree(y, 0); CoCoFree(ws, 0);
+}
+
 static void bench_blas1(const std::string& db, const char* func, bool quick) {
   const long maxN = quick ? (1L << 24) + 1 : (1L << 27) + 1;
   std::vector<long> Ns = sweep(4096, 4096, maxN, 16);
@@ -294,7 +351,7 @@ static void bench_link(const std::string& db, bool quick) {
 
 int main(int argc, char** argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: %s <db_dir> [--quick] [--only gemm|blas1|link]\n", argv[0]);
+    fprintf(stderr, "usage: %s <db_dir> [--quick] [--only gemm|gemv|blas1|link]\n", argv[0]);
     return 2;
   }
   const std::string db = argv[1];
@@ -317,6 +374,7 @@ int main(int argc, char** argv) {
       bench_gemm<double>(db, "Dgemm", quick, queues);
       bench_gemm<float>(db, "Sgemm", quick, queues);
     }
+    if (only.empty() || only == "gemv") bench_gemv(db, quick);
     if (only.empty() || only == "blas1") {
       bench_blas1(db, "Daxpy", quick);
       bench_blas1(db, "Ddot", quick);

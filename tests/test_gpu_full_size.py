@@ -148,3 +148,27 @@ def test_daxpy_ddot_2p28(pkg, L, orc, openblas, loc):
     assert np.array_equal(host(bx), x)
     bx.free()
     by.free()
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("loc", [0, -1])
+@pytest.mark.parametrize("ta", ["N", "T"])
+def test_dgemv_32768(pkg, L, orc, openblas, loc, ta):
+    """dgemv with a 32768 x 32768 matrix (8 GiB), alpha = 1.2, beta = 1.1, everything on the device (one HBM-bound
+    launch) or everything in pinned host memory (A streamed in tiles picked by the autotuner), against OpenBLAS."""
+    n, alpha, beta = 32768, 1.2, 1.1
+    bA, bx, by = filled(pkg, L, n * n, np.float64, 42, loc), filled(pkg, L, n, np.float64, 43, loc), filled(pkg, L, n, np.float64, 44, loc)
+    A, x, y0 = host(bA), host(bx).copy(), host(by).copy()
+    info = pkg.atc_info()
+    print(f"full-size dgemv {ta} {n}x{n} loc={loc}", flush=True)
+    t0 = time.time()
+    pkg.check(L.PARALiA_dgemv(ta.encode(), n, n, alpha, bA.ptr, n, bx.ptr, 1, beta, by.ptr, 1, -1, 0, C.byref(info)), "dgemv")
+    print(f"  first call {1e3 * (time.time() - t0):.1f} ms, T={info.T} ({info.selected_by.decode()}), {info.subkernel_num} subkernels, "
+          f"predicted {1e3 * info.pred_t:.1f} ms", flush=True)
+    ref = y0.copy()
+    assert openblas.orc_openblas_dgemv(ta.encode(), n, n, alpha, A.ctypes.data, n, x.ctypes.data, 1, beta, ref.ctypes.data, 1) == 0
+    err = float(np.linalg.norm(host(by) - ref)) / (alpha * fro(colmajor(A, n, n)) * float(np.linalg.norm(x)) + beta * float(np.linalg.norm(y0)))
+    print(f"  normwise error vs OpenBLAS {err:.3e}", flush=True)
+    assert err < TOL64
+    for b in (bA, bx, by):
+        b.free()
