@@ -147,8 +147,8 @@ def main():
         t0 = time.perf_counter()
         step_host()                     # cold call: autotune + block pool allocation
         t_cold = time.perf_counter() - t0
-        # untimed: the scheduler tries its four stream alignments on the first four streamed calls and keeps the best
-        for _ in range(max(4, args.warmup)):
+        # untimed: the scheduler tries its four stream alignments on the four streamed calls after the cold one and keeps the best
+        for _ in range(max(5, args.warmup)):
             step_host()
         times = []
         for _ in range(args.steps):

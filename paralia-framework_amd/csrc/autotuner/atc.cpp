@@ -374,6 +374,14 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     paralia::PipelineResult r;
     try {
       order_id = paralia::pick_gemm_order(gp, paralia_stage_times(this, T), &r);
+      // PARALIA_GEMM_ORDER pins the subkernel order family (gemm_plan.hpp) when that order fits the block pool
+      const char* o_env = getenv("PARALIA_GEMM_ORDER");
+      if (o_env && *o_env) {
+        try {
+          r = paralia::simulate_plan(paralia::build_gemm_plan(gp, atoi(o_env)), paralia_stage_times(this, T));
+          order_id = atoi(o_env);
+        } catch (const std::runtime_error&) {}
+      }
     } catch (const std::runtime_error& e) { error("%s\n", e.what()); }
     pipeline.t_total = r.t_total; pipeline.t_h2d_busy = r.t_h2d; pipeline.t_exec_busy = r.t_exec;
     pipeline.t_d2h_busy = r.t_d2h; pipeline.order_id = order_id;

@@ -274,6 +274,8 @@ static void bench_link(const std::string& db, bool quick) {
   void *s1, *s2;
   must(pl_stream_create(&s1), "stream");
   must(pl_stream_create(&s2), "stream");
+  void* ev;
+  must(pl_event_create(&ev, 0), "event");
   struct Dir { int to, from; } dirs[2] = {{0, -1}, {-1, 0}};
   for (const Dir& d : dirs) {
     const bool h2d = d.to == 0;
@@ -288,10 +290,15 @@ static void bench_link(const std::string& db, bool quick) {
     double sx = 0, sy = 0, sxx = 0, sxy = 0;
     long np = 0;
     for (long dim : dims) {
-      const int batch = dim <= 1024 ? 8 : 2;
+      // the cadence of a stream of tile copies as the scheduler issues them: every copy is followed by an event
+      // record (its consumers wait on it), and the batch is long enough that the final sync does not weigh
+      const int batch = dim <= 2048 ? 16 : dim <= 4096 ? 8 : 4;
       auto run = [&]() {
         const double t0 = csecond();
-        for (int i = 0; i < batch; ++i) copy(dim, s1, h2d, host, dev);
+        for (int i = 0; i < batch; ++i) {
+          copy(dim, s1, h2d, host, dev);
+          must(pl_event_record(ev, s1), "event record");
+        }
         must(pl_stream_sync(s1), "sync");
         return (csecond() - t0) / batch;
       };
@@ -346,6 +353,7 @@ static void bench_link(const std::string& db, bool quick) {
   }
   pl_stream_destroy(s1);
   pl_stream_destroy(s2);
+  pl_event_destroy(ev);
   CoCoFree(host, -1); CoCoFree(host2, -1); CoCoFree(dev, 0); CoCoFree(dev2, 0);
 }
 

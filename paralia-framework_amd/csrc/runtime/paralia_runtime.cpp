@@ -67,7 +67,8 @@ struct Resources {
   // one runs the streamed 16384^3 fp64 GEMM in 130 ms, the others in 148-169 ms.  The alignment depends on how
   // many streams the application created before this library did, which cannot be queried.  So seven streams
   // are created back to back, "rotation" r uses streams r .. r+3 as (H2D, D2H, compute 0, compute 1), and
-  // the first four large streamed GEMM calls each run under a different rotation; the fastest is kept
+  // the first four large streamed GEMM calls that repeat an already tuned problem each run under a different
+  // rotation; the fastest is kept
   // (PARALIA_STREAM_ROTATION=r skips the trial).  With 8 or more hardware queues all rotations are equal.
   void* ring[7] = {nullptr};
   int rotation = 0;
@@ -338,6 +339,7 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   PMDEntry* entry = nullptr;
   for (auto& e : R.pmd)
     if (e->key == key) { entry = e.get(); break; }
+  const bool cold = entry == nullptr;
   if (entry) ++R.pmd_hits;
   else {
     ++R.pmd_misses;
@@ -400,7 +402,8 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     const GemmPlan& plan = entry->plan;
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T));
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
-    const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab;
+    // a first call of a problem also pays for fresh pool memory and cold caches: it would misjudge its rotation
+    const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab && !cold;
     if (trial) R.res.begin_trial();
     const double t0 = csecond();
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC);
