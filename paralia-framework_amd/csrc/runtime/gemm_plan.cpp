@@ -18,9 +18,21 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   std::vector<int> order;
   order.reserve((size_t)Mg * Ng * Kg);
   auto id = [&](int mi, int ni, int ki) { return (mi * Ng + ni) * Kg + ki; };
+  // First k-step of a panel: walk the tiles in growing squares (shell d = max(mi, ni)), so that every newly fetched
+  // A or B tile at once enables a whole row or column of subkernels; column by column the first Mg fetches would
+  // enable one subkernel each while the compute streams starve.
+  auto first_step_in_shells = [&](int rows, int cols) {
+    for (int d = 0; d < std::max(rows, cols); ++d) {
+      if (d < cols)
+        for (int mi = 0; mi < std::min(d, rows); ++mi) order.push_back(id(mi, d, 0));
+      if (d < rows)
+        for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(d, ni, 0));
+    }
+  };
   if (orient == 0) {
     w = std::min(w, Ng);
-    for (int ki = 0; ki < Kg; ++ki)
+    if (w > 0 && Kg > 0) first_step_in_shells(Mg, w);
+    for (int ki = 1; ki < Kg; ++ki)
       for (int ni = 0; ni < w; ++ni)
         for (int mi = 0; mi < Mg; ++mi) order.push_back(id(mi, ni, ki));
     for (int ni = w; ni < Ng; ++ni)
@@ -28,7 +40,8 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
         for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
   } else {
     w = std::min(w, Mg);
-    for (int ki = 0; ki < Kg; ++ki)
+    if (w > 0 && Kg > 0) first_step_in_shells(w, Ng);
+    for (int ki = 1; ki < Kg; ++ki)
       for (int mi = 0; mi < w; ++mi)
         for (int ni = 0; ni < Ng; ++ni) order.push_back(id(mi, ni, ki));
     for (int mi = w; mi < Mg; ++mi)

@@ -184,6 +184,25 @@ def test_reference_order_is_index_order(pkg):
     assert got == list(itertools.product(range(2), range(3), range(4)))  # mi*Ng*Kg + ni*Kg + ki (dgemm.cpp:139-142)
 
 
+def test_panel_starts_in_growing_squares(pkg):
+    """First k-step of a panel order: after n fetched tiles the subkernels that can run must grow like a square, not
+    one per fetch.  8 x 8 x 8 tiles, panel of 5 column tiles (order 5): the subkernels launched before the i-th fetch
+    of the first k-step."""
+    rows, _ = pkg.plan_rows(16384, 16384, 16384, 2048, 1, 1, 1, 1, 8, 2, 0, 5)
+    first = [(r["mi"], r["ni"]) for r in rows if r["kind"] == GEMM and r["ki"] == 0][:40]
+    assert first[:9] == [(0, 0), (0, 1), (1, 0), (1, 1), (0, 2), (1, 2), (2, 0), (2, 1), (2, 2)]
+    assert sorted(first) == sorted(itertools.product(range(8), range(5)))     # the whole 8 x 5 panel, once each
+    fetches_before = []
+    n_fetch = 0
+    for r in rows:
+        if r["kind"] in (0, 1):
+            n_fetch += 1
+        elif r["kind"] == GEMM and r["ki"] == 0 and r["ni"] < 5:
+            fetches_before.append(n_fetch)
+    # 2 tiles -> 1 subkernel, 4 -> 4, 6 -> 9, 8 -> 16, 10 -> 25 (5 x 5), then one fetched A tile per 5 subkernels
+    assert [fetches_before[i] for i in (0, 3, 8, 15, 24, 29, 39)] == [2, 4, 6, 8, 10, 11, 13]
+
+
 def test_pipeline_simulation(pkg, L):
     import ctypes as C
     busy = (C.c_double * 3)()
