@@ -153,6 +153,11 @@ int PARALiA_stream_rotation(int* rotation, int* settled);
 /* directory holding Processed/ lookup tables and link models (DEPLOYDB, CMakeLists.txt:376) */
 int PARALiA_set_db_dir(const char* dir);
 
+/* cols runs of width_bytes, run c at dst + c*dst_pitch <- src + c*src_pitch, split over `threads` host threads.  The
+ * gather / scatter step of the pinned bounce buffers that stand in for the reference's pinning of pageable operands
+ * (prepareAsync, dgemm.cpp:413-416). */
+int PARALiA_host_copy2d(void* dst, long dst_pitch, const void* src, long src_pitch, long width_bytes, long cols, int threads);
+
 /* ---- driver helper surface (CoCoMalloc / CoCoFree / CoCoVecInit / Dtest_equality, dgemm_runner.cpp:55-99) ---- */
 int PARALiA_malloc(void** ptr, long long bytes, int loc);
 int PARALiA_free(void* ptr, int loc);

@@ -74,6 +74,7 @@ _SIGS = {
     "PARALiA_dgemv": (_i, [_c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _l, _ll, C.POINTER(atc_info)]),
     "PARALiA_daxpy": (_i, [_l, _d, _vp, _l, _vp, _l, _l, C.POINTER(atc_info)]),
     "PARALiA_ddot": (_i, [_l, _vp, _l, _vp, _l, C.POINTER(_d), _l, C.POINTER(atc_info)]),
+    "PARALiA_host_copy2d": (_i, [_vp, _l, _vp, _l, _l, _l, _i]),
     "PARALiA_dev_cache_free": (_i, [_i]),
     "PARALiA_runtime_stats": (_i, [C.POINTER(_l), C.POINTER(_l), C.POINTER(_ll), C.POINTER(_l)]),
     "PARALiA_runtime_reset": (_i, []),

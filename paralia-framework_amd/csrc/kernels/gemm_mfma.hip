@@ -25,6 +25,12 @@
 #ifndef PLK_WAVES_PER_EU
 #define PLK_WAVES_PER_EU 2
 #endif
+#ifndef PLK_F32_BK
+#define PLK_F32_BK 32
+#endif
+#ifndef PLK_F32_WAVES_PER_EU
+#define PLK_F32_WAVES_PER_EU 2
+#endif
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
 #endif
@@ -45,6 +51,7 @@ template <> struct Traits<double> {
   using acc_t = double4_t;
   static constexpr int VEC = 2;      // elements per 16-byte vector
   static constexpr int BK = PLK_F64_BK;  // k-panel depth
+  static constexpr int WAVES = PLK_WAVES_PER_EU;  // wavefronts per SIMD the register budget is sized for
   static constexpr int BLK = 16;     // MFMA block edge
   static constexpr int KSTEP = 4;    // k consumed per MFMA
   static constexpr int NACC = 4;     // accumulator elements per lane per block
@@ -62,12 +69,13 @@ template <> struct Traits<float> {
   using vec_t = fvec4;
   using acc_t = float16_t;
   static constexpr int VEC = 4;
-  static constexpr int BK = 32;
+  static constexpr int BK = PLK_F32_BK;
+  static constexpr int WAVES = PLK_F32_WAVES_PER_EU;
   static constexpr int BLK = 32;
   static constexpr int KSTEP = 2;
   static constexpr int NACC = 16;
   static constexpr int S_MN = 160;   // 640 B = 128 mod 256
-  static constexpr int S_K = 36;     // 144 B
+  static constexpr int S_K = BK + 4;  // 144 B at BK = 32
   static constexpr int NV = 128 * BK / VEC / 256;
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -172,7 +180,7 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
 template <typename T, bool AK, bool BKM>
-__global__ __launch_bounds__(NTHREADS, PLK_WAVES_PER_EU) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
+__global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
                                                           long ldc, int gm, int gn, int vecA, int vecB) {
   using Tr = Traits<T>;

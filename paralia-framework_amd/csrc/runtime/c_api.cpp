@@ -8,6 +8,7 @@
 #include "PARALiA.hpp"
 #include "backend_wrappers.hpp"
 #include "gemm_plan.hpp"
+#include "host_staging.hpp"
 #include "paralia_hip.h"
 
 namespace paralia {
@@ -105,6 +106,15 @@ int PARALiA_ddot(long N, double* x, long incx, double* y, long incy, double* res
     std::unique_ptr<ATC> predef(make_predef(T, 0));
     std::unique_ptr<ATC> out(paralia::ddot_impl(N, x, incx, y, incy, result, predef.get()));
     fill_info(info, out.get());
+  });
+}
+// The multi-threaded strided host copy that gathers / scatters tiles of pageable operands (host_staging.hpp).
+int PARALiA_host_copy2d(void* dst, long dst_pitch, const void* src, long src_pitch, long width_bytes, long cols, int threads) {
+  return guarded([&] {
+    if (!dst || !src || dst_pitch < width_bytes || src_pitch < width_bytes || width_bytes < 0 || cols < 0 || threads < 1)
+      throw paralia_error(PL_ERR_ARG, "PARALiA_host_copy2d: invalid argument\n");
+    paralia::CopyThreads pool(threads);
+    pool.copy2d(dst, (size_t)dst_pitch, src, (size_t)src_pitch, (size_t)width_bytes, cols);
   });
 }
 int PARALiA_dev_cache_free(int dev_id) {

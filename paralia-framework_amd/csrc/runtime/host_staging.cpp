@@ -1,0 +1,167 @@
+// Pinned bounce buffers and copy threads for pageable host operands; see host_staging.hpp.
+#include "host_staging.hpp"
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+#include "backend_wrappers.hpp"
+#include "paralia_hip.h"
+
+namespace paralia {
+
+namespace {
+void chk(int rc, const char* what) {
+  if (rc != 0) throw paralia_error(rc, std::string(what) + " failed: " + (rc == PL_ERR_HIP ? pl_last_error() : "invalid argument"));
+}
+}  // namespace
+
+CopyThreads::CopyThreads(int nthreads) {
+  for (int i = 1; i < nthreads; ++i) workers_.emplace_back([this] { worker(); });
+}
+
+CopyThreads::~CopyThreads() {
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    stop_ = true;
+    ++generation_;
+  }
+  cv_start_.notify_all();
+  for (std::thread& t : workers_) t.join();
+}
+
+void CopyThreads::run_chunks() {
+  const Job j = job_;  // stable while a generation runs
+  for (;;) {
+    const long c0 = next_.fetch_add(j.chunk);
+    if (c0 >= j.cols) break;
+    const long c1 = std::min(j.cols, c0 + j.chunk);
+    if (j.dst_pitch == j.width && j.src_pitch == j.width) {
+      memcpy(j.dst + (size_t)c0 * j.width, j.src + (size_t)c0 * j.width, (size_t)(c1 - c0) * j.width);
+    } else {
+      for (long c = c0; c < c1; ++c) memcpy(j.dst + (size_t)c * j.dst_pitch, j.src + (size_t)c * j.src_pitch, j.width);
+    }
+  }
+}
+
+void CopyThreads::worker() {
+  long seen = 0;
+  for (;;) {
+    {
+      std::unique_lock<std::mutex> lk(mu_);
+      cv_start_.wait(lk, [&] { return generation_ != seen; });
+      seen = generation_;
+      if (stop_) return;
+    }
+    run_chunks();
+    {
+      std::lock_guard<std::mutex> lk(mu_);
+      if (--running_ == 0) cv_done_.notify_one();
+    }
+  }
+}
+
+void CopyThreads::copy2d(void* dst, size_t dst_pitch, const void* src, size_t src_pitch, size_t width_bytes, long cols) {
+  if (cols <= 0 || width_bytes == 0) return;
+  const int n = threads();
+  {
+    std::lock_guard<std::mutex> lk(mu_);
+    job_.dst = (char*)dst; job_.src = (const char*)src;
+    job_.dst_pitch = dst_pitch; job_.src_pitch = src_pitch; job_.width = width_bytes; job_.cols = cols;
+    // chunks of at least 256 KiB, a few per thread so that a slow thread does not hold everyone up
+    const long by_size = (long)std::max<size_t>(1, (256u << 10) / width_bytes);
+    job_.chunk = std::max(by_size, (cols + 4L * n - 1) / (4L * n));
+    next_.store(0);
+    running_ = (int)workers_.size();
+    ++generation_;
+  }
+  cv_start_.notify_all();
+  run_chunks();  // the caller works too
+  std::unique_lock<std::mutex> lk(mu_);
+  cv_done_.wait(lk, [&] { return running_ == 0; });
+}
+
+HostStager::~HostStager() {
+  try { release(); } catch (...) {}
+  delete pool_;
+}
+
+CopyThreads* HostStager::threads() {
+  if (!pool_) {
+    const char* env = getenv("PARALIA_COPY_THREADS");
+    int n = env && atoi(env) > 0 ? atoi(env) : (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()));
+    pool_ = new CopyThreads(std::min(n, 64));
+  }
+  return pool_;
+}
+
+void HostStager::release() {
+  for (int s = 0; s < SLOTS; ++s) {
+    if (in_[s]) pl_free_pinned(in_[s]);
+    if (out_[s]) pl_free_pinned(out_[s]);
+    if (in_ev_[s]) pl_event_destroy(in_ev_[s]);
+    if (out_ev_[s]) pl_event_destroy(out_ev_[s]);
+    in_[s] = out_[s] = nullptr;
+    in_ev_[s] = out_ev_[s] = nullptr;
+    in_used_[s] = false;
+    pending_[s] = Pending();
+  }
+  slot_bytes_ = 0;
+}
+
+void HostStager::reserve(long long tile_bytes) {
+  if (tile_bytes <= slot_bytes_) return;
+  finish();
+  for (int s = 0; s < SLOTS; ++s)
+    if (in_used_[s]) chk(pl_event_sync(in_ev_[s]), "event sync");
+  release();
+  for (int s = 0; s < SLOTS; ++s) {
+    void* p = nullptr;
+    chk(pl_malloc_pinned(&p, tile_bytes), "pinned staging allocation");
+    in_[s] = (char*)p;
+    chk(pl_malloc_pinned(&p, tile_bytes), "pinned staging allocation");
+    out_[s] = (char*)p;
+    chk(pl_event_create(&in_ev_[s], 0), "event create");
+    chk(pl_event_create(&out_ev_[s], 0), "event create");
+  }
+  slot_bytes_ = tile_bytes;
+}
+
+void HostStager::fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream) {
+  if (rows <= 0 || cols <= 0) return;
+  const long long bytes = (long long)rows * cols * elem;
+  reserve(bytes);
+  const int s = (int)(in_next_++ % SLOTS);
+  if (in_used_[s]) chk(pl_event_sync(in_ev_[s]), "event sync");  // the slot's previous tile has left for the device
+  threads()->copy2d(in_[s], (size_t)rows * elem, src, (size_t)ld_src * elem, (size_t)rows * elem, cols);
+  chk(pl_copy_async(dst, in_[s], bytes, stream), "staged tile copy");
+  chk(pl_event_record(in_ev_[s], stream), "event record");
+  in_used_[s] = true;
+}
+
+void HostStager::flush(int s) {
+  Pending& p = pending_[s];
+  if (!p.active) return;
+  chk(pl_event_sync(out_ev_[s]), "event sync");
+  threads()->copy2d(p.dst, (size_t)p.ld * p.elem, out_[s], (size_t)p.rows * p.elem, (size_t)p.rows * p.elem, p.cols);
+  p.active = false;
+}
+
+void HostStager::write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream) {
+  if (rows <= 0 || cols <= 0) return;
+  const long long bytes = (long long)rows * cols * elem;
+  reserve(bytes);
+  const int s = (int)(out_next_++ % SLOTS);
+  flush(s);
+  chk(pl_copy_async(out_[s], src, bytes, stream), "staged tile copy");
+  chk(pl_event_record(out_ev_[s], stream), "event record");
+  Pending& p = pending_[s];
+  p.dst = dst; p.ld = ld_dst; p.rows = rows; p.cols = cols; p.elem = elem; p.active = true;
+}
+
+void HostStager::finish() {
+  for (int i = 0; i < SLOTS; ++i) flush((int)((out_next_ + i) % SLOTS));  // oldest first
+}
+
+}  // namespace paralia

@@ -1,0 +1,86 @@
+// Staging of pageable (not pinned) host operands.
+//
+// The reference pins whatever host memory it is given (cudaHostRegister in the operands' prepareAsync,
+// Library_scheduler/src/Functions/dgemm.cpp:413-416) so that every tile copy runs at the pinned rate.  Registering
+// existing memory is not available to this runtime, and a strided 2-D copy straight from pageable memory runs at
+// about 1 GB/s.  So tiles of pageable operands travel through a small ring of pinned bounce buffers: worker threads
+// gather a tile (strided rows -> dense) into a pinned slot, one contiguous asynchronous copy moves it to the device,
+// and the reverse for results.  Pure host logic apart from the C ABI calls; no HIP header.
+#ifndef PARALIA_HOST_STAGING_HPP
+#define PARALIA_HOST_STAGING_HPP
+
+#include <atomic>
+#include <condition_variable>
+#include <cstddef>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+namespace paralia {
+
+// Fixed pool of worker threads running one strided 2-D memcpy at a time, split by columns.
+class CopyThreads {
+ public:
+  explicit CopyThreads(int nthreads);
+  ~CopyThreads();
+  CopyThreads(const CopyThreads&) = delete;
+  CopyThreads& operator=(const CopyThreads&) = delete;
+  // cols runs of width_bytes each, run c at dst + c*dst_pitch  <-  src + c*src_pitch.  Returns when all are copied.
+  void copy2d(void* dst, size_t dst_pitch, const void* src, size_t src_pitch, size_t width_bytes, long cols);
+  int threads() const { return (int)workers_.size() + 1; }
+
+ private:
+  struct Job {
+    char* dst = nullptr;
+    const char* src = nullptr;
+    size_t dst_pitch = 0, src_pitch = 0, width = 0;
+    long cols = 0, chunk = 1;
+  };
+  void worker();
+  void run_chunks();
+  std::vector<std::thread> workers_;
+  std::mutex mu_;
+  std::condition_variable cv_start_, cv_done_;
+  Job job_;
+  std::atomic<long> next_{0};
+  long generation_ = 0;
+  int running_ = 0;
+  bool stop_ = false;
+};
+
+// Ring of pinned slots for tiles on their way to the device, and a second ring for tiles coming back.
+class HostStager {
+ public:
+  HostStager() = default;
+  ~HostStager();
+  HostStager(const HostStager&) = delete;
+  HostStager& operator=(const HostStager&) = delete;
+  // dst (device, dense, leading dimension = rows)  <-  src (pageable host, leading dimension ld_src), on `stream`.
+  void fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream);
+  // dst (pageable host, leading dimension ld_dst)  <-  src (device, dense) on `stream`; the host-side scatter happens
+  // when the slot is needed again or in finish().
+  void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream);
+  // Completes every pending scatter.  Call after the streams were synchronised.
+  void finish();
+  // Sizes the slots for tiles of up to tile_bytes (waits for tiles in flight and reallocates when they must grow).
+  void reserve(long long tile_bytes);
+  void release();
+
+ private:
+  static constexpr int SLOTS = 4;
+  struct Pending { void* dst = nullptr; long ld = 0, rows = 0, cols = 0; int elem = 0; bool active = false; };
+  void flush(int slot);
+  CopyThreads* threads();
+  char* in_[SLOTS] = {nullptr};
+  char* out_[SLOTS] = {nullptr};
+  void* in_ev_[SLOTS] = {nullptr};
+  void* out_ev_[SLOTS] = {nullptr};
+  bool in_used_[SLOTS] = {false};
+  Pending pending_[SLOTS];
+  long long slot_bytes_ = 0;
+  long in_next_ = 0, out_next_ = 0;
+  CopyThreads* pool_ = nullptr;
+};
+
+}  // namespace paralia
+#endif

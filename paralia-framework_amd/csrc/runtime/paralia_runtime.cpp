@@ -17,6 +17,7 @@
 #include "PARALiA.hpp"
 #include "backend_wrappers.hpp"
 #include "gemm_plan.hpp"
+#include "host_staging.hpp"
 #include "paralia_hip.h"
 
 namespace paralia {
@@ -58,6 +59,8 @@ struct Resources {
   void* exec[MAX_EXEC_QUEUES] = {nullptr};
   int nexec = 0;
   std::vector<void*> events;
+  std::unique_ptr<HostStager> stager_;  // pinned bounce buffers for pageable host operands, created on first use
+  HostStager& stager() { if (!stager_) stager_.reset(new HostStager()); return *stager_; }
   double* dot_ws = nullptr;      // ddot partials
   double* dot_result = nullptr;  // device scalar
   double* dot_host = nullptr;    // pinned scalar
@@ -152,6 +155,7 @@ struct Resources {
     if (dot_ws) pl_free_device(dot_ws);
     if (dot_host) pl_free_pinned(dot_host);
     gemv_x.release(); gemv_y.release(); gemv_ws.release();
+    stager_.reset();
     *this = Resources();
   }
 };
@@ -227,7 +231,7 @@ template <> struct GemmFns<float> {
 
 template <typename T>
 static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb, T alpha, const T* A, long lda, const T* B,
-                              long ldb, T beta, T* C, long ldc) {
+                              long ldb, T beta, T* C, long ldc, const bool pageable[3]) {
   const GemmProblem& p = plan.p;
   const bool at = (ta == 'T'), bt = (tb == 'T');
   const long Tt = p.T;
@@ -237,6 +241,10 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   R.res.ensure_events(nsig);
   std::vector<void*> ev(plan.cmds.size(), nullptr);
   size_t next_ev = 0;
+  // tiles of pageable operands go through pinned bounce buffers (a strided copy straight from pageable memory
+  // runs at about 1 GB/s)
+  HostStager& stager = R.res.stager();
+  if (pageable[0] || pageable[1] || pageable[2]) stager.reserve((long long)Tt * Tt * (long long)sizeof(T));
 
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
@@ -246,17 +254,20 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       case CMD_FETCH_A: {
         const long rows = at ? p.tk(c.ki) : p.tm(c.mi), cols = at ? p.tm(c.mi) : p.tk(c.ki);
         const T* src = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda;
-        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, lda, rows, cols, sizeof(T), s), "fetch A tile");
+        if (pageable[0]) stager.fetch(R.pool.at(c.block), src, lda, rows, cols, sizeof(T), s);
+        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, lda, rows, cols, sizeof(T), s), "fetch A tile");
       } break;
       case CMD_FETCH_B: {
         const long rows = bt ? p.tn(c.ni) : p.tk(c.ki), cols = bt ? p.tk(c.ki) : p.tn(c.ni);
         const T* src = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb;
-        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
+        if (pageable[1]) stager.fetch(R.pool.at(c.block), src, ldb, rows, cols, sizeof(T), s);
+        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
       } break;
       case CMD_FETCH_C: {
         const long rows = p.tm(c.mi), cols = p.tn(c.ni);
         const T* src = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
-        chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
+        if (pageable[2]) stager.fetch(R.pool.at(c.block), src, ldc, rows, cols, sizeof(T), s);
+        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
       } break;
       case CMD_GEMM: {
         const long m = p.tm(c.mi), n = p.tn(c.ni), k = p.tk(c.ki);
@@ -285,7 +296,8 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       case CMD_WRITEBACK: {
         const long m = p.tm(c.mi), n = p.tn(c.ni);
         T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
-        chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
+        if (pageable[2]) stager.write_back(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s);
+        else chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
       } break;
     }
     if (c.signals) {
@@ -294,6 +306,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
     }
   }
   R.res.sync_all();
+  stager.finish();
 }
 
 template <typename T>
@@ -406,7 +419,8 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab && !cold;
     if (trial) R.res.begin_trial();
     const double t0 = csecond();
-    execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC);
+    const bool pageable[3] = {locA == -2, locB == -2, locC == -2};
+    execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC, pageable);
     if (trial) R.res.end_trial((csecond() - t0) / (2.0 * M * N * (double)K));
   }
   return atc_copy(atc);
@@ -702,7 +716,8 @@ ATC_p dgemv_impl(char TransA, long M, long N, double alpha, double* A, long ldA,
       void* ev_ex = R.res.events[2 + 2 * r];
       double* Ad = (double*)R.pool.at(r);
       if (t >= ring) chk(pl_stream_wait_event(s_in, ev_ex), "stream wait event");  // the slot's previous tile was consumed
-      chk(pl_copy2d_async(Ad, tm, A + mi * T + ni * T * ldA, ldA, tm, tn, 8, s_in), "fetch A tile");
+      if (locA == -2) R.res.stager().fetch(Ad, A + mi * T + ni * T * ldA, ldA, tm, tn, 8, s_in);
+      else chk(pl_copy2d_async(Ad, tm, A + mi * T + ni * T * ldA, ldA, tm, tn, 8, s_in), "fetch A tile");
       chk(pl_event_record(ev_in, s_in), "event record");
       chk(pl_stream_wait_event(s_ex, ev_in), "stream wait event");
       // tile (mi, ni) multiplies the x tile of its reduction index into the y tile of its output index

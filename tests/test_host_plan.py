@@ -250,3 +250,21 @@ def test_pipeline_simulation_link_contention(pkg, L):
     a = L.PARALiA_gemm_plan_simulate(*args3, 4, *base, 1.0, 1.0, None, None)
     b = L.PARALiA_gemm_plan_simulate(*args3, 4, *base, 1.2, 1.2, None, None)
     assert a <= b < a * 1.03
+
+
+@pytest.mark.parametrize("threads", [1, 3, 8])
+@pytest.mark.parametrize("rows,cols,ld", [(1, 1, 1), (37, 91, 50), (2048, 300, 2048), (1000, 1, 4000), (5, 4000, 9)])
+def test_host_copy2d_gather_and_scatter(L, threads, rows, cols, ld):
+    """The threaded strided host copy behind the pageable-operand path: gather a sub-matrix into a dense tile and
+    scatter it back; bytes outside the sub-matrix must stay untouched."""
+    import numpy as np
+    rng = np.random.default_rng(rows * cols + threads)
+    src = rng.random(ld * cols)
+    dense = np.full(rows * cols, -1.0)
+    assert L.PARALiA_host_copy2d(dense.ctypes.data, rows * 8, src.ctypes.data, ld * 8, rows * 8, cols, threads) == 0
+    assert np.array_equal(dense.reshape(cols, rows), src.reshape(cols, ld)[:, :rows])
+    back = np.full(ld * cols, -2.0)
+    assert L.PARALiA_host_copy2d(back.ctypes.data, ld * 8, dense.ctypes.data, rows * 8, rows * 8, cols, threads) == 0
+    assert np.array_equal(back.reshape(cols, ld)[:, :rows], src.reshape(cols, ld)[:, :rows])
+    assert np.all(back.reshape(cols, ld)[:, rows:] == -2.0)
+    assert L.PARALiA_host_copy2d(back.ctypes.data, rows * 8 - 1, dense.ctypes.data, rows * 8, rows * 8, cols, threads) != 0
