@@ -65,6 +65,15 @@ void CopyThreads::worker() {
 void CopyThreads::copy2d(void* dst, size_t dst_pitch, const void* src, size_t src_pitch, size_t width_bytes, long cols) {
   if (cols <= 0 || width_bytes == 0) return;
   const int n = threads();
+  constexpr size_t PIECE = 256u << 10;
+  if (cols == 1 && width_bytes >= 4 * PIECE) {
+    // one long run (a vector): cut it into pieces the threads can share, the remainder is copied here
+    const long pieces = (long)(width_bytes / PIECE);
+    copy2d(dst, PIECE, src, PIECE, PIECE, pieces);
+    const size_t done = (size_t)pieces * PIECE;
+    if (done < width_bytes) memcpy((char*)dst + done, (const char*)src + done, width_bytes - done);
+    return;
+  }
   {
     std::lock_guard<std::mutex> lk(mu_);
     job_.dst = (char*)dst; job_.src = (const char*)src;

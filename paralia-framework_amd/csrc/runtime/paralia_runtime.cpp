@@ -473,6 +473,8 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
   R.res.ensure_streams(1);
   R.res.ensure_events(3 * (size_t)ring);
   void* s_in = R.res.h2d; void* s_ex = R.res.exec[0]; void* s_out = R.res.d2h;
+  HostStager& stager = R.res.stager();
+  if (locx == -2 || locy == -2) stager.reserve(blk);
   std::vector<void*> ev_in(ring), ev_ex(ring), ev_out(ring);
   for (int r = 0; r < ring; ++r) { ev_in[r] = R.res.events[3 * r]; ev_ex[r] = R.res.events[3 * r + 1]; ev_out[r] = R.res.events[3 * r + 2]; }
   for (long t = 0; t < tiles; ++t) {
@@ -489,8 +491,9 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
     if (t >= ring) {  // the ring slot is free once its previous tenant has been consumed / written back
       chk(pl_stream_wait_event(s_in, (write_y && ry) ? ev_out[r] : ev_ex[r]), "stream wait event");
     }
-    if (rx) chk(pl_copy_async(xd, xs, bx, s_in), "fetch x tile");
-    if (ry) chk(pl_copy_async(yd, ys, by, s_in), "fetch y tile");
+    // pageable vectors go through the pinned bounce buffers like matrix tiles do (a span is one long column)
+    if (rx) { if (locx == -2) stager.fetch(xd, xs, bx / 8, bx / 8, 1, 8, s_in); else chk(pl_copy_async(xd, xs, bx, s_in), "fetch x tile"); }
+    if (ry) { if (locy == -2) stager.fetch(yd, ys, by / 8, by / 8, 1, 8, s_in); else chk(pl_copy_async(yd, ys, by, s_in), "fetch y tile"); }
     if (rx || ry) {
       chk(pl_event_record(ev_in[r], s_in), "event record");
       chk(pl_stream_wait_event(s_ex, ev_in[r]), "stream wait event");
@@ -499,11 +502,13 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
     chk(pl_event_record(ev_ex[r], s_ex), "event record");
     if (write_y && ry) {
       chk(pl_stream_wait_event(s_out, ev_ex[r]), "stream wait event");
-      chk(pl_copy_async(ys, yd, by, s_out), "write back y tile");
+      if (locy == -2) stager.write_back(ys, by / 8, yd, by / 8, 1, 8, s_out);
+      else chk(pl_copy_async(ys, yd, by, s_out), "write back y tile");
       chk(pl_event_record(ev_out[r], s_out), "event record");
     }
   }
   R.res.sync_all();
+  stager.finish();
 }
 
 static void blas1_common_checks(const char* routine, long N, double* x, long incx, double* y, long incy, int* locx, int* locy) {
