@@ -330,17 +330,24 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       const Modeler* m = unit_modeler_list[0];
       long best_T = -1, prev = -1;
       double best_t = DBL_MAX;
-      for (long i = 0; i < m->exec->lines(); i++) {
+      // Largest tiles first: they have few subkernels and are cheap to simulate, and once a good makespan is known
+      // the small tiles, whose kernels alone already take longer than that, are dismissed without building a plan.
+      for (long i = m->exec->lines() - 1; i >= 0; i--) {
         const long cand = m->exec->T[i];
         if (cand == prev) continue;
         prev = cand;
         // tiles may be shallower than T in K (depth min(T, K)), so only M and N bound the candidates
         if (cand > std::min(problem.D1, problem.D2)) continue;
+        // MinAllowedTBLAS3 (ModelLvl3.cpp): tiles below 1024 are not considered when the problem is larger than that
+        if (cand < m->getMinT() && std::min(problem.D1, problem.D2) >= m->getMinT()) continue;
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         if (gp.pool_blocks < 3 || gp.subkernels() > 20000) continue;
+        const paralia::StageTimes st = paralia_stage_times(this, cand);
+        if (best_T > 0 && (double)gp.subkernels() * st.exec_time(cand, std::min(cand, problem.D1), std::min(cand, problem.D2),
+                                                                   std::min(cand, problem.D3)) * 0.9 > best_t) continue;
         paralia::PipelineResult r;
         try {
-          paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
+          paralia::pick_gemm_order(gp, st, &r);
         } catch (const std::runtime_error&) { continue; }
         // predictions of neighbouring T differ by less than the model's accuracy: the reference's penalty terms
         // (ragged edges, too few or too many subkernels, Autotuner.cpp:571-603) break such near-ties
@@ -350,7 +357,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
           get_T_slowdowns(sl, (int)cand);
           score *= 1.0 + 0.02 * sl[0];
         }
-        if (score < best_t) { best_t = score; best_T = cand; }
+        if (score <= best_t) { best_t = score; best_T = cand; }  // ties go to the smaller tile
       }
       if (best_T < 0) {
         // C narrower than every benchmarked tile: one tile across the short side, as square as that allows

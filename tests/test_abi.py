@@ -57,3 +57,34 @@ def test_csv_row_round_trip(pkg, L, tmp_path):
     line = "2048,1,1,0, N,N,1.00000,0.00000,16384,16384,16384,-1,-1,-1,-1, 1.300000e-01,1.250000e-01,-1.000000e+00\n"
     parts = [p.strip() for p in line.split(",")]
     assert len(parts) == 18 and parts[0] == "2048" and parts[4] == "N" and float(parts[15]) == 0.13
+
+
+def test_predictor_driver_emits_a_runner_row(pkg, tmp_path):
+    """dgemm_predictor needs no GPU: it parses the reference's 15 driver arguments (testing.cpp:273-329), autotunes and
+    appends one row in the runner log format (testing.cpp:424) whose first four columns are T, unit count, unit token
+    and cache limit (ATC::print_csv)."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(pkg.LIB_PATH), "..", "bin", "dgemm_predictor")
+    if not os.path.exists(exe):
+        pytest.skip("driver executables not built")
+    env = dict(os.environ, PARALIA_TESTLIBDIR=str(tmp_path))
+    args = "-1 -1 -1 -1 N N 1.0 0.0 16384 16384 16384 -1 -1 -1 -1".split()
+    run = subprocess.run([exe] + args, env=env, capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stderr
+    logs = list(tmp_path.glob("CoCoPeLiaDgemmPredictor_MI355X_*.log"))
+    assert len(logs) == 1
+    parts = [p.strip() for p in logs[0].read_text().strip().split(",")]
+    assert len(parts) == 18
+    assert parts[:4] == ["2048", "1", "1", "0"] and parts[4:6] == ["N", "N"]
+    assert [int(p) for p in parts[8:15]] == [16384, 16384, 16384, -1, -1, -1, -1]
+    assert 0.1 < float(parts[16]) < 0.15            # predicted seconds for 16384^3 streamed from the host
+    assert "T =  2048" in run.stderr and "pipeline-model" in run.stderr
+    # a preset tile goes to the other log and is kept
+    run = subprocess.run([exe] + "1 1 4096 -1 N N 1.0 0.0 16384 16384 16384 -1 -1 -1 -1".split(), env=env, capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stderr
+    row = next(tmp_path.glob("CoCoPeLiaDgemmPredictor_predefined_vals_MI355X_*.log")).read_text()
+    assert row.startswith("4096,1,1,")
+    # wrong argument count is the reference's usage error
+    run = subprocess.run([exe, "1", "2"], env=env, capture_output=True, text=True, timeout=60)
+    assert run.returncode != 0 and "Incorrect input arguments" in run.stderr
