@@ -101,6 +101,52 @@ def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks):
     return out
 
 
+def check_async_safety(rows):
+    """Every data hazard on a pool block is ordered by stream order plus the recorded waits (transitively): a reader
+    runs after the command that produced what it reads, and a command that overwrites a block runs after every
+    earlier reader and writer of that block.  Happens-before sets are bit masks."""
+    before = [0] * len(rows)
+    last_on_stream = {}
+    last_write = {}   # block -> command that last wrote it
+    users = {}        # block -> commands that read it since
+    for i, r in enumerate(rows):
+        deps = 0
+        if r["stream"] in last_on_stream:
+            j = last_on_stream[r["stream"]]
+            deps |= before[j] | (1 << j)
+        for w in r["waits"]:
+            deps |= before[w] | (1 << w)
+        before[i] = deps
+        last_on_stream[r["stream"]] = i
+        k = r["kind"]
+        reads, writes = [], []
+        if k in (FETCH_A, FETCH_B, FETCH_C):
+            writes = [r["block"]]
+        elif k == GEMM:
+            reads = [x for x in (r["a_block"], r["b_block"]) if x >= 0]
+            if r["block"] >= 0:
+                (writes if r["beta_mode"] == BETA_ZERO else reads).append(r["block"])
+                if r["beta_mode"] != BETA_ZERO:
+                    writes.append(r["block"])
+        elif k == REDUCE:
+            reads = [r["block"], r["a_block"]]
+            writes = [r["block"]]
+        elif k == WRITEBACK:
+            reads = [r["block"]]
+        for blk in reads:
+            w = last_write.get(blk)
+            assert w is not None, "cmd %d reads block %d that nothing wrote" % (i, blk)
+            assert w == i or (deps >> w) & 1, "cmd %d reads block %d before its writer %d is known to be done" % (i, blk, w)
+        for blk in writes:
+            for u in users.get(blk, []) + ([last_write[blk]] if blk in last_write else []):
+                assert u == i or (deps >> u) & 1, "block %d overwritten by cmd %d before cmd %d is known to be done" % (blk, i, u)
+        for blk in reads:
+            users.setdefault(blk, []).append(i)
+        for blk in writes:
+            last_write[blk] = i
+            users[blk] = []
+
+
 ORDERS = [10000, 0, 1, 3, 10002, 10004]
 
 
@@ -122,6 +168,7 @@ def test_plan_invariants_and_replay(pkg, order, locs, beta_zero):
     alpha, beta = 2.0, (0.0 if beta_zero else 3.0)
     got = replay(rows, M, N, K, T, alpha, beta, A, B, C, full)
     assert np.array_equal(got, alpha * (A @ B) + beta * C)
+    check_async_safety(rows)
 
 
 @pytest.mark.parametrize("pool", [3, 4, 7, 12])
@@ -139,34 +186,7 @@ def test_plan_with_eviction(pkg, pool, beta_zero):
     C = rng.integers(-5, 6, (M, N)).astype(np.float64)
     beta = 0.0 if beta_zero else -2.0
     assert np.array_equal(replay(rows, M, N, K, T, 1.0, beta, A, B, C, pool), A @ B + beta * C)
-    # asynchronous safety: every user of a block's previous tenant is ordered (transitively, through stream order
-    # and waits) before the command that overwrites the block
-    users = {}
-    order_before = [set() for _ in rows]
-    last_on_stream = {}
-    for i, r in enumerate(rows):
-        deps = set()
-        if r["stream"] in last_on_stream:
-            j = last_on_stream[r["stream"]]
-            deps |= order_before[j] | {j}
-        for w in r["waits"]:
-            deps |= order_before[w] | {w}
-        order_before[i] = deps
-        last_on_stream[r["stream"]] = i
-        writes = [r["block"]] if r["kind"] in (FETCH_A, FETCH_B, FETCH_C) or (r["kind"] == GEMM and r["beta_mode"] == BETA_ZERO) else []
-        for b in writes:
-            for u in users.get(b, []):
-                assert u in deps, "block %d overwritten by cmd %d before its user %d is known to be done" % (b, i, u)
-            users[b] = []
-        reads = []
-        if r["kind"] == GEMM:
-            reads = [x for x in (r["a_block"], r["b_block"], r["block"]) if x >= 0]
-        elif r["kind"] == REDUCE:
-            reads = [r["block"], r["a_block"]]
-        elif r["kind"] == WRITEBACK:
-            reads = [r["block"]]
-        for b in reads:
-            users.setdefault(b, []).append(i)
+    check_async_safety(rows)
 
 
 def test_plan_too_small_pool_is_an_error(pkg):
@@ -268,3 +288,35 @@ def test_host_copy2d_gather_and_scatter(L, threads, rows, cols, ld):
     assert np.array_equal(back.reshape(cols, ld)[:, :rows], src.reshape(cols, ld)[:, :rows])
     assert np.all(back.reshape(cols, ld)[:, rows:] == -2.0)
     assert L.PARALiA_host_copy2d(back.ctypes.data, rows * 8 - 1, dense.ctypes.data, rows * 8, rows * 8, cols, threads) != 0
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_plans_are_safe_and_correct(pkg, seed):
+    """Random shapes (ragged tiles, K = 0 and T larger than a dimension included), operand placements, order families
+    and pool sizes from the minimum to the full working set: every plan that builds must keep all invariants, replay to
+    the exact result and order every hazard; a plan that does not fit must say so."""
+    rng = np.random.default_rng(1000 + seed)
+    M, N = (int(x) for x in rng.integers(1, 200, 2))
+    K = int(rng.integers(0, 200))
+    T = int(rng.choice([16, 24, 32, 50, 64, 128, 256]))
+    a_r, b_r, c_r = (int(x) for x in rng.integers(0, 2, 3))
+    beta_zero = int(rng.integers(0, 2))
+    nq = int(rng.integers(1, 5))
+    Mg, Ng, Kg = grids(M, N, K, T)
+    full = 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
+    pool = int(rng.choice([0, 3, 4, 5, max(3, full // 3), max(3, full // 2), full]))
+    orient, w = int(rng.integers(0, 2)), int(rng.integers(0, max(Mg, Ng) + 2))
+    order = orient * 10000 + w
+    A = rng.integers(-4, 5, (M, K)).astype(np.float64)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float64)
+    C = rng.integers(-4, 5, (M, N)).astype(np.float64)
+    alpha, beta = 2.0, (0.0 if beta_zero else -3.0)
+    try:
+        rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, nq, pool, order)
+    except pkg.ParaliaError as e:
+        assert (a_r or b_r or c_r) and pool and pool < full and ("too small" in str(e) or "< 3 blocks" in str(e))
+        return
+    eff_pool = pool if pool else full
+    check_plan(rows, stats, M, N, K, T, a_r, b_r, c_r, beta_zero, eff_pool, nq)
+    assert np.array_equal(replay(rows, M, N, K, T, alpha, beta, A, B, C, eff_pool), alpha * (A @ B) + beta * C)
+    check_async_safety(rows)
