@@ -375,8 +375,10 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     d.beta_is_zero = key.beta_zero;
     const bool any_remote = key.loc[0] < 0 || key.loc[1] < 0 || key.loc[2] < 0;
     d.pool_budget_bytes = any_remote ? pool_budget(atc->cache_limit, R.pool.bytes()) : 0;
-    if (any_remote && atc->cache_limit > 0 && atc->T > 0 && atc->cache_limit < 3LL * atc->T * atc->T * (long long)sizeof(T))
-      error("PARALiA%s: Problem cannot run with less memory than %lld\n", GemmFns<T>::name, 3LL * atc->T * atc->T * (long long)sizeof(T));
+    // a preset tile larger than every dimension is the whole problem: the limit is judged on the tile that will be used
+    const long long t_eff = std::min<long long>(atc->T, std::max(M, std::max(N, K)));
+    if (any_remote && atc->cache_limit > 0 && atc->T > 0 && atc->cache_limit < 3LL * t_eff * t_eff * (long long)sizeof(T))
+      error("PARALiA%s: Problem cannot run with less memory than %lld\n", GemmFns<T>::name, 3LL * t_eff * t_eff * (long long)sizeof(T));
     // alpha == 0 or K == 0: C <- beta*C only, one "subkernel" per C tile with an empty K; K must not
     // constrain the tile choice then
     if (d.D3 == 0) d.D3 = std::min(M, N);

@@ -193,3 +193,32 @@ def test_routine_autotuned_call(pkg, L, orc, openblas):
     ref = y0.copy()
     openblas.orc_openblas_dgemv(b"N", M, N, 1.2, ptr(A), M, ptr(x), 1, 1.1, ptr(ref), 1)
     assert norm_err(by.get(), ref, 1.2, A, x, 1.1, y0) < TOL
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_gemv_cases(pkg, L, orc, openblas, seed):
+    """Random shapes, transposes, placements (device, pinned, pageable), tile sizes, increments of either sign, padded
+    leading dimension, alpha / beta including 0, against OpenBLAS."""
+    rng = np.random.default_rng(900 + seed)
+    M, N = (int(x) for x in rng.integers(1, 900, 2))
+    ta = str(rng.choice(["N", "T"]))
+    lda = M + int(rng.integers(0, 5))
+    incx, incy = (int(x) for x in rng.choice([1, 1, 2, -1, -3], 2))
+    alpha = float(rng.choice([0.0, 1.0, -0.75, 1.23]))
+    beta = float(rng.choice([0.0, 1.0, 0.5]))
+    locs = tuple(int(x) for x in rng.choice([-2, -1, 0], 3))
+    T = int(rng.choice([-1, 64, 100, 256, 2048]))
+    lx, ly = (N, M) if ta == "N" else (M, N)
+    A, x, y0 = rand_f64(lda * N, seed), rand_f64(span(lx, incx), seed + 100), rand_f64(span(ly, incy), seed + 200)
+    ref = y0.copy()
+    assert openblas.orc_openblas_dgemv(ta.encode(), M, N, alpha, ptr(A), lda, ptr(x), incx, beta, ptr(ref), incy) == 0
+    bA, bx, by = place(pkg, A, locs[0]), place(pkg, x, locs[1]), place(pkg, y0, locs[2])
+    call_gemv(pkg, L, ta, M, N, alpha, bA, lda, bx, incx, beta, by, incy, T=T)
+    got = by.get()
+    if alpha == 0.0 and beta == 0.0:
+        assert np.all(got[::abs(incy)] == 0)
+    else:
+        assert norm_err(got, ref, alpha, A, x, beta, y0) < TOL
+    gaps = np.ones(y0.size, dtype=bool)
+    gaps[::abs(incy)] = False
+    assert np.array_equal(got[gaps], y0[gaps])

@@ -285,3 +285,41 @@ def test_vec_init_matches_oracle_generator(pkg, L):
     b = Buf(pkg, n, np.float32, 0)
     pkg.check(L.PARALiA_vec_init_f32(b.ptr, n, 7, 0), "vec init f32")
     assert np.array_equal(b.get(), rand_f32(n, 7))
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_gemm_cases(pkg, L, orc, openblas, seed):
+    """Random shapes (1 .. 600, ragged tiles), transposes, operand placements (device, pinned, pageable), tile sizes
+    (autotuned or preset, also larger than a dimension), padded leading dimensions, alpha / beta including 0 and
+    block-pool limits below the working set, in fp64 and fp32, against OpenBLAS on the same seeded inputs."""
+    rng = np.random.default_rng(500 + seed)
+    dtype = np.float64 if seed % 3 else np.float32
+    gen = rand_f64 if dtype == np.float64 else rand_f32
+    M, N, K = (int(x) for x in rng.integers(1, 600, 3))
+    ta, tb = (str(x) for x in rng.choice(["N", "T"], 2))
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + int(rng.integers(0, 9)), rb + int(rng.integers(0, 9)), M + int(rng.integers(0, 9))
+    alpha = float(rng.choice([0.0, 1.0, -0.75, 1.23]))
+    beta = float(rng.choice([0.0, 1.0, 0.5, -1.1]))
+    locs = tuple(int(x) for x in rng.choice([-2, -1, 0], 3))
+    T = int(rng.choice([-1, 32, 64, 100, 128, 256, 1024]))
+    A, B, C0 = gen(lda * ca, 3 * seed), gen(ldb * cb, 3 * seed + 1), gen(ldc * N, 3 * seed + 2)
+    limit = 0
+    if T > 0 and min(locs) < 0 and rng.integers(0, 3) == 0:
+        limit = int(rng.integers(3, 9)) * min(T, max(M, N, K)) ** 2 * np.dtype(dtype).itemsize
+        L.PARALiA_dev_cache_free(0)
+    bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, C0, locs[2])
+    call_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, bA, lda, bB, ldb, bC, ldc, T=T, cache_limit=limit)
+    got = bC.get()
+    ref = openblas_ref(openblas, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    tol = TOL64 if dtype == np.float64 else TOL32
+    if alpha == 0.0 and beta == 0.0:
+        assert np.all(got.reshape(N, ldc)[:, :M] == 0)
+    else:
+        assert normwise(orc, dtype, got, ref, M, N, ldc, alpha, beta, A, ra, ca, lda, B, rb, cb, ldb, C0) < tol
+    pad = np.ones(ldc * N, dtype=bool)
+    pad.reshape(N, ldc)[:, :M] = False
+    assert np.array_equal(got[pad], C0[pad])
+    if limit:
+        L.PARALiA_dev_cache_free(0)
