@@ -323,3 +323,30 @@ def test_random_gemm_cases(pkg, L, orc, openblas, seed):
     assert np.array_equal(got[pad], C0[pad])
     if limit:
         L.PARALiA_dev_cache_free(0)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_blas1_cases(pkg, L, orc, seed):
+    """daxpy and ddot with random lengths, increments of either sign, placements (device, pinned, pageable) and 1-D
+    tile sizes: daxpy bit for bit against the oracle's fused multiply-add (gaps of strided vectors untouched), ddot
+    against the long-double sum."""
+    rng = np.random.default_rng(1300 + seed)
+    n = int(rng.integers(1, 300000))
+    incx, incy = (int(v) for v in rng.choice([1, 1, 2, 3, -1, -2], 2))
+    locs = tuple(int(v) for v in rng.choice([-2, -1, 0], 2))
+    T = int(rng.choice([-1, 1000, 4096, 65536, 1 << 20]))
+    alpha = float(rng.choice([0.0, 1.0, -1.5, 0.7]))
+    sx, sy = (n - 1) * abs(incx) + 1, (n - 1) * abs(incy) + 1
+    x, y0 = rand_f64(sx, 2 * seed), rand_f64(sy, 2 * seed + 1)
+    bx, by = place(pkg, x, locs[0]), place(pkg, y0, locs[1])
+    print("random blas1", n, incx, incy, locs, T, alpha, flush=True)
+    res = C.c_double(0.5)
+    pkg.check(L.PARALiA_ddot(n, bx.ptr, incx, by.ptr, incy, C.byref(res), T, None), "PARALiA_ddot")
+    exact = float(orc.orc_ddot_longdouble(n, ptr(x), incx, ptr(y0), incy))
+    bound = 1e-13 * float(np.linalg.norm(x[::abs(incx)]) * np.linalg.norm(y0[::abs(incy)])) + 1e-300
+    assert abs((res.value - 0.5) - exact) <= bound
+    pkg.check(L.PARALiA_daxpy(n, alpha, bx.ptr, incx, by.ptr, incy, T, None), "PARALiA_daxpy")
+    ref = y0.copy()
+    orc.orc_daxpy(n, alpha, ptr(x), incx, ptr(ref), incy)
+    assert np.array_equal(by.get(), ref)
+    assert np.array_equal(bx.get(), x)
