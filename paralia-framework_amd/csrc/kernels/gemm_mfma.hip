@@ -6,7 +6,7 @@
 // MFMA kernel:
 //   * one workgroup = 256 threads = 4 wavefronts (2 x 2), macro tile 128 x 128, each wave owns 64 x 64;
 //   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2);
-//   * A and B k-panels (16 doubles / 32 floats deep) are staged global -> registers -> LDS, double-buffered,
+//   * A and B k-panels (16 elements deep) are staged global -> registers -> LDS, double-buffered,
 //     one barrier per k-panel; the next panel's global loads are in flight while the current one is multiplied;
 //   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
@@ -26,7 +26,7 @@
 #define PLK_WAVES_PER_EU 2
 #endif
 #ifndef PLK_F32_BK
-#define PLK_F32_BK 32
+#define PLK_F32_BK 16
 #endif
 #ifndef PLK_F32_WAVES_PER_EU
 #define PLK_F32_WAVES_PER_EU 2
@@ -75,7 +75,7 @@ template <> struct Traits<float> {
   static constexpr int KSTEP = 2;
   static constexpr int NACC = 16;
   static constexpr int S_MN = 160;   // 640 B = 128 mod 256
-  static constexpr int S_K = BK + 4;  // 144 B at BK = 32
+  static constexpr int S_K = BK + 4;  // 80 B: rows 16-byte aligned, the 32 lanes of a block spread over all banks
   static constexpr int NV = 128 * BK / VEC / 256;
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -296,23 +296,49 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
           else if (slot < SIDE) gload_one<T, BKM>(gb, ldb, rb[slot - 3 * NV], tid, slot - 3 * NV);
         }
         mfma_step(am[ks & 1], bnv[ks & 1]);
-        // issue order inside the k-step: operand reads first, then one side instruction after every few MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
+        if (MFMAS >= 4 * NB) {
+          // many short MFMAs per k-step (fp64: 16): operand reads first, then one side instruction after every few MFMAs
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
 #pragma unroll
-        for (int q = 0; q < PER_STEP; ++q) {
-          const int slot = ks * PER_STEP + q;
-          __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / PER_STEP > 0 ? MFMAS / PER_STEP : 1, 0);
-          if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-          else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          for (int q = 0; q < PER_STEP; ++q) {
+            const int slot = ks * PER_STEP + q;
+            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / PER_STEP > 0 ? MFMAS / PER_STEP : 1, 0);
+            if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+        } else {
+          // few long MFMAs per k-step (fp32: 4 of 64 cycles): one operand read and one side instruction behind each
+          // MFMA, so that a wave issues them while its own MFMA occupies the pipe.  With everything in front of the
+          // MFMAs the two waves of a SIMD reach their non-MFMA stretch together and the pipe idles (130 -> 138 TFLOP/s).
+#pragma unroll
+          for (int m = 0; m < MFMAS; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (m < 2 * NB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            constexpr int SPM = (PER_STEP + MFMAS - 1) / MFMAS;  // side instructions per MFMA
+#pragma unroll
+            for (int q = m * SPM; q < (m + 1) * SPM && q < PER_STEP; ++q) {
+              const int slot = ks * PER_STEP + q;
+              if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+              else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+          }
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
       __syncthreads();
       read_ops(cur ^ 1, 0, am[KS & 1], bnv[KS & 1]);
       mfma_step(am[(KS - 1) & 1], bnv[(KS - 1) & 1]);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+      if (MFMAS >= 4 * NB) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+      } else {
+#pragma unroll
+        for (int m = 0; m < MFMAS; ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (m < 2 * NB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   } else {
