@@ -189,8 +189,10 @@ struct Runtime {
   long pmd_hits = 0, pmd_misses = 0;
 };
 static Runtime& rt() {
-  static Runtime r;
-  return r;
+  // never destroyed: at process exit the HIP runtime may already be gone, and freeing pinned buffers, events or
+  // streams from a static destructor would call into it
+  static Runtime* r = new Runtime();
+  return *r;
 }
 
 static int host_or_dev(int loc) { return loc >= 0 ? 0 : -1; }  // the scheduler routes by "on device 0" vs "host"
