@@ -96,7 +96,7 @@ def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL6
 def test_dgemm_16384_host_operands(pkg, L):
     """dgemm 16384^3, alpha = 1, beta = 0, all operands in pinned host memory, T picked by the autotuner."""
     info = check_gemm(pkg, L, np.float64, "N", "N", 16384, 16384, 16384, 1.0, 0.0, (-1, -1, -1))
-    assert info.subkernel_num == (16384 // info.T) ** 3
+    assert info.subkernel_num == (-(-16384 // info.T)) ** 3
 
 
 @pytest.mark.timeout(600)
