@@ -169,6 +169,10 @@ void HostStager::write_back(void* dst, long ld_dst, const void* src, long rows, 
   p.dst = dst; p.ld = ld_dst; p.rows = rows; p.cols = cols; p.elem = elem; p.active = true;
 }
 
+void HostStager::abandon() {
+  for (int s = 0; s < SLOTS; ++s) pending_[s].active = false;
+}
+
 void HostStager::finish() {
   for (int i = 0; i < SLOTS; ++i) flush((int)((out_next_ + i) % SLOTS));  // oldest first
 }

@@ -62,6 +62,8 @@ class HostStager {
   void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream);
   // Completes every pending scatter.  Call after the streams were synchronised.
   void finish();
+  // Forgets pending scatters without performing them: after a failed call their destinations may no longer be valid.
+  void abandon();
   // Sizes the slots for tiles of up to tile_bytes (waits for tiles in flight and reallocates when they must grow).
   void reserve(long long tile_bytes);
   void release();
@@ -80,6 +82,15 @@ class HostStager {
   long long slot_bytes_ = 0;
   long in_next_ = 0, out_next_ = 0;
   CopyThreads* pool_ = nullptr;
+};
+
+// Completes the staged write-backs on the normal path, drops them when the call unwinds with an error.
+struct StagerScope {
+  HostStager& stager;
+  bool finished = false;
+  explicit StagerScope(HostStager& s) : stager(s) {}
+  void finish() { stager.finish(); finished = true; }
+  ~StagerScope() { if (!finished) stager.abandon(); }
 };
 
 }  // namespace paralia

@@ -247,6 +247,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   // runs at about 1 GB/s)
   HostStager& stager = R.res.stager();
   if (pageable[0] || pageable[1] || pageable[2]) stager.reserve((long long)Tt * Tt * (long long)sizeof(T));
+  StagerScope staged(stager);
 
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
@@ -308,7 +309,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
     }
   }
   R.res.sync_all();
-  stager.finish();
+  staged.finish();
 }
 
 template <typename T>
@@ -479,6 +480,7 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
   void* s_in = R.res.h2d; void* s_ex = R.res.exec[0]; void* s_out = R.res.d2h;
   HostStager& stager = R.res.stager();
   if (locx == -2 || locy == -2) stager.reserve(blk);
+  StagerScope staged(stager);
   std::vector<void*> ev_in(ring), ev_ex(ring), ev_out(ring);
   for (int r = 0; r < ring; ++r) { ev_in[r] = R.res.events[3 * r]; ev_ex[r] = R.res.events[3 * r + 1]; ev_out[r] = R.res.events[3 * r + 2]; }
   for (long t = 0; t < tiles; ++t) {
@@ -512,7 +514,7 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
     }
   }
   R.res.sync_all();
-  stager.finish();
+  staged.finish();
 }
 
 static void blas1_common_checks(const char* routine, long N, double* x, long incx, double* y, long incy, int* locx, int* locy) {
