@@ -34,6 +34,8 @@ int main(const int argc, const char* argv[]) {
       const short locs[3] = {A_loc, B_loc, C_loc};
       for (int i = 0; i < 3; ++i) d.loc[i] = d.out_loc[i] = locs[i] >= 0 ? 0 : -1;
       d.beta_is_zero = beta == 0.0;
+      // no device is queried here: only an explicit limit bounds the block pool
+      if (predef_control_values && predef_control_values->cache_limit > 0) d.pool_budget_bytes = predef_control_values->cache_limit;
       (void)T_in;
       return d;
     };

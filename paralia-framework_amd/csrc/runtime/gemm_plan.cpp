@@ -13,40 +13,56 @@ namespace paralia {
 
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
-  const int orient = order_id / 10000;
+  order_id %= 40000;                       // the eviction policy does not change the order
+  const bool repeat = order_id >= 20000;  // every panel k-outer, not only the first
+  const int orient = (order_id % 20000) / 10000;
   int w = order_id % 10000;
   std::vector<int> order;
   order.reserve((size_t)Mg * Ng * Kg);
   auto id = [&](int mi, int ni, int ki) { return (mi * Ng + ni) * Kg + ki; };
-  // First k-step of a panel: walk the tiles in growing squares (shell d = max(mi, ni)), so that every newly fetched
-  // A or B tile at once enables a whole row or column of subkernels; column by column the first Mg fetches would
-  // enable one subkernel each while the compute streams starve.
-  auto first_step_in_shells = [&](int rows, int cols) {
+  // One panel of C tiles, rows [m0, m1) x columns [n0, n1), in k-outer order.  Its first k-step walks the tiles in
+  // growing squares (shell d = max(row, column) inside the panel), so that every newly fetched A or B tile at once
+  // enables a whole row or column of subkernels; column by column the first fetches would enable one subkernel each
+  // while the compute streams starve.
+  auto panel = [&](int m0, int m1, int n0, int n1) {
+    const int rows = m1 - m0, cols = n1 - n0;
+    if (rows <= 0 || cols <= 0 || Kg <= 0) return;
     for (int d = 0; d < std::max(rows, cols); ++d) {
       if (d < cols)
-        for (int mi = 0; mi < std::min(d, rows); ++mi) order.push_back(id(mi, d, 0));
+        for (int mi = 0; mi < std::min(d, rows); ++mi) order.push_back(id(m0 + mi, n0 + d, 0));
       if (d < rows)
-        for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(d, ni, 0));
+        for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(m0 + d, n0 + ni, 0));
+    }
+    for (int ki = 1; ki < Kg; ++ki) {
+      if (orient == 0) {
+        for (int ni = n0; ni < n1; ++ni)
+          for (int mi = m0; mi < m1; ++mi) order.push_back(id(mi, ni, ki));
+      } else {
+        for (int mi = m0; mi < m1; ++mi)
+          for (int ni = n0; ni < n1; ++ni) order.push_back(id(mi, ni, ki));
+      }
     }
   };
   if (orient == 0) {
     w = std::min(w, Ng);
-    if (w > 0 && Kg > 0) first_step_in_shells(Mg, w);
-    for (int ki = 1; ki < Kg; ++ki)
-      for (int ni = 0; ni < w; ++ni)
-        for (int mi = 0; mi < Mg; ++mi) order.push_back(id(mi, ni, ki));
-    for (int ni = w; ni < Ng; ++ni)
-      for (int mi = 0; mi < Mg; ++mi)
-        for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+    if (repeat) {
+      for (int n0 = 0; n0 < Ng; n0 += std::max(w, 1)) panel(0, Mg, n0, std::min(Ng, n0 + std::max(w, 1)));
+    } else {
+      panel(0, Mg, 0, w);
+      for (int ni = w; ni < Ng; ++ni)
+        for (int mi = 0; mi < Mg; ++mi)
+          for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+    }
   } else {
     w = std::min(w, Mg);
-    if (w > 0 && Kg > 0) first_step_in_shells(w, Ng);
-    for (int ki = 1; ki < Kg; ++ki)
-      for (int mi = 0; mi < w; ++mi)
-        for (int ni = 0; ni < Ng; ++ni) order.push_back(id(mi, ni, ki));
-    for (int mi = w; mi < Mg; ++mi)
-      for (int ni = 0; ni < Ng; ++ni)
-        for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+    if (repeat) {
+      for (int m0 = 0; m0 < Mg; m0 += std::max(w, 1)) panel(m0, std::min(Mg, m0 + std::max(w, 1)), 0, Ng);
+    } else {
+      panel(0, w, 0, Ng);
+      for (int mi = w; mi < Mg; ++mi)
+        for (int ni = 0; ni < Ng; ++ni)
+          for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+    }
   }
   return order;
 }
@@ -63,6 +79,18 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p) {
       if (w < g) ids.push_back(order_id_of(orient, w));
     ids.push_back(order_id_of(orient, g));
   }
+  // every panel k-outer: what a block pool smaller than the working set needs (each fetched tile is used by a whole
+  // row or column of the panel before it is evicted); a panel as wide as the grid is already listed above
+  for (int orient = 0; orient < 2; ++orient) {
+    const int g = orient == 0 ? p.Ng() : p.Mg();
+    for (int w : widths)
+      if (w < g) ids.push_back(20000 + order_id_of(orient, w));
+  }
+  // with evictions in sight, every order also with the eviction policy that favours long-untouched tiles
+  if (p.pool_blocks < gemm_full_block_num(p)) {
+    const size_t n = ids.size();
+    for (size_t i = 0; i < n; ++i) ids.push_back(40000 + ids[i]);
+  }
   return ids;
 }
 
@@ -78,6 +106,7 @@ struct Block {
   int kind = -1;  // -1 free, 0 A tile, 1 B tile, 2 accumulator, 3 source C
   int idx = -1;
   int content_cmd = -1;        // command after which the content is valid (the fetch)
+  int last_touch = -1;         // latest command that wrote or read the content
   std::vector<int> pending;    // commands that must complete before the block may be overwritten
   bool ever_used = false;
 };
@@ -123,6 +152,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
   std::deque<int> free_list;
   for (int b = 0; b < (int)blocks.size(); ++b) free_list.push_back(b);
   int c_seq = 0;
+  const bool slack_policy = order_id >= 40000;
+  int cur_pos = 0;
   std::vector<Cmd>& cmds = plan.cmds;
   cmds.reserve(plan.task_order.size() * 2 + 16);
 
@@ -130,17 +161,22 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     blocks[b].kind = -1;
     blocks[b].idx = -1;
     blocks[b].pending.assign(1, after_cmd);
+    blocks[b].last_touch = after_cmd;
     free_list.push_back(b);
   };
 
   // Returns a block whose previous content may be dropped; "waits" receives what a writer must wait for.
   auto alloc = [&](int pin1, int pin2, std::vector<int>& waits) -> int {
+    // Policy 0 recycles a free block if there is one, else evicts the tile whose next use is farthest away: the fewest
+    // fetches, but the block is often one read a moment ago (a tile that has just died, or in a k-outer panel the most
+    // recent tiles, which the next panel needs last), so the fetch waits for that subkernel and the copy stream never
+    // gets ahead.  Policy 1 also looks at the tiles not needed within the next pool-size subkernels and takes, among
+    // them and the oldest free block, the one untouched for longest: its readers finished long ago, so the fetch
+    // can start at once.  Which policy wins depends on whether copies or subkernels bound the schedule; the
+    // simulation decides.
     int b = -1;
-    if (!free_list.empty()) {
-      b = free_list.front();
-      free_list.pop_front();
-    } else {
-      int best_next = -1;
+    int best_next = -1, best_touch = INT_MAX;
+    if (free_list.empty() || slack_policy) {
       for (int i = 0; i < (int)blocks.size(); ++i) {
         if (i == pin1 || i == pin2) continue;
         int next;
@@ -151,13 +187,23 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
           const auto& u = b_uses[blocks[i].idx];
           next = b_ptr[blocks[i].idx] < (int)u.size() ? u[b_ptr[blocks[i].idx]] : INT_MAX;
         } else {
-          continue;  // accumulators and source-C blocks are exclusive: never evicted
+          continue;  // free blocks; accumulators and source-C blocks are exclusive: never evicted
         }
-        if (next > best_next) {
+        if (slack_policy && next - cur_pos > (int)blocks.size()) {
+          if (blocks[i].last_touch < best_touch) {
+            best_touch = blocks[i].last_touch;
+            b = i;
+          }
+        } else if (best_touch == INT_MAX && next > best_next) {
           best_next = next;
           b = i;
         }
       }
+    }
+    if (!free_list.empty() && !(best_touch < blocks[free_list.front()].last_touch)) {
+      b = free_list.front();
+      free_list.pop_front();
+    } else {
       if (b < 0) throw std::runtime_error("PARALiA gemm: device block pool too small for this subkernel order");
       if (blocks[b].kind == 0) a_blk[blocks[b].idx] = -1;
       else b_blk[blocks[b].idx] = -1;
@@ -171,6 +217,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
 
   auto note_reader = [&](int b, int cmd_idx) {
     // one pending reader per stream is enough: streams run their commands in order
+    blocks[b].last_touch = cmd_idx;
     auto& pend = blocks[b].pending;
     for (int& w : pend)
       if (cmds[w].stream == cmds[cmd_idx].stream) {
@@ -184,6 +231,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     const int t = plan.task_order[pos];
     const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
     const int ai = mi * Kg + ki, bi = ki * Ng + ni, ci = mi * Ng + ni;
+    cur_pos = pos;
     ++a_ptr[ai];
     ++b_ptr[bi];
     int ablk = -1, bblk = -1;
@@ -197,7 +245,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
         c.kind = CMD_FETCH_A; c.mi = mi; c.ki = ki; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
         for (int x : w) add_wait(cmds, cmds.back(), x);
-        blocks[b].kind = 0; blocks[b].idx = ai; blocks[b].content_cmd = (int)cmds.size() - 1;
+        blocks[b].kind = 0; blocks[b].idx = ai; blocks[b].content_cmd = blocks[b].last_touch = (int)cmds.size() - 1;
         a_blk[ai] = b;
         ++plan.n_fetch[0];
       }
@@ -212,7 +260,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
         c.kind = CMD_FETCH_B; c.ki = ki; c.ni = ni; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
         for (int x : w) add_wait(cmds, cmds.back(), x);
-        blocks[b].kind = 1; blocks[b].idx = bi; blocks[b].content_cmd = (int)cmds.size() - 1;
+        blocks[b].kind = 1; blocks[b].idx = bi; blocks[b].content_cmd = blocks[b].last_touch = (int)cmds.size() - 1;
         b_blk[bi] = b;
         ++plan.n_fetch[1];
       }
@@ -243,6 +291,19 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     const int gemm_idx = (int)cmds.size() - 1;
     if (ablk >= 0) note_reader(ablk, gemm_idx);
     if (bblk >= 0) note_reader(bblk, gemm_idx);
+    // A tile that no later subkernel reads gives its block back at once (its readers stay pending on the block): the
+    // FIFO then hands out the longest-dead block first, so the fetch that reuses it rarely waits and the copy stream
+    // can run a whole k-step ahead of the subkernels even when the pool is much smaller than the operands.
+    if (ablk >= 0 && a_ptr[ai] == (int)a_uses[ai].size()) {
+      blocks[ablk].kind = -1; blocks[ablk].idx = -1;
+      a_blk[ai] = -1;
+      free_list.push_back(ablk);
+    }
+    if (bblk >= 0 && b_ptr[bi] == (int)b_uses[bi].size()) {
+      blocks[bblk].kind = -1; blocks[bblk].idx = -1;
+      b_blk[bi] = -1;
+      free_list.push_back(bblk);
+    }
 
     if (++fired[ci] == Kg && p.c_remote) {
       const int accb = c_blk[ci];

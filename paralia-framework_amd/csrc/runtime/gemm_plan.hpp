@@ -67,6 +67,10 @@ struct GemmPlan {
 // panel in k-outer (outer-product) order, the remaining columns tile by tile (ni, mi, ki);
 // orient 1: the same with row-tiles (remaining rows in the reference's index order mi, ni, ki).
 // w = 0 with orient 1 is exactly the reference's subkernel index order (dgemm.cpp:139-142).
+// id = 20000 + orient * 10000 + w: every group of w column-tiles (row-tiles) is processed as such a k-outer panel,
+// one after the other; this is the family for block pools smaller than the working set.
+// + 40000: same order, but evictions prefer the tile untouched for longest among those not needed soon (instead of
+// the one needed farthest in the future), which lets fetches run ahead of the subkernels.
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
 std::vector<int> gemm_candidate_orders(const GemmProblem& p);

@@ -50,7 +50,7 @@ def fro(Mx, chunk=1 << 26):
     return float(np.sqrt(sum(float(np.sum(np.square(flat[i:i + chunk], dtype=np.float64))) for i in range(0, flat.size, chunk))))
 
 
-def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL64, panels=3):
+def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL64, panels=3, cache_limit=0):
     ra, ca = (M, K) if ta == "N" else (K, M)
     rb, cb = (K, N) if tb == "N" else (N, K)
     t0 = time.time()
@@ -60,7 +60,7 @@ def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL6
     fn = L.PARALiA_dgemm if np.dtype(dtype) == np.float64 else L.PARALiA_sgemm
     print(f"full-size gemm {np.dtype(dtype).name} {ta}{tb} {M}x{N}x{K} alpha={alpha} beta={beta} locs={locs} T={T} (init {time.time() - t0:.1f}s)", flush=True)
     t0 = time.time()
-    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), bA.ptr, ra, bB.ptr, rb, float(beta), bC.ptr, M, T, 0, C.byref(info)), "gemm")
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), bA.ptr, ra, bB.ptr, rb, float(beta), bC.ptr, M, T, cache_limit, C.byref(info)), "gemm")
     print(f"  first call {1e3 * (time.time() - t0):.1f} ms, T={info.T} ({info.selected_by.decode()}), order {info.order_id}, "
           f"{info.subkernel_num} subkernels, predicted {1e3 * info.pred_t:.1f} ms", flush=True)
     got = colmajor(host(bC), M, N)
@@ -97,6 +97,14 @@ def test_dgemm_16384_host_operands(pkg, L):
     """dgemm 16384^3, alpha = 1, beta = 0, all operands in pinned host memory, T picked by the autotuner."""
     info = check_gemm(pkg, L, np.float64, "N", "N", 16384, 16384, 16384, 1.0, 0.0, (-1, -1, -1))
     assert info.subkernel_num == (-(-16384 // info.T)) ** 3
+
+
+@pytest.mark.timeout(600)
+def test_dgemm_16384_pool_limited(pkg, L):
+    """The same problem with the device block pool limited to 1 GB, a sixth of the 6.4 GB working set: tiles are
+    evicted and fetched again, beta != 0 so that C tiles are fetched late and combined on the device."""
+    info = check_gemm(pkg, L, np.float64, "N", "N", 16384, 16384, 16384, 1.0, 0.5, (-1, -1, -1), cache_limit=10 ** 9)
+    assert 4 * info.T * info.T * 8 <= 10 ** 9
 
 
 @pytest.mark.timeout(600)

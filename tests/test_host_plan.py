@@ -147,7 +147,7 @@ def check_async_safety(rows):
             users[blk] = []
 
 
-ORDERS = [10000, 0, 1, 3, 10002, 10004]
+ORDERS = [10000, 0, 1, 3, 10002, 10004, 20002, 30001, 50000, 60002]
 
 
 @pytest.mark.parametrize("order", ORDERS)
@@ -306,7 +306,7 @@ def test_random_plans_are_safe_and_correct(pkg, seed):
     full = 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
     pool = int(rng.choice([0, 3, 4, 5, max(3, full // 3), max(3, full // 2), full]))
     orient, w = int(rng.integers(0, 2)), int(rng.integers(0, max(Mg, Ng) + 2))
-    order = orient * 10000 + w
+    order = orient * 10000 + w + (20000 if w > 0 and rng.integers(0, 2) else 0) + (40000 if rng.integers(0, 2) else 0)
     A = rng.integers(-4, 5, (M, K)).astype(np.float64)
     B = rng.integers(-4, 5, (K, N)).astype(np.float64)
     C = rng.integers(-4, 5, (M, N)).astype(np.float64)
