@@ -83,6 +83,20 @@ int pl_dgemm_tile(char transA, char transB, long M, long N, long K, double alpha
 int pl_sgemm_tile(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
                   const float* B, long ldb, float beta, float* C, long ldc, void* stream);
 
+/* The same product with a device workspace: when the 128 x 128 tiles of C are too few to occupy the compute units
+ * (small or skinny products), K is split over several workgroups per tile, their partial products go to the
+ * workspace and a second kernel adds them in a fixed order (the result is reproducible).  cuBLAS makes the same
+ * choice internally behind the call sites above.  pl_gemm_tile_workspace_bytes returns what a given shape can
+ * use (0: it would not be split); a null or smaller workspace falls back to the unsplit kernel.  The workspace
+ * must not be shared by launches that may overlap (one per stream). */
+long pl_gemm_tile_workspace_bytes(long M, long N, long K, int elem_size);
+int pl_dgemm_tile_ws(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                     const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
+                     void* stream);
+int pl_sgemm_tile_ws(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                     const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
+                     void* stream);
+
 /* out <- beta*src + acc on an M x N tile (out may alias acc): the ALGO_WR_LAZY reduce of a finished C tile
  * with the caller's original C (dgemm.cpp:173-179; CMakeLists.txt:78-88). */
 int pl_dgeadd_tile(long M, long N, double beta, const double* src, long ld_src, const double* acc, long ld_acc,

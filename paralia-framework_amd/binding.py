@@ -61,6 +61,9 @@ _SIGS = {
     "pl_sync_check": (_i, []),
     "pl_dgemm_tile": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp]),
     "pl_sgemm_tile": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp]),
+    "pl_gemm_tile_workspace_bytes": (_l, [_l, _l, _l, _i]),
+    "pl_dgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _vp]),
+    "pl_sgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _vp]),
     "pl_dgeadd_tile": (_i, [_l, _l, _d, _vp, _l, _vp, _l, _vp, _l, _vp]),
     "pl_sgeadd_tile": (_i, [_l, _l, _f, _vp, _l, _vp, _l, _vp, _l, _vp]),
     "pl_daxpy": (_i, [_l, _d, _vp, _l, _vp, _l, _vp]),

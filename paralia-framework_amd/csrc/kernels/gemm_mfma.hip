@@ -182,11 +182,20 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 template <typename T, bool AK, bool BKM>
 __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
-                                                          long ldc, int gm, int gn, int vecA, int vecB) {
+                                                          long ldc, int gm, int gn, int vecA, int vecB, int kchunk) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
   using acc_t = typename Tr::acc_t;
   constexpr int BK = Tr::BK, BLK = Tr::BLK, NB = WM / BLK;
+  if (kchunk > 0) {
+    // split K: the workgroups of grid row y multiply k in [y * kchunk, (y + 1) * kchunk) and leave their plain partial
+    // product in slice y of the workspace passed as C (M x N, dense); splitk_reduce_kernel combines the slices
+    const int k0 = blockIdx.y * kchunk;
+    A += AK ? (long)k0 : (long)k0 * lda;
+    B += BKM ? (long)k0 : (long)k0 * ldb;
+    K = min(K - k0, kchunk);
+    C += (long)blockIdx.y * M * N;
+  }
   constexpr int ASZ = Lds<T, AK>::SIZE, BSZ = Lds<T, BKM>::SIZE;
 
   __shared__ __attribute__((aligned(16))) T smem[2 * (ASZ + BSZ)];
@@ -399,9 +408,54 @@ __global__ void scale_kernel(int M, int N, T beta, T* __restrict__ C, long ldc) 
   }
 }
 
+// C = alpha * (slice 0 + slice 1 + ...) + beta * C, slices added in index order: the result does not depend on timing.
+template <typename T>
+__global__ void splitk_reduce_kernel(int M, int N, int splits, T alpha, const T* __restrict__ ws, T beta, T* __restrict__ C, long ldc) {
+  const long total = (long)M * N;
+  for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long)gridDim.x * blockDim.x) {
+    T sum = ws[e];
+    for (int z = 1; z < splits; ++z) sum += ws[(long)z * total + e];
+    T* p = C + (e / M) * ldc + e % M;
+    T v = alpha * sum;
+    if (beta != T(0)) v += beta * *p;
+    *p = v;
+  }
+}
+
+// How many ways to split K so that a product with few C tiles still fills the 256 compute units.
+// The estimate counts rounds of 256 workgroups, each costing its k extent plus a fixed prologue / epilogue share, and
+// the pass that adds the slices (workspace written once and read once).  1 = do not split.
+template <typename T>
+int pick_splits(long M, long N, long K, int* kchunk_out) {
+  const long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  *kchunk_out = 0;
+  // with more than about half the compute units covered, a second product running on another stream (the way the
+  // scheduler issues subkernels) fills the rest better than a split would
+  if (tiles > 160 || K < 256) return 1;
+  const double us_per_k = sizeof(T) == 8 ? 0.117 : 0.0585;  // one workgroup, one unit of k, at the measured tile rate
+  auto main_us = [&](long blocks, long kc) { return (double)((blocks + 255) / 256) * (double)(kc + 48) * us_per_k; };
+  double best = main_us(tiles, K);
+  int best_s = 1;
+  const long max_ws = 256L << 20;  // workspace bound: the slices of very long, very thin products stay small anyway
+  for (int s = 2; s <= 64; ++s) {
+    const long kc = (((K + s - 1) / s) + 15) / 16 * 16;
+    if (kc < 128) break;
+    const long se = (K + kc - 1) / kc;
+    if (se < 2) continue;
+    if (se * M * N * (long)sizeof(T) > max_ws) break;
+    const double t = main_us(tiles * se, kc) + 4.0 + (double)(2 * se + 1) * (double)M * (double)N * sizeof(T) / 4.0e6;
+    if (t < best * 0.95) {
+      best = t;
+      best_s = (int)se;
+      *kchunk_out = (int)kc;
+    }
+  }
+  return best_s;
+}
+
 template <typename T>
 int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
-                T* C, long ldc, hipStream_t stream) {
+                T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0) {
   using Tr = Traits<T>;
   const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
   const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
@@ -423,17 +477,37 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   if ((long)gm * gn > INT32_MAX) return 2;
   const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
   const int vecB = ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % Tr::VEC == 0) ? 1 : 0;
-  dim3 grid(gm * gn), block(NTHREADS);
-#define PLK_LAUNCH(AKF, BKF)                                                                                    \
-  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF>), grid, block, 0, stream, (int)M, (int)N, (int)K, alpha, A, lda, B, \
-                     ldb, beta, C, ldc, gm, gn, vecA, vecB)
+  int kchunk = 0;
+  int splits = workspace ? pick_splits<T>(M, N, K, &kchunk) : 1;
+  if (splits > 1 && (long)splits * M * N * (long)sizeof(T) > workspace_bytes) splits = 1, kchunk = 0;
+  dim3 grid(gm * gn, splits), block(NTHREADS);
+  // split: plain partial products into the dense workspace slices, alpha and beta applied by the reduction
+  const T k_alpha = splits > 1 ? T(1) : alpha, k_beta = splits > 1 ? T(0) : beta;
+  T* const k_C = splits > 1 ? workspace : C;
+  const long k_ldc = splits > 1 ? M : ldc;
+#define PLK_LAUNCH(AKF, BKF)                                                                                      \
+  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, A, lda, B, \
+                     ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, kchunk)
   // op(A) K-major <=> TransA == 'T'; op(B) K-major <=> TransB == 'N'
   if (an && bnn) PLK_LAUNCH(false, true);
   else if (an && bt) PLK_LAUNCH(false, false);
   else if (at && bnn) PLK_LAUNCH(true, true);
   else PLK_LAUNCH(true, false);
 #undef PLK_LAUNCH
+  if (splits > 1) {
+    const long total = M * N;
+    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3(blocks), dim3(256), 0, stream, (int)M, (int)N, splits, alpha, workspace, beta, C, ldc);
+  }
   return hipGetLastError() == hipSuccess ? 0 : 4;
+}
+
+template <typename T>
+long workspace_bytes_for(long M, long N, long K) {
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  int kchunk = 0;
+  const int s = pick_splits<T>(M, N, K, &kchunk);
+  return s > 1 ? (long)s * M * N * (long)sizeof(T) : 0;
 }
 
 }  // namespace plk
@@ -446,4 +520,22 @@ extern "C" int pl_dgemm_tile(char transA, char transB, long M, long N, long K, d
 extern "C" int pl_sgemm_tile(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
                              const float* B, long ldb, float beta, float* C, long ldc, void* stream) {
   return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream);
+}
+
+extern "C" long pl_gemm_tile_workspace_bytes(long M, long N, long K, int elem_size) {
+  return elem_size == 8 ? plk::workspace_bytes_for<double>(M, N, K) : elem_size == 4 ? plk::workspace_bytes_for<float>(M, N, K) : 0;
+}
+
+extern "C" int pl_dgemm_tile_ws(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                                const double* B, long ldb, double beta, double* C, long ldc, void* workspace,
+                                long workspace_bytes, void* stream) {
+  return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                  (double*)workspace, workspace_bytes);
+}
+
+extern "C" int pl_sgemm_tile_ws(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                                const float* B, long ldb, float beta, float* C, long ldc, void* workspace,
+                                long workspace_bytes, void* stream) {
+  return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                 (float*)workspace, workspace_bytes);
 }

@@ -116,6 +116,9 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
   CoCoVecInit(C, 2 * ld * ld, 44, 0);
   std::vector<void*> st(queues);
   for (auto& s : st) must(pl_stream_create(&s), "stream");
+  const long ws_cap = 512L << 20;
+  std::vector<void*> ws(queues);
+  for (auto& w : ws) w = CoCoMalloc(ws_cap, 0, 1);
   const T alpha = (T)1.1234, beta = (T)1;
   std::vector<Row> rows;
   const char flags[2] = {'N', 'T'};
@@ -126,11 +129,16 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
       FILE* fp = fopen(raw, "w");
       if (!fp) { fprintf(stderr, "cannot write %s\n", raw); exit(1); }
       for (long Tt : Ts) {
+        // launched the way the runtime launches a subkernel: with a split-K workspace per stream
+        const long ws_bytes = pl_gemm_tile_workspace_bytes(Tt, Tt, Tt, (int)sizeof(T));
+        if (ws_bytes > ws_cap) { fprintf(stderr, "split-K workspace larger than expected\n"); exit(1); }
         auto launch = [&](int q) {
           if (sizeof(T) == 8)
-            must(pl_dgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const double*)A, Tt, (const double*)B, Tt, beta, (double*)(C + (long)q * ld * ld), Tt, st[q]), "gemm");
+            must(pl_dgemm_tile_ws(ta, tb, Tt, Tt, Tt, alpha, (const double*)A, Tt, (const double*)B, Tt, beta, (double*)(C + (long)q * ld * ld), Tt,
+                                  ws[q], ws_bytes, st[q]), "gemm");
           else
-            must(pl_sgemm_tile(ta, tb, Tt, Tt, Tt, alpha, (const float*)A, Tt, (const float*)B, Tt, beta, (float*)(C + (long)q * ld * ld), Tt, st[q]), "gemm");
+            must(pl_sgemm_tile_ws(ta, tb, Tt, Tt, Tt, alpha, (const float*)A, Tt, (const float*)B, Tt, beta, (float*)(C + (long)q * ld * ld), Tt,
+                                  ws[q], ws_bytes, st[q]), "gemm");
         };
         // long enough that the ramp at both ends of a batch does not weigh on the steady-state rate
         const int batch = (Tt <= 2048 ? 16 : Tt <= 4096 ? 6 : 2) * queues;
@@ -160,6 +168,7 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
   fclose(fp);
   for (auto s : st) pl_stream_destroy(s);
   CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
+  for (auto w : ws) CoCoFree(w, 0);
 }
 
 static void bench_gemv(const std::string& db, bool quick) {

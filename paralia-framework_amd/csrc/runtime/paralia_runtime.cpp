@@ -142,6 +142,8 @@ struct Resources {
     }
     void release() { if (p) pl_free_device(p); p = nullptr; cap = 0; }
   } gemv_x, gemv_y, gemv_ws;
+  // split-K workspaces of the tile GEMM, one per exec stream (launches on different streams may overlap)
+  Scratch gemm_ws[MAX_EXEC_QUEUES];
   void* stream(int id) const { return id == STREAM_H2D ? h2d : id == STREAM_D2H ? d2h : exec[id - STREAM_EXEC0]; }
   void sync_all() {
     if (h2d) chk(pl_stream_sync(h2d), "stream sync");
@@ -155,6 +157,7 @@ struct Resources {
     if (dot_ws) pl_free_device(dot_ws);
     if (dot_host) pl_free_pinned(dot_host);
     gemv_x.release(); gemv_y.release(); gemv_ws.release();
+    for (Scratch& w : gemm_ws) w.release();
     stager_.reset();
     *this = Resources();
   }
@@ -217,7 +220,9 @@ template <typename T> struct GemmFns;
 template <> struct GemmFns<double> {
   static constexpr const char* name = "Dgemm";
   static int tile(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
-                  double be, double* C, long ldc, void* s) { return pl_dgemm_tile(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, s); }
+                  double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
+    return pl_dgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
   static int geadd(long M, long N, double be, const double* s, long lds, const double* a, long lda, double* o, long ldo, void* st) {
     return pl_dgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
   }
@@ -225,7 +230,9 @@ template <> struct GemmFns<double> {
 template <> struct GemmFns<float> {
   static constexpr const char* name = "Sgemm";
   static int tile(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
-                  float be, float* C, long ldc, void* s) { return pl_sgemm_tile(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, s); }
+                  float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
+    return pl_sgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
   static int geadd(long M, long N, float be, const float* s, long lds, const float* a, long lda, float* o, long ldo, void* st) {
     return pl_sgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
   }
@@ -248,6 +255,17 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   HostStager& stager = R.res.stager();
   if (pageable[0] || pageable[1] || pageable[2]) stager.reserve((long long)Tt * Tt * (long long)sizeof(T));
   StagerScope staged(stager);
+  // what the tile kernel can use to split K when a tile product has too few workgroups (small T): the largest need
+  // over the full and the ragged tile extents
+  long ws_bytes = 0;
+  for (int e = 0; e < 8; ++e) {
+    const long m = (e & 1) ? p.tm(p.Mg() - 1) : std::min<long>(Tt, p.M), n = (e & 2) ? p.tn(p.Ng() - 1) : std::min<long>(Tt, p.N);
+    const long k = p.Kg() > 0 ? ((e & 4) ? p.tk(p.Kg() - 1) : std::min<long>(Tt, p.K)) : 0;
+    ws_bytes = std::max(ws_bytes, pl_gemm_tile_workspace_bytes(m, n, k, (int)sizeof(T)));
+  }
+  void* ws[MAX_EXEC_QUEUES] = {nullptr};
+  if (ws_bytes > 0)
+    for (int q = 0; q < std::max(1, std::min(p.exec_queues, MAX_EXEC_QUEUES)); ++q) ws[q] = R.res.gemm_ws[q].ensure(ws_bytes);
 
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
@@ -289,7 +307,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         const T bp = c.beta_mode == BETA_ZERO ? T(0) : c.beta_mode == BETA_ONE ? T(1) : beta;
         if (la < 1) la = 1;
         if (lb < 1) lb = 1;
-        chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, s), "tile gemm launch");
+        chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, s), "tile gemm launch");
       } break;
       case CMD_REDUCE: {
         const long m = p.tm(c.mi), n = p.tn(c.ni);
@@ -414,7 +432,9 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   if (!any_remote) {
     // Every operand already in HBM: one launch over the caller's matrices.
     R.res.ensure_streams(1);
-    chk(GemmFns<T>::tile(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, R.res.exec[0]), "gemm launch");
+    const long ws_bytes = no_ab ? 0 : pl_gemm_tile_workspace_bytes(M, N, K, (int)sizeof(T));
+    void* ws = ws_bytes > 0 ? R.res.gemm_ws[0].ensure(ws_bytes) : nullptr;
+    chk(GemmFns<T>::tile(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, ws, ws_bytes, R.res.exec[0]), "gemm launch");
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;

@@ -88,3 +88,18 @@ def test_predictor_driver_emits_a_runner_row(pkg, tmp_path):
     # wrong argument count is the reference's usage error
     run = subprocess.run([exe, "1", "2"], env=env, capture_output=True, text=True, timeout=60)
     assert run.returncode != 0 and "Incorrect input arguments" in run.stderr
+
+
+def test_split_k_workspace_sizing(L):
+    """Host-side decision only: products whose 128 x 128 tiles cover the chip are not split; small or skinny ones ask
+    for whole M x N slices, at least two, with chunks of at least 128 in k."""
+    assert L.pl_gemm_tile_workspace_bytes(16384, 16384, 16384, 8) == 0
+    assert L.pl_gemm_tile_workspace_bytes(2048, 2048, 2048, 8) == 0      # 256 tiles: one per compute unit
+    assert L.pl_gemm_tile_workspace_bytes(1024, 1024, 128, 8) == 0       # K too short to split
+    assert L.pl_gemm_tile_workspace_bytes(0, 10, 10, 8) == 0 and L.pl_gemm_tile_workspace_bytes(10, 10, 10, 3) == 0
+    for M, N, K, esz in ((1024, 1024, 1024, 8), (1024, 1024, 1024, 4), (128, 128, 65536, 8), (300, 200, 777, 8)):
+        b = L.pl_gemm_tile_workspace_bytes(M, N, K, esz)
+        assert b > 0 and b % (M * N * esz) == 0
+        s = b // (M * N * esz)
+        assert 2 <= s <= 64 and K / s >= 112 and b <= 256 << 20
+    assert L.pl_gemm_tile_workspace_bytes(1024, 1024, 1024, 8) == 4 * 1024 * 1024 * 8

@@ -245,3 +245,79 @@ def test_geadd(pkg, L, dtype):
     pkg.check(fn(M2, N, -2.0, ds2.ptr, M2, da2.ptr, M2, da2.ptr, M2, None), "geadd in place")
     sync(pkg)
     assert np.array_equal(da2.get(), -2.0 * src2 + acc2)
+
+
+def run_gemm_ws(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc, ws_elems=None):
+    """The workspace entry point; returns (result, workspace bytes the shape asked for)."""
+    esz = np.dtype(dtype).itemsize
+    need = int(L.pl_gemm_tile_workspace_bytes(M, N, K, esz))
+    n_ws = max(1, need // esz) if ws_elems is None else ws_elems
+    dA, dB, dC = Buf(pkg, A.size, dtype, 0).set(A), Buf(pkg, B.size, dtype, 0).set(B), Buf(pkg, C0.size, dtype, 0).set(C0)
+    dW = Buf(pkg, n_ws, dtype, 0).set(np.full(n_ws, np.nan, dtype=dtype))      # stale workspace content must not matter
+    fn = L.pl_dgemm_tile_ws if dtype == np.float64 else L.pl_sgemm_tile_ws
+    print("gemm_ws", np.dtype(dtype).name, ta, tb, M, N, K, alpha, beta, lda, ldb, ldc, "workspace", need, flush=True)
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, float(alpha), dA.ptr, lda, dB.ptr, ldb, float(beta), dC.ptr, ldc, dW.ptr, n_ws * esz, None), "gemm tile ws")
+    sync(pkg)
+    return dC.get(), need
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(256, 256, 1024), (300, 200, 777), (128, 128, 4096), (1000, 1000, 1000), (64, 1500, 513), (130, 2, 300)])
+def test_dgemm_tile_split_k_vs_openblas(pkg, L, orc, openblas, ta, tb, dims):
+    """Few C tiles and a long K: K is split over several workgroups per tile and the partial products are added by a
+    second kernel.  Ragged chunks (K not a multiple of the chunk), beta != 0, padded leading dimensions."""
+    M, N, K = dims
+    alpha, beta = 1.2, 1.1
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 2, M + 6
+    A, B, C0 = rand_f64(lda * ca, 1), rand_f64(ldb * cb, 2), rand_f64(ldc * N, 3)
+    got, need = run_gemm_ws(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    assert need > 0 and need % (M * N * 8) == 0 and need // (M * N * 8) >= 2
+    ref = C0.copy()
+    assert openblas.orc_openblas_dgemm(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(ref), ldc) == 0
+    d = abs(alpha) * orc.orc_fro_norm_f64(ptr(A), ra, ca, lda) * orc.orc_fro_norm_f64(ptr(B), rb, cb, ldb) + abs(beta) * orc.orc_fro_norm_f64(ptr(C0), M, N, ldc)
+    assert orc.orc_normwise_err_f64(ptr(got), ptr(ref), M, N, ldc, ldc, d) < TOL64
+    pad = np.ones(ldc * N, dtype=bool)
+    pad.reshape(N, ldc)[:, :M] = False
+    assert np.array_equal(got[pad], C0[pad])
+    # twice the same call: the slices are added in a fixed order, so the bits repeat
+    again, _ = run_gemm_ws(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+    assert np.array_equal(got, again)
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N")])
+def test_gemm_tile_split_k_exact_and_fallback(pkg, L, orc, ta, tb):
+    """Integer-valued data: the split result equals the unsplit one bit for bit, for fp64 and fp32; beta = 0 with a
+    NaN-filled C; a workspace that is too small falls back to the unsplit kernel."""
+    M, N, K = 257, 131, 2048
+    rng = np.random.default_rng(6)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    for dtype in (np.float64, np.float32):
+        A = rng.integers(-4, 5, ra * ca).astype(dtype)
+        B = rng.integers(-4, 5, rb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, M * N).astype(dtype)
+        for alpha, beta in ((2.0, 3.0), (1.0, 0.0)):
+            Cin = np.full(M * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+            got, need = run_gemm_ws(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, ra, B, rb, Cin, M)
+            assert need > 0
+            plain = run_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, ra, B, rb, Cin, M)
+            assert np.array_equal(got, plain)
+            small, _ = run_gemm_ws(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, ra, B, rb, Cin, M, ws_elems=16)
+            assert np.array_equal(small, plain)
+    ref = C0.astype(np.float64)
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    orc.orc_dgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, 1.0, ptr(A64), ra, ptr(B64), rb, 0.0, ptr(ref), M)
+    assert np.array_equal(got.astype(np.float64), ref)
+
+
+def test_sgemm_tile_split_k_vs_openblas(pkg, L, orc, openblas):
+    M, N, K = 384, 200, 3001
+    A, B, C0 = rand_f32(M * K, 1), rand_f32(N * K, 2), rand_f32(M * N, 3)
+    got, need = run_gemm_ws(pkg, L, np.float32, "N", "T", M, N, K, 0.75, -1.5, A, M, B, N, C0, M)
+    assert need > 0
+    ref = C0.copy()
+    assert openblas.orc_openblas_sgemm(b"N", b"T", M, N, K, 0.75, ptr(A), M, ptr(B), N, -1.5, ptr(ref), M) == 0
+    d = 0.75 * float(np.linalg.norm(A.astype(np.float64))) * float(np.linalg.norm(B.astype(np.float64))) + 1.5 * float(np.linalg.norm(C0.astype(np.float64)))
+    assert float(np.linalg.norm(got.astype(np.float64) - ref.astype(np.float64))) / d < TOL32
