@@ -13,6 +13,53 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+# The driver executables are started by a small launcher process that is itself started before any test has touched
+# the GPU (a process that has initialised the GPU must not start other programs on these machines).
+_LAUNCHER_CODE = r"""
+import json, subprocess, sys
+for line in sys.stdin:
+    req = json.loads(line)
+    try:
+        r = subprocess.run(req["argv"], env=req["env"], capture_output=True, text=True, timeout=req["timeout"])
+        out = {"rc": r.returncode, "stdout": r.stdout, "stderr": r.stderr}
+    except subprocess.TimeoutExpired as e:
+        out = {"rc": 124, "stdout": "", "stderr": "timeout after %s s" % req["timeout"]}
+    except OSError as e:
+        out = {"rc": 127, "stdout": "", "stderr": str(e)}
+    sys.stdout.write(json.dumps(out) + "\n")
+    sys.stdout.flush()
+"""
+_launcher = None
+
+
+def pytest_collection_finish(session):
+    global _launcher
+    if _launcher is None and any("test_gpu_drivers" in item.nodeid for item in session.items):
+        _launcher = subprocess.Popen([sys.executable, "-u", "-c", _LAUNCHER_CODE], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    global _launcher
+    if _launcher is not None:
+        _launcher.stdin.close()
+        _launcher.wait(timeout=30)
+        _launcher = None
+
+
+@pytest.fixture(scope="session")
+def run_program():
+    """run_program(argv, env, timeout) -> dict(rc, stdout, stderr), executed by the launcher process."""
+    import json
+    if _launcher is None:
+        pytest.skip("launcher process not started")
+
+    def run(argv, env=None, timeout=300):
+        _launcher.stdin.write(json.dumps({"argv": [str(a) for a in argv], "env": dict(env or os.environ), "timeout": timeout}) + "\n")
+        _launcher.stdin.flush()
+        return json.loads(_launcher.stdout.readline())
+    return run
+
+
 def load_package():
     """The package directory is named paralia-framework_amd (not an identifier): import it by path."""
     name = "paralia_framework_amd"
