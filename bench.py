@@ -211,7 +211,7 @@ def main():
         if orc.orc_openblas_open(None) == 0:
             cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
             cores = orc.orc_openblas_threads(cores) or cores
-            ncols = max(256, min(n, 2048))  # a column panel of C: M x ncols x K of the same problem
+            ncols = max(256, min(n, 8192))  # a column panel of C: M x ncols x K of the same problem (a few seconds on 16 cores)
             ref = np.zeros(n * ncols)
             orc.orc_openblas_dgemm(b"N", b"N", n, 256, n, 1.0, hA.ptr, n, hB.ptr, n, 0.0, ob.ptr(ref), n)  # warm-up
             t0 = time.perf_counter()
@@ -224,6 +224,13 @@ def main():
                    "sample": "OpenBLAS cblas_dgemm (%s) on the first %d columns of C of the same problem (M=%d, N=%d, K=%d), %.1f s"
                              % (os.path.basename(orc.orc_openblas_path().decode()), ncols, n, ncols, n, t_cpu),
                    "gpu_vs_openblas_normwise_err": err}
+            # the reference's own CPU-runnable configuration: dgemm 4096^3, alpha = 1.2, beta = 1.1, on the same cores
+            m1 = min(n, 4096)
+            c1 = np.ones(m1 * m1)
+            orc.orc_openblas_dgemm(b"N", b"N", m1, m1, m1, 1.2, hA.ptr, n, hB.ptr, n, 1.1, ob.ptr(c1), m1)
+            t0 = time.perf_counter()
+            orc.orc_openblas_dgemm(b"N", b"N", m1, m1, m1, 1.2, hA.ptr, n, hB.ptr, n, 1.1, ob.ptr(c1), m1)
+            cpu["dgemm_4096_alpha1.2_beta1.1_gflops"] = 2.0 * m1 ** 3 / (time.perf_counter() - t0) / 1e9
         else:
             cpu = {"value": None, "unit": "GFLOP/s", "cores": 0, "kind": "port", "sample": "OpenBLAS absent on this box"}
 
