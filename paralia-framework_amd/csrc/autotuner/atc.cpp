@@ -11,6 +11,7 @@
 #include <cfloat>
 #include <cmath>
 #include <cstdlib>
+#include <algorithm>
 #include <cstring>
 
 #include "Autotuner.hpp"
@@ -328,10 +329,22 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       T_selected_by = "cocopelia-reuse";
     } else {
       const Modeler* m = unit_modeler_list[0];
-      long best_T = -1, prev = -1;
-      double best_t = DBL_MAX;
-      // Largest tiles first: they have few subkernels and are cheap to simulate, and once a good makespan is known
-      // the small tiles, whose kernels alone already take longer than that, are dismissed without building a plan.
+      // Two passes over the benchmarked tile sizes.  The first prices each T with a handful of representative
+      // subkernel orders (largest tiles first: they have few subkernels and are cheap to simulate, and once a good
+      // makespan is known the small tiles, whose kernels alone already take longer than that, are dismissed without
+      // building a plan).  The second runs the full order search only for the (at most three) T whose penalised probe is within 10 % of the best.
+      struct Cand { long T; double probe_t; };
+      // predictions of neighbouring T differ by less than the model's accuracy: the reference's penalty terms
+      // (ragged edges, too few or too many subkernels, Autotuner.cpp:571-603) break such near-ties
+      auto penalty = [&](long cand) {
+        if (cand > min_dim) return 1.0;
+        double sl[6];
+        get_T_slowdowns(sl, (int)cand);
+        return 1.0 + 0.02 * sl[0];
+      };
+      std::vector<Cand> cands;
+      long prev = -1;
+      double best_probe = DBL_MAX;
       for (long i = m->exec->lines() - 1; i >= 0; i--) {
         const long cand = m->exec->T[i];
         if (cand == prev) continue;
@@ -343,21 +356,36 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         if (gp.pool_blocks < 3 || gp.subkernels() > 20000) continue;
         const paralia::StageTimes st = paralia_stage_times(this, cand);
-        if (best_T > 0 && (double)gp.subkernels() * st.exec_time(cand, std::min(cand, problem.D1), std::min(cand, problem.D2),
-                                                                   std::min(cand, problem.D3)) * 0.9 > best_t) continue;
+        if ((double)gp.subkernels() * st.exec_time(cand, std::min(cand, problem.D1), std::min(cand, problem.D2),
+                                                    std::min(cand, problem.D3)) * 0.9 > best_probe) continue;
         paralia::PipelineResult r;
         try {
-          paralia::pick_gemm_order(gp, st, &r);
+          paralia::pick_gemm_order(gp, st, &r, /*probe=*/true);
         } catch (const std::runtime_error&) { continue; }
-        // predictions of neighbouring T differ by less than the model's accuracy: the reference's penalty terms
-        // (ragged edges, too few or too many subkernels, Autotuner.cpp:571-603) break such near-ties
-        double score = r.t_total;
-        if (cand <= min_dim) {
-          double sl[6];
-          get_T_slowdowns(sl, (int)cand);
-          score *= 1.0 + 0.02 * sl[0];
-        }
-        if (score <= best_t) { best_t = score; best_T = cand; }  // ties go to the smaller tile
+        cands.push_back({cand, r.t_total * penalty(cand)});
+        best_probe = std::min(best_probe, r.t_total);
+      }
+      long best_T = -1;
+      double best_t = DBL_MAX;
+      // at most the three best probes go on (kept in table order, largest T first, so that ties still go to the
+      // smaller tile below)
+      double cut = DBL_MAX;
+      if (cands.size() > 3) {
+        std::vector<double> ts;
+        for (const Cand& c : cands) ts.push_back(c.probe_t);
+        std::nth_element(ts.begin(), ts.begin() + 2, ts.end());
+        cut = ts[2];
+      }
+      for (const Cand& c : cands) {
+        if (c.probe_t > 1.1 * best_probe || c.probe_t > cut) continue;
+        const long cand = c.T;
+        paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
+        paralia::PipelineResult r;
+        try {
+          paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
+        } catch (const std::runtime_error&) { continue; }
+        const double score = r.t_total * penalty(cand);
+        if (score <= best_t) { best_t = score; best_T = cand; }  // ties go to the smaller tile (largest T comes first)
       }
       if (best_T < 0) {
         // C narrower than every benchmarked tile: one tile across the short side, as square as that allows

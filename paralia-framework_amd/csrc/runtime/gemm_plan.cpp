@@ -67,27 +67,40 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   return order;
 }
 
-std::vector<int> gemm_candidate_orders(const GemmProblem& p) {
+std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe) {
   std::vector<int> ids;
   ids.push_back(order_id_of(1, 0));  // the reference's index order; needs the fewest blocks
   if (!(p.a_remote || p.b_remote || p.c_remote)) return ids;
+  const bool limited = p.pool_blocks < gemm_full_block_num(p);
   static const int widths[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 48, 64};
+  static const int probe_widths[] = {2, 4};
   for (int orient = 0; orient < 2; ++orient) {
     const int g = orient == 0 ? p.Ng() : p.Mg();
-    if (orient == 0) ids.push_back(order_id_of(0, 0));
-    for (int w : widths)
-      if (w < g) ids.push_back(order_id_of(orient, w));
+    if (orient == 0 && !probe) ids.push_back(order_id_of(0, 0));
+    if (probe) {
+      for (int w : probe_widths)
+        if (w < g) ids.push_back(order_id_of(orient, w));
+    } else {
+      for (int w : widths)
+        if (w < g) ids.push_back(order_id_of(orient, w));
+    }
     ids.push_back(order_id_of(orient, g));
   }
   // every panel k-outer: what a block pool smaller than the working set needs (each fetched tile is used by a whole
   // row or column of the panel before it is evicted); a panel as wide as the grid is already listed above
-  for (int orient = 0; orient < 2; ++orient) {
-    const int g = orient == 0 ? p.Ng() : p.Mg();
-    for (int w : widths)
-      if (w < g) ids.push_back(20000 + order_id_of(orient, w));
-  }
+  if (!probe || limited)
+    for (int orient = 0; orient < 2; ++orient) {
+      const int g = orient == 0 ? p.Ng() : p.Mg();
+      if (probe) {
+        for (int w : probe_widths)
+          if (w < g) ids.push_back(20000 + order_id_of(orient, w));
+      } else {
+        for (int w : widths)
+          if (w < g) ids.push_back(20000 + order_id_of(orient, w));
+      }
+    }
   // with evictions in sight, every order also with the eviction policy that favours long-untouched tiles
-  if (p.pool_blocks < gemm_full_block_num(p)) {
+  if (limited) {
     const size_t n = ids.size();
     for (size_t i = 0; i < n; ++i) ids.push_back(40000 + ids[i]);
   }
@@ -444,11 +457,11 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
   return r;
 }
 
-int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best_out) {
+int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best_out, bool probe) {
   int best_id = -1;
   PipelineResult best;
   std::string last_err;
-  for (int id : gemm_candidate_orders(p)) {
+  for (int id : gemm_candidate_orders(p, probe)) {
     try {
       GemmPlan plan = build_gemm_plan(p, id);
       PipelineResult r = simulate_plan(plan, st);

@@ -73,7 +73,8 @@ struct GemmPlan {
 // the one needed farthest in the future), which lets fetches run ahead of the subkernels.
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
-std::vector<int> gemm_candidate_orders(const GemmProblem& p);
+// probe = true: a handful of representative orders, enough to rank tile sizes before the full search
+std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe = false);
 
 // Throws std::runtime_error when pool_blocks cannot hold the minimum working set (3 blocks, dgemm.cpp:90-93).
 GemmPlan build_gemm_plan(const GemmProblem& p, int order_id);
@@ -98,7 +99,7 @@ struct PipelineResult {
 };
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st);
 // Builds every candidate order, simulates it, returns the id with the smallest makespan.
-int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best);
+int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best, bool probe = false);
 
 }  // namespace paralia
 #endif
