@@ -75,7 +75,11 @@ template <> struct Traits<float> {
   static constexpr int KSTEP = 2;
   static constexpr int NACC = 16;
   static constexpr int S_MN = 160;   // 640 B = 128 mod 256
-  static constexpr int S_K = BK + 4;  // 80 B: rows 16-byte aligned, the 32 lanes of a block spread over all banks
+  // 18 words: lane (idx, kk) of an operand read sits in bank (18 * idx + kk) mod 64, all 64 distinct.  Rows are then
+  // only 8-byte aligned, so a 16-byte vector goes to LDS as two 8-byte stores (lds_put).  A 16-byte aligned stride
+  // (20 words) costs two-way conflicts on every operand read (measured: conflict cycles 54 % -> 33 % of the LDS
+  // cycles, the rest comes from the stores; worth 1 % on TN, nothing on NN: LDS is not what limits these variants).
+  static constexpr int S_K = BK + 2;
   static constexpr int NV = 128 * BK / VEC / 256;
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -139,12 +143,28 @@ __device__ __forceinline__ void gload_one(const T* __restrict__ base, long ld, t
   Slot<T, KMAJOR>::coords(tid, i, c, s);
   reg = *reinterpret_cast<const typename Traits<T>::vec_t*>(base + c + (long)s * ld);
 }
+typedef float fvec2 __attribute__((ext_vector_type(2)));
+
+// One 16-byte vector into LDS; PUTS<T, KMAJOR> is the number of store instructions that takes.
+template <typename T, bool KMAJOR> constexpr int PUTS = (KMAJOR && sizeof(T) == 4) ? 2 : 1;
+template <typename T, bool KMAJOR>
+__device__ __forceinline__ void lds_put(T* __restrict__ p, const typename Traits<T>::vec_t& v) {
+  if constexpr (KMAJOR && sizeof(T) == 4) {
+    fvec2 lo, hi;
+    lo.x = v[0]; lo.y = v[1]; hi.x = v[2]; hi.y = v[3];
+    *reinterpret_cast<fvec2*>(p) = lo;
+    *reinterpret_cast<fvec2*>(p + 2) = hi;
+  } else {
+    *reinterpret_cast<typename Traits<T>::vec_t*>(p) = v;
+  }
+}
+
 template <typename T, bool KMAJOR>
 __device__ __forceinline__ void lds_store_one(T* __restrict__ xs, const typename Traits<T>::vec_t& reg, int tid, int i) {
   int c, s;
   Slot<T, KMAJOR>::coords(tid, i, c, s);
   const int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
-  *reinterpret_cast<typename Traits<T>::vec_t*>(xs + off) = reg;
+  lds_put<T, KMAJOR>(xs + off, reg);
 }
 
 template <typename T, bool KMAJOR>
@@ -157,7 +177,7 @@ __device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Tra
     Slot<T, KMAJOR>::coords(tid, i, c, s);
     // the contiguous run is also contiguous in LDS for both layouts
     int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
-    *reinterpret_cast<vec_t*>(xs + off) = regs[i];
+    lds_put<T, KMAJOR>(xs + off, regs[i]);
   }
 }
 
@@ -312,7 +332,8 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
           for (int q = 0; q < PER_STEP; ++q) {
             const int slot = ks * PER_STEP + q;
             __builtin_amdgcn_sched_group_barrier(0x008, MFMAS / PER_STEP > 0 ? MFMAS / PER_STEP : 1, 0);
-            if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            if (slot < NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
+            else if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
             else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
           }
           __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
@@ -328,7 +349,8 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
 #pragma unroll
             for (int q = m * SPM; q < (m + 1) * SPM && q < PER_STEP; ++q) {
               const int slot = ks * PER_STEP + q;
-              if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+              if (slot < NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
+              else if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
               else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
           }
