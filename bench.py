@@ -184,8 +184,6 @@ def main():
 
     # ------------------------------------------------------------------ daxpy, device-resident (config 2)
     nd = 1 << 28
-    for b in (dA, dB, dC, hC):
-        pass
     dx, dy = dA, dB  # reuse the 2 GiB device buffers: 2^28 doubles each
     if dx.n >= nd:
         for _ in range(5):
@@ -200,6 +198,27 @@ def main():
         t_ax = ms.value / 20 / 1e3
         daxpy = {"workload": "daxpy N=2^28 fp64, x and y in HBM", "GBps": 24.0 * nd / t_ax / 1e9, "ms": t_ax * 1e3,
                  "frac_of_hbm_peak": 24.0 * nd / t_ax / HBM_PEAK}
+        # ddot N = 2^28 and dgemv 16384 x 16384 (the 2 GiB of A as the matrix), device-resident, same event timing
+        def timed(launch, reps):
+            for _ in range(3):
+                launch()
+            pkg.check(L.pl_stream_sync(s), "sync")
+            pkg.check(L.pl_event_record(e0, s), "record")
+            for _ in range(reps):
+                launch()
+            pkg.check(L.pl_event_record(e1, s), "record")
+            pkg.check(L.pl_stream_sync(s), "sync")
+            pkg.check(L.pl_event_elapsed_ms(e0, e1, C.byref(ms)), "elapsed")
+            return ms.value / reps / 1e3
+
+        ws = Buf(pkg, max(int(L.pl_ddot_workspace_doubles()), int(L.pl_dgemv_workspace_doubles(b"N", 16384, 16384))) + 1, np.float64, 0)
+        res, yv = Buf(pkg, 1, np.float64, 0), Buf(pkg, 16384, np.float64, 0)
+        t_dot = timed(lambda: pkg.check(L.pl_ddot(nd, dx.ptr, 1, dy.ptr, 1, res.ptr, 0, ws.ptr, s), "ddot"), 20)
+        t_mv = timed(lambda: pkg.check(L.pl_dgemv(b"N", 16384, 16384, 1.2, dx.ptr, 16384, dy.ptr, 1, 1.1, yv.ptr, 1, ws.ptr, s), "dgemv"), 20)
+        daxpy["ddot_GBps"] = 16.0 * nd / t_dot / 1e9
+        daxpy["ddot_frac_of_hbm_peak"] = 16.0 * nd / t_dot / HBM_PEAK
+        daxpy["dgemv_16384_GBps"] = 8.0 * (16384.0 * 16384 + 3 * 16384) / t_mv / 1e9
+        daxpy["dgemv_16384_frac_of_hbm_peak"] = 8.0 * (16384.0 * 16384 + 3 * 16384) / t_mv / HBM_PEAK
     else:
         daxpy = None
 
