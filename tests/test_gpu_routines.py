@@ -110,6 +110,21 @@ def test_dgemm_block_pool_smaller_than_working_set(pkg, L, orc, openblas, blocks
     assert pool.value == 0
 
 
+@pytest.mark.parametrize("blocks", [5, 9, 14, 20, 33, 60, 100])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_dgemm_pool_sweep_picks_different_orders(pkg, L, orc, openblas, blocks, beta):
+    """A 6 x 5 x 7 grid of ragged tiles (138 blocks when everything fits) in pools from 5 to 100 blocks: the
+    autotuner moves between the order families and the two eviction policies, the result stays the same."""
+    M, N, K, T = 1436, 1180, 1700, 256
+    A, B, C0 = rand_f64(M * K, 11), rand_f64(K * N, 12), rand_f64(M * N, 13)
+    ref = openblas_ref(openblas, np.float64, "T", "N", M, N, K, -0.7, beta, A, K, B, K, C0, M)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    info = call_gemm(pkg, L, np.float64, "T", "N", M, N, K, -0.7, beta, bA, K, bB, K, bC, M, T=T, cache_limit=blocks * T * T * 8)
+    print("  order", info.order_id, "subkernels", info.subkernel_num, flush=True)
+    assert info.subkernel_num == 6 * 5 * 7
+    assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 0.7, beta, A, K, M, K, B, K, N, K, C0) < TOL64
+
+
 def test_dgemm_too_little_memory_is_an_error(pkg, L):
     M = N = K = 512
     A = rand_f64(M * K, 1)
