@@ -54,6 +54,7 @@ template <> struct Traits<double> {
   static constexpr int WAVES = PLK_WAVES_PER_EU;  // wavefronts per SIMD the register budget is sized for
   static constexpr int BLK = 16;     // MFMA block edge
   static constexpr int KSTEP = 4;    // k consumed per MFMA
+  static constexpr int KV = 1;       // MFMA k-steps served by one refresh of the operand registers
   static constexpr int NACC = 4;     // accumulator elements per lane per block
   static constexpr int S_MN = 144;   // LDS row stride, [k][mn] layout (1152 B = 128 mod 256)
   static constexpr int S_K = BK + 2; // LDS row stride, [mn][k] layout
@@ -73,6 +74,7 @@ template <> struct Traits<float> {
   static constexpr int WAVES = PLK_F32_WAVES_PER_EU;
   static constexpr int BLK = 32;
   static constexpr int KSTEP = 2;
+  static constexpr int KV = 2;       // two k-steps per refresh: their operands come with one LDS instruction
   static constexpr int NACC = 16;
   static constexpr int S_MN = 160;   // 640 B = 128 mod 256
   // 18 words: lane (idx, kk) of an operand read sits in bank (18 * idx + kk) mod 64, all 64 distinct.  Rows are then
@@ -263,23 +265,36 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     }
   };
 
-  const T* const lane_a = smem + Lds<T, AK>::at(kk, wm + idx);         // this lane's A operand of k-step 0, block 0
-  const T* const lane_b = smem + ASZ + Lds<T, BKM>::at(kk, wn + idx);  // this lane's B operand
-  constexpr int A_KS = Lds<T, AK>::at(Tr::KSTEP, 0), A_BL = Lds<T, AK>::at(0, BLK);    // strides per k-step / per block
-  constexpr int B_KS = Lds<T, BKM>::at(Tr::KSTEP, 0), B_BL = Lds<T, BKM>::at(0, BLK);
-  constexpr int KS = BK / Tr::KSTEP;
+  // fp32 operands in the [k][mn] layout: lane idx of block j takes row NB * idx + j instead of j * BLK + idx, so the
+  // rows a lane needs for its NB blocks are adjacent in LDS and come with one 8-byte read instead of NB 4-byte ones
+  // (every operand read issued between MFMAs costs MFMA issue slots: 1 read per MFMA loses 8 % of the pipe rate,
+  // 1 per 2 about half of that).  The epilogue maps the accumulators back with the same rule.
+  constexpr bool A_PAIR = sizeof(T) == 4 && !AK, B_PAIR = sizeof(T) == 4 && !BKM;
+  const T* const lane_a = smem + Lds<T, AK>::at(kk, wm + (A_PAIR ? NB * idx : idx));         // this lane's A operand of k-step 0, block 0
+  const T* const lane_b = smem + ASZ + Lds<T, BKM>::at(kk, wn + (B_PAIR ? NB * idx : idx));  // this lane's B operand
+  constexpr int A_KS = Lds<T, AK>::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : Lds<T, AK>::at(0, BLK);    // strides per k-step / per block
+  constexpr int B_KS = Lds<T, BKM>::at(Tr::KSTEP, 0), B_BL = B_PAIR ? 1 : Lds<T, BKM>::at(0, BLK);
+  constexpr int NREADS = (A_PAIR ? 1 : NB) + (B_PAIR ? 1 : NB);  // LDS read instructions per k-step
+  constexpr int KV = Tr::KV;
+  constexpr int KS = BK / (Tr::KSTEP * KV);  // operand refreshes ("steps") per panel
+  constexpr int A_KV = Lds<T, AK>::at(Tr::KSTEP, 0), B_KV = Lds<T, BKM>::at(Tr::KSTEP, 0);  // k-step stride inside a step
 
-  auto read_ops = [&](int buf, int ks, T (&am)[NB], T (&bnv)[NB]) {
+  auto read_ops = [&](int buf, int ks, T (&am)[KV][NB], T (&bnv)[KV][NB]) {
 #pragma unroll
-    for (int j = 0; j < NB; ++j) am[j] = lane_a[buf * STAGE + ks * A_KS + j * A_BL];
+    for (int v = 0; v < KV; ++v) {
 #pragma unroll
-    for (int i = 0; i < NB; ++i) bnv[i] = lane_b[buf * STAGE + ks * B_KS + i * B_BL];
+      for (int j = 0; j < NB; ++j) am[v][j] = lane_a[buf * STAGE + ks * KV * A_KS + v * A_KV + j * A_BL];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) bnv[v][i] = lane_b[buf * STAGE + ks * KV * B_KS + v * B_KV + i * B_BL];
+    }
   };
-  auto mfma_step = [&](const T (&am)[NB], const T (&bnv)[NB]) {
+  auto mfma_step = [&](const T (&am)[KV][NB], const T (&bnv)[KV][NB]) {
 #pragma unroll
-    for (int i = 0; i < NB; ++i)
+    for (int v = 0; v < KV; ++v)
 #pragma unroll
-      for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[i], am[j], acc[i][j]);
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[v][i], am[v][j], acc[i][j]);
   };
 
   if (fast && nkt > 0 && nfull == nkt) {
@@ -292,7 +307,7 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     // So every LDS read, LDS write and global load is issued under the shadow of 16 (fp64) / 4 (fp32) MFMAs, and
     // one barrier per panel sits where the MFMA queue still has a k-step of work behind it.  The loop body has
     // no branches: past the end, the loads re-read the last panel and the stores fill a buffer nobody reads.
-    T am[2][NB], bnv[2][NB];
+    T am[2][KV][NB], bnv[2][KV][NB];
     auto fetch_fast = [&](int kt) {
       gload<T, AK, false>(Ab + kt * a_kstep, lda, 0, 0, true, ra, tid);
       gload<T, BKM, false>(Bb + kt * b_kstep, ldb, 0, 0, true, rb, tid);
@@ -305,7 +320,7 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     read_ops(0, 0, am[0], bnv[0]);
     constexpr int NV = Tr::NV, SIDE = 4 * NV;              // 2*NV LDS stores, then 2*NV global loads
     constexpr int PER_STEP = (SIDE + KS - 2) / (KS - 1);     // side instructions placed in each pre-barrier k-step
-    constexpr int MFMAS = NB * NB;
+    constexpr int MFMAS = KV * NB * NB;
     for (int kt = 0; kt < nkt; ++kt) {
       const int cur = kt & 1;
       T* const nxt_a = smem + (cur ^ 1) * STAGE;
@@ -325,7 +340,7 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
           else if (slot < SIDE) gload_one<T, BKM>(gb, ldb, rb[slot - 3 * NV], tid, slot - 3 * NV);
         }
         mfma_step(am[ks & 1], bnv[ks & 1]);
-        if (MFMAS >= 4 * NB) {
+        if (sizeof(T) == 8) {
           // many short MFMAs per k-step (fp64: 16): operand reads first, then one side instruction after every few MFMAs
           __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
 #pragma unroll
@@ -341,17 +356,24 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
           // few long MFMAs per k-step (fp32: 4 of 64 cycles): one operand read and one side instruction behind each
           // MFMA, so that a wave issues them while its own MFMA occupies the pipe.  With everything in front of the
           // MFMAs the two waves of a SIMD reach their non-MFMA stretch together and the pipe idles (130 -> 138 TFLOP/s).
+          // The NREADS operand reads and PER_STEP side instructions alternate and are spread evenly over the MFMAs.
+          constexpr int EXTRA = NREADS + PER_STEP, BOTH = 2 * (NREADS < PER_STEP ? NREADS : PER_STEP);
 #pragma unroll
           for (int m = 0; m < MFMAS; ++m) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (m < 2 * NB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            constexpr int SPM = (PER_STEP + MFMAS - 1) / MFMAS;  // side instructions per MFMA
 #pragma unroll
-            for (int q = m * SPM; q < (m + 1) * SPM && q < PER_STEP; ++q) {
-              const int slot = ks * PER_STEP + q;
-              if (slot < NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
-              else if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
-              else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            for (int e = 0; e < EXTRA; ++e) {
+              if (e * MFMAS / EXTRA != m) continue;
+              const bool is_read = e < BOTH ? (e % 2 == 0) : (NREADS > PER_STEP);
+              if (is_read) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+              } else {
+                const int q = e < BOTH ? e / 2 : e - NREADS;
+                const int slot = ks * PER_STEP + q;
+                if (slot < NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
+                else if (slot < 2 * NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
+                else if (slot < SIDE) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+              }
             }
           }
         }
@@ -360,14 +382,16 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
       __syncthreads();
       read_ops(cur ^ 1, 0, am[KS & 1], bnv[KS & 1]);
       mfma_step(am[(KS - 1) & 1], bnv[(KS - 1) & 1]);
-      if (MFMAS >= 4 * NB) {
+      if (sizeof(T) == 8) {
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * NB, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
       } else {
 #pragma unroll
         for (int m = 0; m < MFMAS; ++m) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (m < 2 * NB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#pragma unroll
+          for (int e = 0; e < NREADS; ++e)
+            if (e * MFMAS / NREADS == m) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -385,7 +409,7 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
       if (kt + 1 < nkt) fetch(kt + 1);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        T am[NB], bnv[NB];
+        T am[KV][NB], bnv[KV][NB];
         read_ops(cur, ks, am, bnv);
         mfma_step(am, bnv);
       }
@@ -397,17 +421,18 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     }
   }
 
-  // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk))
+  // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk)), or with the paired row rule
+  // C(m0 + wm + NB*idx + j, n0 + wn + NB*drow(r, kk) + i)
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
 #pragma unroll
     for (int r = 0; r < Tr::NACC; ++r) {
-      const int n = wn + i * BLK + Tr::drow(r, kk);
+      const int n = B_PAIR ? wn + NB * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
       if (n < nrem) {
         T* ccol = C + (long)(n0 + n) * ldc + m0;
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
-          const int m = wm + j * BLK + idx;
+          const int m = A_PAIR ? wm + NB * idx + j : wm + j * BLK + idx;
           if (m < mrem) {
             T v = alpha * acc[i][j][r];
             if (beta != T(0)) v += beta * ccol[m];
