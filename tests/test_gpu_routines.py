@@ -125,6 +125,22 @@ def test_dgemm_pool_sweep_picks_different_orders(pkg, L, orc, openblas, blocks, 
     assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 0.7, beta, A, K, M, K, B, K, N, K, C0) < TOL64
 
 
+@pytest.mark.parametrize("order", [1, 10003, 20002, 30002, 40000, 60002, 70001])
+def test_dgemm_with_pinned_order_family(pkg, L, orc, openblas, order, monkeypatch):
+    """Every order family and both eviction policies executed for real (PARALIA_GEMM_ORDER pins the plan) in a pool of
+    24 blocks for a 5 x 4 x 6 tile grid (75 blocks when everything fits); K differs per order so that each call is a
+    new problem for the metadata cache."""
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+    M, N, T = 1200, 1000, 256
+    K = 1500 + order % 97
+    A, B, C0 = rand_f64(M * K, 21), rand_f64(K * N, 22), rand_f64(M * N, 23)
+    ref = openblas_ref(openblas, np.float64, "N", "N", M, N, K, 1.25, -0.5, A, M, B, K, C0, M)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    info = call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.25, -0.5, bA, M, bB, K, bC, M, T=T, cache_limit=24 * T * T * 8)
+    assert info.order_id == order
+    assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.25, 0.5, A, M, K, M, B, K, N, K, C0) < TOL64
+
+
 def test_dgemm_too_little_memory_is_an_error(pkg, L):
     M = N = K = 512
     A = rand_f64(M * K, 1)

@@ -211,3 +211,31 @@ def test_dgemv_autotune(L, pkg, monkeypatch):
     monkeypatch.setenv("PARALIA_T_SELECT", "cocopelia")
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemv", 8192, 8192, 1, b"N", b"N", HOST3, 0, -1, 0, C.byref(info)) == 0
     assert info.selected_by == b"cocopelia-bidirectional" and info.T in (1024, 2048, 4096)
+
+
+def test_gemm_order_can_be_pinned_and_pool_limits_change_the_pick(L, pkg, monkeypatch):
+    """PARALIA_GEMM_ORDER pins the order family / eviction policy when that plan fits the pool; a block pool smaller
+    than the working set makes the search consider the repeated-panel orders (20000+) and the slack-aware eviction
+    policy (40000+), and its prediction can only get worse as the pool shrinks."""
+    info = pkg.atc_info()
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 1024, 0, C.byref(info)) == 0
+    free_pick, free_t = info.order_id, info.pred_t
+    assert free_pick < 40000                       # nothing is evicted: only one policy is tried
+    for order in (1, 10003, 20002, 30004):
+        monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+        assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 1024, 0, C.byref(info)) == 0
+        assert info.order_id == order and info.pred_t >= free_t * (1 - 1e-12)
+    monkeypatch.delenv("PARALIA_GEMM_ORDER")
+    prev = free_t
+    for blocks in (120, 60, 30, 12, 5):
+        limit = blocks * 1024 * 1024 * 8
+        assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 1024, limit, C.byref(info)) == 0
+        assert info.pred_t >= prev * (1 - 1e-9), (blocks, info.pred_t, prev)
+        prev = info.pred_t
+    assert info.pred_t > free_t                    # five blocks: nearly every subkernel fetches both operands again
+    # an order that needs more blocks than the pool has is not forced: the search result stands
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", "8")  # 8 column tiles as one k-outer panel: 64 accumulators at least
+    assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 1024, 5 * 1024 * 1024 * 8, C.byref(info)) == 0
+    assert info.order_id != 8
