@@ -25,9 +25,9 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 FP64_MFMA_PEAK = 78.6e12   # MI355X dense FP64 matrix peak, FLOP/s
 HBM_PEAK = 8.0e12          # MI355X HBM3E peak, B/s
 # HBM bytes of one 16384^3 launch of the tile kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
-# daxpy of known size: FETCH_SIZE 50,801,693 KiB x 2.0 + WRITE_SIZE 2,097,152 KiB x 1.0
+# daxpy of known size: FETCH_SIZE 50,324,042 KiB x 2.0 + WRITE_SIZE 2,097,152 KiB x 1.0
 # (profiles/dgemm_16384_daxpy_2p28_pmc_hbm_traffic.txt).
-GEMM_TRAFFIC_BYTES = 1.0619e11
+GEMM_TRAFFIC_BYTES = 1.0521e11
 
 
 def load_package():
