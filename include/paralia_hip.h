@@ -161,9 +161,8 @@ int PARALiA_dev_cache_free(int dev_id);
 /* metadata-cache and pool counters (PMD_cache, dgemm.cpp:342-368); reset drops the cached problems */
 int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries);
 int PARALiA_runtime_reset(void);
-/* which of the four stream-to-hardware-queue alignments the scheduler used last, and whether that one was settled
- * (every large streamed GEMM problem tries the four on its first four repeat calls and keeps its best); no
- * counterpart in the reference */
+/* which of the four stream-to-hardware-queue alignments the scheduler uses, and whether its start-up trial of
+ * them (first four large streamed GEMM calls) is over; no counterpart in the reference */
 int PARALiA_stream_rotation(int* rotation, int* settled);
 /* directory holding Processed/ lookup tables and link models (DEPLOYDB, CMakeLists.txt:376) */
 int PARALiA_set_db_dir(const char* dir);

@@ -70,13 +70,13 @@ struct Resources {
   // one runs the streamed 16384^3 fp64 GEMM in 130 ms, the others in 148-169 ms.  The alignment depends on how
   // many streams the application created before this library did, which cannot be queried.  So seven streams
   // are created back to back, "rotation" r uses streams r .. r+3 as (H2D, D2H, compute 0, compute 1), and
-  // the first four calls that repeat an already tuned large streamed GEMM each run under a different rotation; the
-  // fastest is kept for that problem (which alignment wins depends on whether the two compute streams or the two
-  // copy streams are the busy pair: dgemm 40000 x 40000 x 2048 loses 4 % under the alignment that is best for
-  // 16384^3).  PARALIA_STREAM_ROTATION=r skips the trials.  With 8 or more hardware queues all rotations are equal.
+  // the first four large streamed GEMM calls that repeat an already tuned problem each run under a different
+  // rotation; the fastest is kept
+  // (PARALIA_STREAM_ROTATION=r skips the trial).  With 8 or more hardware queues all rotations are equal.
   void* ring[7] = {nullptr};
   int rotation = 0;
-  bool rotation_pinned = false;
+  int trials = 0;            // rotations tried so far; 4 = settled
+  double trial_rate[4] = {0, 0, 0, 0};
   void set_rotation(int r) {
     rotation = r;
     h2d = ring[r];
@@ -89,10 +89,28 @@ struct Resources {
       for (void*& s : ring) chk(pl_stream_create(&s), "stream create");
       nexec = 2;
       const char* env = getenv("PARALIA_STREAM_ROTATION");
-      rotation_pinned = env && atoi(env) >= 0 && atoi(env) < 4;
-      set_rotation(rotation_pinned ? atoi(env) : 0);
+      if (env && atoi(env) >= 0 && atoi(env) < 4) {
+        set_rotation(atoi(env));
+        trials = 4;
+      } else {
+        set_rotation(0);
+      }
     }
     for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
+  }
+  // Called around a large streamed GEMM: picks the rotation to try, then records seconds per flop.
+  void begin_trial() {
+    if (trials < 4) set_rotation(trials);
+  }
+  void end_trial(double seconds_per_flop) {
+    if (trials >= 4) return;
+    trial_rate[trials++] = seconds_per_flop;
+    if (trials == 4) {
+      int best = 0;
+      for (int r = 1; r < 4; ++r)
+        if (trial_rate[r] < trial_rate[best]) best = r;
+      set_rotation(best);
+    }
   }
   void ensure_events(size_t n) {
     while (events.size() < n) {
@@ -164,10 +182,6 @@ struct PMDEntry {
   PMDKey key;
   std::unique_ptr<ATC> atc;
   GemmPlan plan;
-  // stream alignment of this problem (see Resources::ring): rotations tried so far, their rates, and the pick
-  int rot_trials = 0;
-  double rot_rate[4] = {0, 0, 0, 0};
-  int rotation = -1;
 };
 
 struct Runtime {
@@ -426,24 +440,13 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     const GemmPlan& plan = entry->plan;
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T));
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
-    // Stream alignment: a large plan tries the four rotations on its first four repeat calls (the first call of a
-    // problem also pays for fresh pool memory and cold caches and would misjudge its rotation), then keeps its best.
-    const bool large = plan.cmds.size() >= 64 && !no_ab && !R.res.rotation_pinned;
-    const bool trial = large && entry->rot_trials < 4 && !cold;
-    if (trial) R.res.set_rotation(entry->rot_trials);
-    else if (large && entry->rotation >= 0) R.res.set_rotation(entry->rotation);
+    // a first call of a problem also pays for fresh pool memory and cold caches: it would misjudge its rotation
+    const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab && !cold;
+    if (trial) R.res.begin_trial();
     const double t0 = csecond();
     const bool pageable[3] = {locA == -2, locB == -2, locC == -2};
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC, pageable);
-    if (trial) {
-      entry->rot_rate[entry->rot_trials++] = csecond() - t0;
-      if (entry->rot_trials == 4) {
-        entry->rotation = 0;
-        for (int r = 1; r < 4; ++r)
-          if (entry->rot_rate[r] < entry->rot_rate[entry->rotation]) entry->rotation = r;
-        R.res.set_rotation(entry->rotation);
-      }
-    }
+    if (trial) R.res.end_trial((csecond() - t0) / (2.0 * M * N * (double)K));
   }
   return atc_copy(atc);
 }
@@ -789,12 +792,7 @@ void stream_rotation(int* rotation, int* settled) {
   Runtime& R = rt();
   std::lock_guard<std::mutex> lk(R.mu);
   if (rotation) *rotation = R.res.rotation;
-  // settled: the alignment in use was pinned by the environment or picked by the problem that ran last
-  if (settled) {
-    *settled = R.res.rotation_pinned ? 1 : 0;
-    for (const auto& e : R.pmd)
-      if (e->rotation == R.res.rotation && e->rot_trials == 4) *settled = 1;
-  }
+  if (settled) *settled = R.res.trials >= 4 ? 1 : 0;
 }
 
 void runtime_reset() {
