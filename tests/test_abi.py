@@ -1,6 +1,8 @@
 """The C ABI: the library loads, exports every symbol include/paralia_hip.h declares, and its argument checks
 answer with status codes before anything touches a GPU."""
 import ctypes as C
+
+import pytest
 import os
 import re
 
@@ -103,3 +105,29 @@ def test_split_k_workspace_sizing(L):
         s = b // (M * N * esz)
         assert 2 <= s <= 64 and K / s >= 112 and b <= 256 << 20
     assert L.pl_gemm_tile_workspace_bytes(1024, 1024, 1024, 8) == 4 * 1024 * 1024 * 8
+
+
+def test_runner_row_is_readable_by_the_reference_plotters(pkg, tmp_path):
+    """The reference's plotting scripts read runner logs with pandas: no header, skipinitialspace, 18 columns of which
+    0-5, 8-13 and 15-17 are used (T, units, unit token, cache / ratio, TransA, TransB, M, N, K, the three locations and
+    three timings: Benchmarking/Python_Scripts/CoCoPeLiA_plotters/input_parsing.py:41-47).  A row written by the
+    predictor driver must come through that call with the right types."""
+    import os
+    import subprocess
+    pd = pytest.importorskip("pandas")
+    exe = os.path.join(os.path.dirname(pkg.LIB_PATH), "..", "bin", "dgemm_predictor")
+    if not os.path.exists(exe):
+        pytest.skip("driver executables not built")
+    env = dict(os.environ, PARALIA_TESTLIBDIR=str(tmp_path))
+    for args in ("1 1 2048 -1 N T 1.0 0.5 8192 4096 2048 -1 0 -1 -1", "1 1 1024 -1 T N 1.0 0.5 4096 4096 4096 -1 -1 -1 -1"):
+        run = subprocess.run([exe] + args.split(), env=env, capture_output=True, text=True, timeout=120)
+        assert run.returncode == 0, run.stderr
+    log = next(tmp_path.glob("CoCoPeLiaDgemmPredictor_predefined_vals_MI355X_*.log"))
+    names = ["T", "dev_num", "dev_ids_token", "cpu_ratio", "TransA", "TransB", "M", "N", "K", "Aloc", "Bloc", "Cloc", "t0", "t1", "t2"]
+    df = pd.read_csv(log, header=None, skipinitialspace=True, names=names, usecols=[0, 1, 2, 3, 4, 5, 8, 9, 10, 11, 12, 13, 15, 16, 17],
+                     dtype={"T": int, "dev_num": int, "dev_ids_token": int, "TransA": str, "TransB": str, "M": int, "N": int, "K": int,
+                            "Aloc": int, "Bloc": int, "Cloc": int, "t0": float, "t1": float, "t2": float})
+    assert len(df) == 2
+    assert list(df["T"]) == [2048, 1024] and list(df["TransA"]) == ["N", "T"] and list(df["TransB"]) == ["T", "N"]
+    assert list(df["M"]) == [8192, 4096] and list(df["N"]) == [4096, 4096] and list(df["K"]) == [2048, 4096]
+    assert list(df["Bloc"]) == [0, -1] and (df["t1"] > 0).all()
