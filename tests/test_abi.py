@@ -1,10 +1,10 @@
 """The C ABI: the library loads, exports every symbol include/paralia_hip.h declares, and its argument checks
 answer with status codes before anything touches a GPU."""
 import ctypes as C
-
-import pytest
 import os
 import re
+
+import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
