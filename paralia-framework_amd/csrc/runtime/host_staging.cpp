@@ -99,7 +99,7 @@ HostStager::~HostStager() {
 CopyThreads* HostStager::threads() {
   if (!pool_) {
     const char* env = getenv("PARALIA_COPY_THREADS");
-    int n = env && atoi(env) > 0 ? atoi(env) : (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()));
+    int n = env && atoi(env) > 0 ? atoi(env) : (int)std::min(4u, std::max(1u, std::thread::hardware_concurrency()));
     pool_ = new CopyThreads(std::min(n, 64));
   }
   return pool_;
