@@ -4,10 +4,13 @@
 // cublasDgemm / cublasSgemm through backend_run_operation (Library_scheduler/src/Subkernel.cpp:168,228;
 // direct call form Database_builder/CuCuBLAS/src/dgemm_microbench.cu:141-142).  Here it is a hand-written
 // MFMA kernel:
-//   * one workgroup = 256 threads = 4 wavefronts (2 x 2), macro tile 128 x 128, each wave owns 64 x 64;
-//   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2);
-//   * A and B k-panels (16 elements deep) are staged global -> registers -> LDS, double-buffered,
-//     one barrier per k-panel; the next panel's global loads are in flight while the current one is multiplied;
+//   * one workgroup = 256 threads = 4 wavefronts (2 x 2), macro tile 128 x 128 (each wave owns 64 x 64, two
+//     workgroups per CU), and for fp32 also 256 x 256 (each wave owns 128 x 128 with 256 accumulator registers, one
+//     workgroup per CU) for problems with enough such tiles to fill the CUs;
+//   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2 or 4 x 4);
+//   * A and B k-panels (16 elements deep, 32 for the large tile) are staged global -> registers -> LDS,
+//     double-buffered, one barrier per k-panel; the next panel's global loads are in flight while the current one is
+//     multiplied;
 //   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
 //     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
@@ -17,19 +20,14 @@
 // leading dimension allow it and the workgroup's tile is interior, element loads with zero fill otherwise.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 // Row index (MFMA i) of accumulator element r for lane group g = lane / 16 in the 16x16 fp64 result block.
 #ifndef PLK_F64_BK
 #define PLK_F64_BK 16
 #endif
-#ifndef PLK_WAVES_PER_EU
-#define PLK_WAVES_PER_EU 2
-#endif
 #ifndef PLK_F32_BK
 #define PLK_F32_BK 16
-#endif
-#ifndef PLK_F32_WAVES_PER_EU
-#define PLK_F32_WAVES_PER_EU 2
 #endif
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
@@ -42,7 +40,10 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef double dvec2 __attribute__((ext_vector_type(2)));
 typedef float fvec4 __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 128, BN = 128, NTHREADS = 256, WM = 64, WN = 64;
+constexpr int NTHREADS = 256;
+#ifndef PLK_F32_BIG_BK
+#define PLK_F32_BIG_BK 32
+#endif
 
 template <typename T> struct Traits;
 
@@ -50,15 +51,11 @@ template <> struct Traits<double> {
   using vec_t = dvec2;
   using acc_t = double4_t;
   static constexpr int VEC = 2;      // elements per 16-byte vector
-  static constexpr int BK = PLK_F64_BK;  // k-panel depth
-  static constexpr int WAVES = PLK_WAVES_PER_EU;  // wavefronts per SIMD the register budget is sized for
   static constexpr int BLK = 16;     // MFMA block edge
   static constexpr int KSTEP = 4;    // k consumed per MFMA
   static constexpr int KV = 1;       // MFMA k-steps served by one refresh of the operand registers
   static constexpr int NACC = 4;     // accumulator elements per lane per block
-  static constexpr int S_MN = 144;   // LDS row stride, [k][mn] layout (1152 B = 128 mod 256)
-  static constexpr int S_K = BK + 2; // LDS row stride, [mn][k] layout
-  static constexpr int NV = 128 * BK / VEC / 256;  // 16-byte vectors per thread per panel
+  static constexpr int PAD_MN = 16;  // [k][mn] rows are extent + PAD_MN elements apart (128 B past a multiple of 256 B)
   static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
@@ -70,53 +67,51 @@ template <> struct Traits<float> {
   using vec_t = fvec4;
   using acc_t = float16_t;
   static constexpr int VEC = 4;
-  static constexpr int BK = PLK_F32_BK;
-  static constexpr int WAVES = PLK_F32_WAVES_PER_EU;
   static constexpr int BLK = 32;
   static constexpr int KSTEP = 2;
   static constexpr int KV = 2;       // two k-steps per refresh: their operands come with one LDS instruction
   static constexpr int NACC = 16;
-  static constexpr int S_MN = 160;   // 640 B = 128 mod 256
-  // 18 words: lane (idx, kk) of an operand read sits in bank (18 * idx + kk) mod 64, all 64 distinct.  Rows are then
-  // only 8-byte aligned, so a 16-byte vector goes to LDS as two 8-byte stores (lds_put).  A 16-byte aligned stride
-  // (20 words) costs two-way conflicts on every operand read (measured: conflict cycles 54 % -> 33 % of the LDS
-  // cycles, the rest comes from the stores; worth 1 % on TN, nothing on NN: LDS is not what limits these variants).
-  static constexpr int S_K = BK + 2;
-  static constexpr int NV = 128 * BK / VEC / 256;
+  static constexpr int PAD_MN = 32;
   static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ int drow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
 };
 
-template <typename T, bool KMAJOR> struct Lds {
+// One staged operand panel: EXT rows or columns of op(X) by BK values of k.
+// [mn][k] layout (K-major operands): rows BK + 2 elements apart.  fp32: lane (idx, kk) of an operand read sits in bank
+// ((BK + 2) * idx + kk) mod 64, all distinct; rows are then only 8-byte aligned, so a 16-byte vector goes to LDS as two
+// 8-byte stores (lds_put).  A 16-byte aligned stride costs two-way conflicts on every operand read.
+template <typename T, bool KMAJOR, int EXT, int BK> struct Lds {
   using Tr = Traits<T>;
-  // elements of one staged panel (128 x BK plus padding)
-  static constexpr int SIZE = KMAJOR ? 128 * Tr::S_K : Tr::BK * Tr::S_MN;
-  static constexpr __host__ __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * Tr::S_K + k : k * Tr::S_MN + mn; }
-};
-
-// One thread's share of a 128 x BK panel: NV 16-byte vectors.  "c" runs along the memory-contiguous
-// dimension (mn for MN-major operands, k for K-major ones), "s" along the leading-dimension stride.
-template <typename T, bool KMAJOR> struct Slot {
-  using Tr = Traits<T>;
-  static constexpr int CVECS = (KMAJOR ? Tr::BK : 128) / Tr::VEC;  // vectors per contiguous run
+  static constexpr int S_K = BK + 2, S_MN = EXT + Tr::PAD_MN;
+  static constexpr int SIZE = KMAJOR ? EXT * S_K : BK * S_MN;  // elements, padding included
+  static constexpr int NV = EXT * BK / Tr::VEC / NTHREADS;     // 16-byte vectors per thread per panel
+  static constexpr __host__ __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * S_K + k : k * S_MN + mn; }
+  // Vector i of thread tid: "c" runs along the memory-contiguous dimension (mn for MN-major operands, k for K-major
+  // ones), "s" along the leading-dimension stride.
+  static constexpr int CVECS = (KMAJOR ? BK : EXT) / Tr::VEC;  // vectors per contiguous run
   static __device__ __forceinline__ void coords(int tid, int i, int& c, int& s) {
     int v = tid + NTHREADS * i;
     c = (v % CVECS) * Tr::VEC;
     s = v / CVECS;
   }
+  static __device__ __forceinline__ int slot_offset(int tid, int i) {
+    int c, s;
+    coords(tid, i, c, s);
+    return KMAJOR ? at(c, s) : at(s, c);  // the contiguous run is also contiguous in LDS for both layouts
+  }
 };
 
-template <typename T, bool KMAJOR, bool GUARD>
+template <typename L, typename T, bool GUARD>
 __device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int crem, int srem, bool vec_ok,
-                                      typename Traits<T>::vec_t (&regs)[Traits<T>::NV], int tid) {
+                                      typename Traits<T>::vec_t (&regs)[L::NV], int tid) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
 #pragma unroll
-  for (int i = 0; i < Tr::NV; ++i) {
+  for (int i = 0; i < L::NV; ++i) {
     int c, s;
-    Slot<T, KMAJOR>::coords(tid, i, c, s);
+    L::coords(tid, i, c, s);
     const T* p = base + c + (long)s * ld;
     if (!GUARD) {
       regs[i] = *reinterpret_cast<const vec_t*>(p);
@@ -139,10 +134,10 @@ __device__ __forceinline__ void gload(const T* __restrict__ base, long ld, int c
 }
 
 // Slot i only, unguarded: the pieces the pipelined loop spreads between MFMAs.
-template <typename T, bool KMAJOR>
+template <typename L, typename T>
 __device__ __forceinline__ void gload_one(const T* __restrict__ base, long ld, typename Traits<T>::vec_t& reg, int tid, int i) {
   int c, s;
-  Slot<T, KMAJOR>::coords(tid, i, c, s);
+  L::coords(tid, i, c, s);
   reg = *reinterpret_cast<const typename Traits<T>::vec_t*>(base + c + (long)s * ld);
 }
 typedef float fvec2 __attribute__((ext_vector_type(2)));
@@ -161,26 +156,15 @@ __device__ __forceinline__ void lds_put(T* __restrict__ p, const typename Traits
   }
 }
 
-template <typename T, bool KMAJOR>
+template <typename L, typename T, bool KMAJOR>
 __device__ __forceinline__ void lds_store_one(T* __restrict__ xs, const typename Traits<T>::vec_t& reg, int tid, int i) {
-  int c, s;
-  Slot<T, KMAJOR>::coords(tid, i, c, s);
-  const int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
-  lds_put<T, KMAJOR>(xs + off, reg);
+  lds_put<T, KMAJOR>(xs + L::slot_offset(tid, i), reg);
 }
 
-template <typename T, bool KMAJOR>
-__device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[Traits<T>::NV], int tid) {
-  using Tr = Traits<T>;
-  using vec_t = typename Tr::vec_t;
+template <typename L, typename T, bool KMAJOR>
+__device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[L::NV], int tid) {
 #pragma unroll
-  for (int i = 0; i < Tr::NV; ++i) {
-    int c, s;
-    Slot<T, KMAJOR>::coords(tid, i, c, s);
-    // the contiguous run is also contiguous in LDS for both layouts
-    int off = KMAJOR ? Lds<T, true>::at(c, s) : Lds<T, false>::at(s, c);
-    lds_put<T, KMAJOR>(xs + off, regs[i]);
-  }
+  for (int i = 0; i < L::NV; ++i) lds_put<T, KMAJOR>(xs + L::slot_offset(tid, i), regs[i]);
 }
 
 // Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
@@ -200,15 +184,20 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
   bn = in / gsz;
 }
 
+// Macro tile BM x BN, four waves in 2 x 2, each owning BM/2 x BN/2; k-panels BK deep.  Tiles with 128 x 128 leave room
+// for two workgroups per CU (two waves per SIMD that fill each other's gaps); larger ones run one workgroup per CU with
+// the whole register file and fewer operand reads and global loads per MFMA.
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
-template <typename T, bool AK, bool BKM>
-__global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
+template <typename T, bool AK, bool BKM, int BM, int BN, int BK>
+__global__ __launch_bounds__(NTHREADS, (BM * BN <= 128 * 128 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
                                                           long ldc, int gm, int gn, int vecA, int vecB, int kchunk) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
   using acc_t = typename Tr::acc_t;
-  constexpr int BK = Tr::BK, BLK = Tr::BLK, NB = WM / BLK;
+  using LA = Lds<T, AK, BM, BK>;
+  using LB = Lds<T, BKM, BN, BK>;
+  constexpr int BLK = Tr::BLK, WM = BM / 2, WN = BN / 2, NBM = WM / BLK, NBN = WN / BLK;
   if (kchunk > 0) {
     // split K: the workgroups of grid row y multiply k in [y * kchunk, (y + 1) * kchunk) and leave their plain partial
     // product in slice y of the workspace passed as C (M x N, dense); splitk_reduce_kernel combines the slices
@@ -218,7 +207,7 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     K = min(K - k0, kchunk);
     C += (long)blockIdx.y * M * N;
   }
-  constexpr int ASZ = Lds<T, AK>::SIZE, BSZ = Lds<T, BKM>::SIZE;
+  constexpr int ASZ = LA::SIZE, BSZ = LB::SIZE;
 
   __shared__ __attribute__((aligned(16))) T smem[2 * (ASZ + BSZ)];
   constexpr int STAGE = ASZ + BSZ;  // buffer b holds A at smem + b*STAGE and B right behind it
@@ -240,61 +229,61 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
   const long a_kstep = AK ? (long)BK : (long)BK * lda;
   const long b_kstep = BKM ? (long)BK : (long)BK * ldb;
 
-  acc_t acc[NB][NB];
+  acc_t acc[NBN][NBM];
 #pragma unroll
-  for (int i = 0; i < NB; ++i)
+  for (int i = 0; i < NBN; ++i)
 #pragma unroll
-    for (int j = 0; j < NB; ++j)
+    for (int j = 0; j < NBM; ++j)
 #pragma unroll
       for (int r = 0; r < Tr::NACC; ++r) acc[i][j][r] = T(0);
 
   const int nkt = (K + BK - 1) / BK;
   const int nfull = K / BK;
-  vec_t ra[Tr::NV], rb[Tr::NV];
+  constexpr int NVA = LA::NV, NVB = LB::NV;
+  vec_t ra[NVA], rb[NVB];
 
   auto fetch = [&](int kt) {
     const T* ap = Ab + kt * a_kstep;
     const T* bp = Bb + kt * b_kstep;
     if (fast && kt < nfull) {
-      gload<T, AK, false>(ap, lda, 0, 0, true, ra, tid);
-      gload<T, BKM, false>(bp, ldb, 0, 0, true, rb, tid);
+      gload<LA, T, false>(ap, lda, 0, 0, true, ra, tid);
+      gload<LB, T, false>(bp, ldb, 0, 0, true, rb, tid);
     } else {
       const int krem = min(K - kt * BK, BK);
-      gload<T, AK, true>(ap, lda, AK ? krem : mrem, AK ? mrem : krem, vecA, ra, tid);
-      gload<T, BKM, true>(bp, ldb, BKM ? krem : nrem, BKM ? nrem : krem, vecB, rb, tid);
+      gload<LA, T, true>(ap, lda, AK ? krem : mrem, AK ? mrem : krem, vecA, ra, tid);
+      gload<LB, T, true>(bp, ldb, BKM ? krem : nrem, BKM ? nrem : krem, vecB, rb, tid);
     }
   };
 
   // fp32 operands in the [k][mn] layout: lane idx of block j takes row NB * idx + j instead of j * BLK + idx, so the
-  // rows a lane needs for its NB blocks are adjacent in LDS and come with one 8-byte read instead of NB 4-byte ones
-  // (every operand read issued between MFMAs costs MFMA issue slots: 1 read per MFMA loses 8 % of the pipe rate,
+  // rows a lane needs for its NB blocks are adjacent in LDS and come with one 8- or 16-byte read instead of NB 4-byte
+  // ones (every operand read issued between MFMAs costs MFMA issue slots: 1 read per MFMA loses 8 % of the pipe rate,
   // 1 per 2 about half of that).  The epilogue maps the accumulators back with the same rule.
   constexpr bool A_PAIR = sizeof(T) == 4 && !AK, B_PAIR = sizeof(T) == 4 && !BKM;
-  const T* const lane_a = smem + Lds<T, AK>::at(kk, wm + (A_PAIR ? NB * idx : idx));         // this lane's A operand of k-step 0, block 0
-  const T* const lane_b = smem + ASZ + Lds<T, BKM>::at(kk, wn + (B_PAIR ? NB * idx : idx));  // this lane's B operand
-  constexpr int A_KS = Lds<T, AK>::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : Lds<T, AK>::at(0, BLK);    // strides per k-step / per block
-  constexpr int B_KS = Lds<T, BKM>::at(Tr::KSTEP, 0), B_BL = B_PAIR ? 1 : Lds<T, BKM>::at(0, BLK);
-  constexpr int NREADS = (A_PAIR ? 1 : NB) + (B_PAIR ? 1 : NB);  // LDS read instructions per k-step
+  const T* const lane_a = smem + LA::at(kk, wm + (A_PAIR ? NBM * idx : idx));         // this lane's A operand of k-step 0, block 0
+  const T* const lane_b = smem + ASZ + LB::at(kk, wn + (B_PAIR ? NBN * idx : idx));  // this lane's B operand
+  constexpr int A_KS = LA::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : LA::at(0, BLK);    // strides per k-step / per block
+  constexpr int B_KS = LB::at(Tr::KSTEP, 0), B_BL = B_PAIR ? 1 : LB::at(0, BLK);
+  constexpr int NREADS = (A_PAIR ? 1 : NBM) + (B_PAIR ? 1 : NBN);  // LDS read instructions per k-step
   constexpr int KV = Tr::KV;
   constexpr int KS = BK / (Tr::KSTEP * KV);  // operand refreshes ("steps") per panel
-  constexpr int A_KV = Lds<T, AK>::at(Tr::KSTEP, 0), B_KV = Lds<T, BKM>::at(Tr::KSTEP, 0);  // k-step stride inside a step
 
-  auto read_ops = [&](int buf, int ks, T (&am)[KV][NB], T (&bnv)[KV][NB]) {
+  auto read_ops = [&](int buf, int ks, T (&am)[KV][NBM], T (&bnv)[KV][NBN]) {
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
 #pragma unroll
-      for (int j = 0; j < NB; ++j) am[v][j] = lane_a[buf * STAGE + ks * KV * A_KS + v * A_KV + j * A_BL];
+      for (int j = 0; j < NBM; ++j) am[v][j] = lane_a[buf * STAGE + (ks * KV + v) * A_KS + j * A_BL];
 #pragma unroll
-      for (int i = 0; i < NB; ++i) bnv[v][i] = lane_b[buf * STAGE + ks * KV * B_KS + v * B_KV + i * B_BL];
+      for (int i = 0; i < NBN; ++i) bnv[v][i] = lane_b[buf * STAGE + (ks * KV + v) * B_KS + i * B_BL];
     }
   };
-  auto mfma_step = [&](const T (&am)[KV][NB], const T (&bnv)[KV][NB]) {
+  auto mfma_step = [&](const T (&am)[KV][NBM], const T (&bnv)[KV][NBN]) {
 #pragma unroll
     for (int v = 0; v < KV; ++v)
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+      for (int i = 0; i < NBN; ++i)
 #pragma unroll
-        for (int j = 0; j < NB; ++j) acc[i][j] = Tr::mfma(bnv[v][i], am[v][j], acc[i][j]);
+        for (int j = 0; j < NBM; ++j) acc[i][j] = Tr::mfma(bnv[v][i], am[v][j], acc[i][j]);
   };
 
   if (fast && nkt > 0 && nfull == nkt) {
@@ -304,23 +293,23 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     //   k-steps 1..  : read the operands of the next k-step while multiplying the current one;
     //   last k-step  : barrier first (everyone is done reading buffer cur and writing buffer cur^1), read the
     //                  operands of panel kt+1's first k-step, multiply the last operands of panel kt.
-    // So every LDS read, LDS write and global load is issued under the shadow of 16 (fp64) / 4 (fp32) MFMAs, and
-    // one barrier per panel sits where the MFMA queue still has a k-step of work behind it.  The loop body has
-    // no branches: past the end, the loads re-read the last panel and the stores fill a buffer nobody reads.
-    T am[2][KV][NB], bnv[2][KV][NB];
+    // So every LDS read, LDS write and global load is issued under the shadow of MFMAs, and one barrier per panel sits
+    // where the MFMA queue still has a k-step of work behind it.  The loop body has no branches: past the end, the
+    // loads re-read the last panel and the stores fill a buffer nobody reads.
+    T am[2][KV][NBM], bnv[2][KV][NBN];
     auto fetch_fast = [&](int kt) {
-      gload<T, AK, false>(Ab + kt * a_kstep, lda, 0, 0, true, ra, tid);
-      gload<T, BKM, false>(Bb + kt * b_kstep, ldb, 0, 0, true, rb, tid);
+      gload<LA, T, false>(Ab + kt * a_kstep, lda, 0, 0, true, ra, tid);
+      gload<LB, T, false>(Bb + kt * b_kstep, ldb, 0, 0, true, rb, tid);
     };
     fetch_fast(0);
-    lds_store<T, AK>(smem, ra, tid);
-    lds_store<T, BKM>(smem + ASZ, rb, tid);
+    lds_store<LA, T, AK>(smem, ra, tid);
+    lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
     fetch_fast(min(1, nkt - 1));
     __syncthreads();
     read_ops(0, 0, am[0], bnv[0]);
-    constexpr int NV = Tr::NV, SIDE = 4 * NV;              // 2*NV LDS stores, then 2*NV global loads
+    constexpr int NVS = NVA + NVB, SIDE = 2 * NVS;           // NVS LDS stores and NVS global loads per panel
     constexpr int PER_STEP = (SIDE + KS - 2) / (KS - 1);     // side instructions placed in each pre-barrier k-step
-    constexpr int MFMAS = KV * NB * NB;
+    constexpr int MFMAS = KV * NBM * NBN;
     constexpr bool ALT = sizeof(T) == 8;
     for (int kt = 0; kt < nkt; ++kt) {
       const int cur = kt & 1;
@@ -339,14 +328,14 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
           // side instruction number "slot" of the panel: fp64 alternates store / load vector by vector (the load
           // refills the registers the store has just read), fp32 issues all stores first, then all loads;
           // measured at 8192^3: fp64 73.5 against 72.0 TFLOP/s, fp32 141.3 against 139.9 the other way round
-          const bool is_store = ALT ? (slot % 2 == 0) : (slot < 2 * NV);
-          const int vec = ALT ? slot / 2 : (slot < 2 * NV ? slot : slot - 2 * NV);  // 0 .. NV-1: A, NV .. 2NV-1: B
+          const bool is_store = ALT ? (slot % 2 == 0) : (slot < NVS);
+          const int vec = ALT ? slot / 2 : (slot < NVS ? slot : slot - NVS);  // 0 .. NVA-1: A, NVA .. NVS-1: B
           if (is_store) {
-            if (vec < NV) lds_store_one<T, AK>(nxt_a, ra[vec], tid, vec);
-            else lds_store_one<T, BKM>(nxt_b, rb[vec - NV], tid, vec - NV);
+            if (vec < NVA) lds_store_one<LA, T, AK>(nxt_a, ra[vec], tid, vec);
+            else lds_store_one<LB, T, BKM>(nxt_b, rb[vec - NVA], tid, vec - NVA);
           } else {
-            if (vec < NV) gload_one<T, AK>(ga, lda, ra[vec], tid, vec);
-            else gload_one<T, BKM>(gb, ldb, rb[vec - NV], tid, vec - NV);
+            if (vec < NVA) gload_one<LA, T>(ga, lda, ra[vec], tid, vec);
+            else gload_one<LB, T>(gb, ldb, rb[vec - NVA], tid, vec - NVA);
           }
         }
         mfma_step(am[ks & 1], bnv[ks & 1]);
@@ -368,10 +357,10 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
             } else {
               const int slot = ks * PER_STEP + (e < BOTH ? e / 2 : e - NREADS);
               if (slot >= SIDE) continue;
-              const bool is_store = ALT ? (slot % 2 == 0) : (slot < 2 * NV);
-              const int vec = ALT ? slot / 2 : (slot < 2 * NV ? slot : slot - 2 * NV);
+              const bool is_store = ALT ? (slot % 2 == 0) : (slot < NVS);
+              const int vec = ALT ? slot / 2 : (slot < NVS ? slot : slot - NVS);
               if (!is_store) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-              else if (vec < NV) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
+              else if (vec < NVA) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
               else __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
             }
           }
@@ -394,8 +383,8 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
     // General loop: edge workgroups, ragged K, unaligned operands.  Same double buffering, loads guarded.
     if (nkt > 0) {
       fetch(0);
-      lds_store<T, AK>(smem, ra, tid);
-      lds_store<T, BKM>(smem + ASZ, rb, tid);
+      lds_store<LA, T, AK>(smem, ra, tid);
+      lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
     }
     __syncthreads();
     for (int kt = 0; kt < nkt; ++kt) {
@@ -403,30 +392,30 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
       if (kt + 1 < nkt) fetch(kt + 1);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        T am[KV][NB], bnv[KV][NB];
+        T am[KV][NBM], bnv[KV][NBN];
         read_ops(cur, ks, am, bnv);
         mfma_step(am, bnv);
       }
       if (kt + 1 < nkt) {
-        lds_store<T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
-        lds_store<T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
+        lds_store<LA, T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
+        lds_store<LB, T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
       }
       __syncthreads();
     }
   }
 
   // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk)), or with the paired row rule
-  // C(m0 + wm + NB*idx + j, n0 + wn + NB*drow(r, kk) + i)
+  // C(m0 + wm + NBM*idx + j, n0 + wn + NBN*drow(r, kk) + i)
 #pragma unroll
-  for (int i = 0; i < NB; ++i) {
+  for (int i = 0; i < NBN; ++i) {
 #pragma unroll
     for (int r = 0; r < Tr::NACC; ++r) {
-      const int n = B_PAIR ? wn + NB * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
+      const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
       if (n < nrem) {
         T* ccol = C + (long)(n0 + n) * ldc + m0;
 #pragma unroll
-        for (int j = 0; j < NB; ++j) {
-          const int m = A_PAIR ? wm + NB * idx + j : wm + j * BLK + idx;
+        for (int j = 0; j < NBM; ++j) {
+          const int m = A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx;
           if (m < mrem) {
             T v = alpha * acc[i][j][r];
             if (beta != T(0)) v += beta * ccol[m];
@@ -438,7 +427,6 @@ __global__ __launch_bounds__(NTHREADS, Traits<T>::WAVES) void gemm_kernel(int M,
   }
 }
 
-// C = beta * C on an M x N column-major view (alpha == 0 or K == 0: A and B are not referenced).
 template <typename T>
 __global__ void scale_kernel(int M, int N, T beta, T* __restrict__ C, long ldc) {
   const long total = (long)M * N;
@@ -468,6 +456,7 @@ __global__ void splitk_reduce_kernel(int M, int N, int splits, T alpha, const T*
 // the pass that adds the slices (workspace written once and read once).  1 = do not split.
 template <typename T>
 int pick_splits(long M, long N, long K, int* kchunk_out) {
+  constexpr int BM = 128, BN = 128;
   const long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   *kchunk_out = 0;
   // with more than about half the compute units covered, a second product running on another stream (the way the
@@ -514,26 +503,52 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (!A || !B || !C) return 5;
-  const int gm = (int)((M + BM - 1) / BM), gn = (int)((N + BN - 1) / BN);
-  if ((long)gm * gn > INT32_MAX) return 2;
-  const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
-  const int vecB = ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % Tr::VEC == 0) ? 1 : 0;
   int kchunk = 0;
   int splits = workspace ? pick_splits<T>(M, N, K, &kchunk) : 1;
   if (splits > 1 && (long)splits * M * N * (long)sizeof(T) > workspace_bytes) splits = 1, kchunk = 0;
+  // fp32: 256 x 256 macro tiles when the model below says they are faster.  Their inner loop runs 2 - 6 % faster per k
+  // (half the operand reads and three quarters of the global loads per MFMA), but a CU holds one such workgroup at a
+  // time, so nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K /
+  // (1 + g), a round of 512 small ones 12 us + 0.1207 us * K, with g and f (beta == 0 / beta != 0) fitted per variant
+  // to 8192^3 and 16384^3 runs.  They pay from K of about 6000 on, for tile counts that fill whole rounds.  Not for
+  // TT (one LDS read per block for the K-major A of the large tile: 137 against 138 TFLOP/s), not with split K.
+  // fp64 stays at 128 x 128: with the 256 accumulator registers of a 256 x 128 tile the compiler spills in the loop.
+  constexpr int BIG = 256;
+  struct LargeTileFit { double g, f0, f1; };
+  const LargeTileFit fit = at ? LargeTileFit{0.065, 110.0, 222.0} : bt ? LargeTileFit{0.043, 38.0, 89.0} : LargeTileFit{0.020, 31.0, 85.0};
+  const long big_tiles = ((M + BIG - 1) / BIG) * ((N + BIG - 1) / BIG);
+  const long small_tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const double big_us = (double)((big_tiles + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * 0.1207 * (double)K / (1.0 + fit.g));
+  const double small_us = (double)((small_tiles + 511) / 512) * (12.0 + 0.1207 * (double)K);
+  const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");  // "0": never, "1": wherever it exists, unset: the model
+  const bool big = sizeof(T) == 4 && splits == 1 && !(at && bt) && (pin && *pin ? atoi(pin) != 0 : big_us < small_us);
+  const int TM_RT = big ? BIG : 128, TN_RT = big ? BIG : 128;
+  const int gm = (int)((M + TM_RT - 1) / TM_RT), gn = (int)((N + TN_RT - 1) / TN_RT);
+  if ((long)gm * gn > INT32_MAX) return 2;
+  const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
+  const int vecB = ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % Tr::VEC == 0) ? 1 : 0;
   dim3 grid(gm * gn, splits), block(NTHREADS);
   // split: plain partial products into the dense workspace slices, alpha and beta applied by the reduction
   const T k_alpha = splits > 1 ? T(1) : alpha, k_beta = splits > 1 ? T(0) : beta;
   T* const k_C = splits > 1 ? workspace : C;
   const long k_ldc = splits > 1 ? M : ldc;
-#define PLK_LAUNCH(AKF, BKF)                                                                                      \
-  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, A, lda, B, \
-                     ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, kchunk)
+  constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
+#define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK)                                                                            \
+  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
+                     A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, kchunk)
+#define PLK_LAUNCH(AKF, BKF)                                                  \
+  do {                                                                        \
+    if constexpr (sizeof(T) == 4) {                                           \
+      if (big) { PLK_LAUNCH_T(AKF, BKF, BIG, BIG, PLK_F32_BIG_BK); break; }   \
+    }                                                                         \
+    PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL);                               \
+  } while (0)
   // op(A) K-major <=> TransA == 'T'; op(B) K-major <=> TransB == 'N'
   if (an && bnn) PLK_LAUNCH(false, true);
   else if (an && bt) PLK_LAUNCH(false, false);
   else if (at && bnn) PLK_LAUNCH(true, true);
   else PLK_LAUNCH(true, false);
+#undef PLK_LAUNCH_T
 #undef PLK_LAUNCH
   if (splits > 1) {
     const long total = M * N;

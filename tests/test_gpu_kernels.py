@@ -2,7 +2,9 @@
 Bit-exact where the arithmetic is exact (integer-valued data, daxpy against the fused form), otherwise within the
 contract's tolerances: normwise relative error <= 1e-13 (fp64) / 1e-5 (fp32) for GEMM, |err| <= 1e-13 |x||y| for ddot,
 <= 1 ulp per element for daxpy."""
+import contextlib
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -12,6 +14,24 @@ from oracle_binding import ptr, rand_f32, rand_f64
 
 pytestmark = pytest.mark.gpu
 TOL64, TOL32 = 1e-13, 1e-5
+
+
+_LARGE_TILE_BITS = {}
+
+
+@contextlib.contextmanager
+def large_tile(pin):
+    """PARALIA_GEMM_LARGE_TILE for the calls inside: "1" forces the 256 x 256 fp32 tile, "0" forbids it, None leaves the
+    choice to the kernel's cost model.  The library reads the variable at every launch."""
+    old = os.environ.pop("PARALIA_GEMM_LARGE_TILE", None)
+    if pin is not None:
+        os.environ["PARALIA_GEMM_LARGE_TILE"] = pin
+    try:
+        yield
+    finally:
+        os.environ.pop("PARALIA_GEMM_LARGE_TILE", None)
+        if old is not None:
+            os.environ["PARALIA_GEMM_LARGE_TILE"] = old
 
 
 def run_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc, a_off=0, b_off=0, c_off=0):
@@ -129,6 +149,50 @@ def test_sgemm_tile_exact_and_unaligned(pkg, L, orc):
     ref = C0.copy()
     orc.orc_sgemm_bruteforce(b"N", b"T", M, N, K, 1.0, ptr(A[3:]), M + 1, ptr(B[1:]), N + 3, 1.0, ptr(ref[2:]), M + 1)
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims,off", [((4096, 4096, 64), 0), ((4000, 4100, 77), 0), ((8192 + 256, 2048, 33), 0), ((4096, 4096, 40), 1)])
+def test_sgemm_large_tile_exact_on_integers(pkg, L, openblas, ta, tb, dims, off):
+    """The 256 x 256 macro tile of fp32 (TT keeps the small one), forced for shapes the cost model would give to the
+    small tile: interior tiles, partial tiles on both edges, k not a multiple of the panel depth, and operands one
+    element off the 16-byte alignment (the element-load path).  Small-integer data, so OpenBLAS gives the exact bits."""
+    M, N, K = dims
+    rng = np.random.default_rng(11)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4 * (1 - off) + off, rb + off, M + 8 * (1 - off) + off
+    A = rng.integers(-4, 5, lda * ca + off).astype(np.float32)
+    B = rng.integers(-4, 5, ldb * cb + off).astype(np.float32)
+    C0 = rng.integers(-4, 5, ldc * N + off).astype(np.float32)
+    with large_tile("1"):
+        got = run_gemm(pkg, L, np.float32, ta, tb, M, N, K, 2.0, -1.0, A, lda, B, ldb, C0, ldc, off, off, off)
+    ref = C0.copy()
+    assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A[off:]), lda, ptr(B[off:]), ldb, -1.0, ptr(ref[off:]), ldc) == 0
+    assert np.array_equal(got, ref)  # includes the padding between columns, which both leave alone
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N")])
+@pytest.mark.parametrize("beta", [0.5, 0.0])
+@pytest.mark.parametrize("pin", ["1", "0", None])
+def test_sgemm_large_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, pin, beta):
+    """Random data at 4096 x 4096 x 8192, where the kernel's cost model picks the large tile by itself (pin None) for
+    beta = 0 and for NT also with beta != 0.  The summation order over k does not depend on the tile, so the three
+    runs give the same bits."""
+    M, N, K = 4096, 4096, 8192
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    A, B, C0 = rand_f32(ra * ca, 1), rand_f32(rb * cb, 2), rand_f32(M * N, 3)
+    with large_tile(pin):
+        got = run_gemm(pkg, L, np.float32, ta, tb, M, N, K, 1.5, beta, A, ra, B, rb, C0, M)
+    ref = C0.copy()
+    assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 1.5, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M) == 0
+    d = 1.5 * orc.orc_fro_norm_f32(ptr(A), ra, ca, ra) * orc.orc_fro_norm_f32(ptr(B), rb, cb, rb) + beta * orc.orc_fro_norm_f32(ptr(C0), M, N, M)
+    assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
+    key = (ta, tb, beta)
+    if key in _LARGE_TILE_BITS:
+        assert np.array_equal(got, _LARGE_TILE_BITS[key])
+    _LARGE_TILE_BITS[key] = got
 
 
 def scaled_ulp(a, b, alpha, x, y0):
