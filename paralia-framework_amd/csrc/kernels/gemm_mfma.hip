@@ -5,8 +5,8 @@
 // direct call form Database_builder/CuCuBLAS/src/dgemm_microbench.cu:141-142).  Here it is a hand-written
 // MFMA kernel:
 //   * one workgroup = 256 threads = 4 wavefronts (2 x 2), macro tile 128 x 128 (each wave owns 64 x 64, two
-//     workgroups per CU), and for fp32 also 256 x 256 (each wave owns 128 x 128 with 256 accumulator registers, one
-//     workgroup per CU) for problems with enough such tiles to fill the CUs;
+//     workgroups per CU); fp32 also has 256 x 128 (two workgroups per CU) and 256 x 256 (each wave owns 128 x 128
+//     with 256 accumulator registers, one workgroup per CU) for problems with enough such tiles to fill the CUs;
 //   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2 or 4 x 4);
 //   * A and B k-panels (16 elements deep, 32 for the large tile) are staged global -> registers -> LDS,
 //     double-buffered, one barrier per k-panel; the next panel's global loads are in flight while the current one is
@@ -189,7 +189,7 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 // the whole register file and fewer operand reads and global loads per MFMA.
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
 template <typename T, bool AK, bool BKM, int BM, int BN, int BK>
-__global__ __launch_bounds__(NTHREADS, (BM * BN <= 128 * 128 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
+__global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 8 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
                                                           long ldc, int gm, int gn, int vecA, int vecB, int kchunk) {
   using Tr = Traits<T>;
@@ -506,23 +506,31 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   int kchunk = 0;
   int splits = workspace ? pick_splits<T>(M, N, K, &kchunk) : 1;
   if (splits > 1 && (long)splits * M * N * (long)sizeof(T) > workspace_bytes) splits = 1, kchunk = 0;
-  // fp32: 256 x 256 macro tiles when the model below says they are faster.  Their inner loop runs 2 - 6 % faster per k
-  // (half the operand reads and three quarters of the global loads per MFMA), but a CU holds one such workgroup at a
-  // time, so nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K /
-  // (1 + g), a round of 512 small ones 12 us + 0.1207 us * K, with g and f (beta == 0 / beta != 0) fitted per variant
-  // to 8192^3 and 16384^3 runs.  They pay from K of about 6000 on, for tile counts that fill whole rounds.  Not for
-  // TT (one LDS read per block for the K-major A of the large tile: 137 against 138 TFLOP/s), not with split K.
-  // fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs) measured 70.7 against 73.4 TFLOP/s.
-  constexpr int BIG = 256;
+  // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
+  //  * 256 x 256 x 32 ("large", NT and TN): its inner loop runs 4 - 6 % faster per k (half the operand reads and three
+  //    quarters of the global loads per MFMA), but a CU holds one such workgroup at a time, so nothing overlaps its
+  //    prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K / (1 + g), a round of 512
+  //    small ones 12 us + 0.1207 us * K, with g and f (beta == 0 / beta != 0) fitted per variant to 8192^3 and 16384^3
+  //    runs.  It pays from K of about 6000 on, for tile counts that fill whole rounds.
+  //  * 256 x 128 x 16 ("wide", NN): still two workgroups per CU, 3 % faster per k (measured with several streams in
+  //    flight: +2.9 % at 4096^3, +4.7 % at 8192^3; for NN the large tile gains less, for NT the wide one loses 1 %).
+  // TT keeps the small tile (K-major A costs the bigger tiles one LDS read per block: 137 against 138 TFLOP/s), and
+  // so does split K.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs) measured 70.7
+  // against 73.4 TFLOP/s.
   struct LargeTileFit { double g, f0, f1; };
-  const LargeTileFit fit = at ? LargeTileFit{0.065, 110.0, 222.0} : bt ? LargeTileFit{0.043, 38.0, 89.0} : LargeTileFit{0.020, 31.0, 85.0};
-  const long big_tiles = ((M + BIG - 1) / BIG) * ((N + BIG - 1) / BIG);
-  const long small_tiles = ((M + 127) / 128) * ((N + 127) / 128);
-  const double big_us = (double)((big_tiles + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * 0.1207 * (double)K / (1.0 + fit.g));
-  const double small_us = (double)((small_tiles + 511) / 512) * (12.0 + 0.1207 * (double)K);
+  const LargeTileFit fit = at ? LargeTileFit{0.065, 110.0, 222.0} : LargeTileFit{0.043, 38.0, 89.0};
+  auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
+  const double k_us = 0.1207 * (double)K;
+  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (12.0 + k_us);
+  const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * k_us / (1.0 + fit.g));
+  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (24.0 + 2.0 * k_us / 1.03);
   const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");  // "0": never, "1": wherever it exists, unset: the model
-  const bool big = sizeof(T) == 4 && splits == 1 && !(at && bt) && (pin && *pin ? atoi(pin) != 0 : big_us < small_us);
-  const int TM_RT = big ? BIG : 128, TN_RT = big ? BIG : 128;
+  const bool pinned = pin && *pin, other = sizeof(T) == 4 && splits == 1 && !(at && bt) && (!pinned || atoi(pin) != 0);
+  // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
+  auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
+  const bool wide = other && an && bnn && (pinned || (wide_us < small_us && fills(tiles_of(256, 128), 512)));
+  const bool big = other && !(an && bnn) && (pinned || (large_us < small_us && fills(tiles_of(256, 256), 256)));
+  const int TM_RT = big || wide ? 256 : 128, TN_RT = big ? 256 : 128;
   const int gm = (int)((M + TM_RT - 1) / TM_RT), gn = (int)((N + TN_RT - 1) / TN_RT);
   if ((long)gm * gn > INT32_MAX) return 2;
   const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
@@ -539,7 +547,8 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
 #define PLK_LAUNCH(AKF, BKF)                                                  \
   do {                                                                        \
     if constexpr (sizeof(T) == 4) {                                           \
-      if (big) { PLK_LAUNCH_T(AKF, BKF, BIG, BIG, PLK_F32_BIG_BK); break; }   \
+      if (big) { PLK_LAUNCH_T(AKF, BKF, 256, 256, PLK_F32_BIG_BK); break; }   \
+      if (wide) { PLK_LAUNCH_T(AKF, BKF, 256, 128, PLK_F32_BK); break; }      \
     }                                                                         \
     PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL);                               \
   } while (0)
