@@ -191,7 +191,7 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 template <typename T, bool AK, bool BKM, int BM, int BN, int BK>
 __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 8 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
-                                                          long ldc, int gm, int gn, int vecA, int vecB, int kchunk) {
+                                                          long ldc, int gm, int gn, int vecA, int vecB, int vecC, int kchunk) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
   using acc_t = typename Tr::acc_t;
@@ -404,6 +404,52 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     }
   }
 
+  // Interior tile: no guards, so the compiler can batch the reads of C.  With the paired row rule (fp32, MN-major A) a
+  // lane's NBM accumulators of one column are adjacent in memory and go out as one 8- or 16-byte access when C is
+  // aligned for it.  Same arithmetic per element as the guarded loop below.
+  if (mrem == BM && nrem == BN) {
+    if constexpr (A_PAIR) {
+      typedef T cvec_t __attribute__((ext_vector_type(NBM)));
+      if (vecC) {
+#pragma unroll
+        for (int i = 0; i < NBN; ++i) {
+#pragma unroll
+          for (int r = 0; r < Tr::NACC; ++r) {
+            const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
+            cvec_t* const cp = reinterpret_cast<cvec_t*>(C + (long)(n0 + n) * ldc + m0 + wm + NBM * idx);
+            cvec_t v;
+#pragma unroll
+            for (int j = 0; j < NBM; ++j) v[j] = alpha * acc[i][j][r];
+            if (beta != T(0)) {
+              const cvec_t c = *cp;
+#pragma unroll
+              for (int j = 0; j < NBM; ++j) v[j] += beta * c[j];
+            }
+            *cp = v;
+          }
+        }
+        return;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NBN; ++i) {
+#pragma unroll
+      for (int r = 0; r < Tr::NACC; ++r) {
+        const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
+        T* const ccol = C + (long)(n0 + n) * ldc + m0;
+        T v[NBM];
+#pragma unroll
+        for (int j = 0; j < NBM; ++j) v[j] = alpha * acc[i][j][r];
+        if (beta != T(0)) {
+#pragma unroll
+          for (int j = 0; j < NBM; ++j) v[j] += beta * ccol[A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx];
+        }
+#pragma unroll
+        for (int j = 0; j < NBM; ++j) ccol[A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx] = v[j];
+      }
+    }
+    return;
+  }
   // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk)), or with the paired row rule
   // C(m0 + wm + NBM*idx + j, n0 + wn + NBN*drow(r, kk) + i)
 #pragma unroll
@@ -518,12 +564,12 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   // so does split K.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs) measured 70.7
   // against 73.4 TFLOP/s.
   struct LargeTileFit { double g, f0, f1; };
-  const LargeTileFit fit = at ? LargeTileFit{0.065, 110.0, 222.0} : LargeTileFit{0.043, 38.0, 89.0};
+  const LargeTileFit fit = at ? LargeTileFit{0.045, 77.0, 114.0} : LargeTileFit{0.042, 23.0, 34.0};
   auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
   const double k_us = 0.1207 * (double)K;
   const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (12.0 + k_us);
   const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * k_us / (1.0 + fit.g));
-  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (24.0 + 2.0 * k_us / 1.03);
+  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (12.0 + 2.0 * k_us / 1.026);
   const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");  // "0": never, "1": wherever it exists, unset: the model
   const bool pinned = pin && *pin, other = sizeof(T) == 4 && splits == 1 && !(at && bt) && (!pinned || atoi(pin) != 0);
   // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
@@ -535,6 +581,8 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   if ((long)gm * gn > INT32_MAX) return 2;
   const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
   const int vecB = ((reinterpret_cast<uintptr_t>(B) & 15) == 0 && ldb % Tr::VEC == 0) ? 1 : 0;
+  // C (or the split-K slices) aligned for 16-byte accesses
+  const int vecC = ((reinterpret_cast<uintptr_t>(splits > 1 ? workspace : C) & 15) == 0 && (splits > 1 ? M : ldc) % 4 == 0) ? 1 : 0;
   dim3 grid(gm * gn, splits), block(NTHREADS);
   // split: plain partial products into the dense workspace slices, alpha and beta applied by the reduction
   const T k_alpha = splits > 1 ? T(1) : alpha, k_beta = splits > 1 ? T(0) : beta;
@@ -543,7 +591,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
 #define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK)                                                                            \
   hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
-                     A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, kchunk)
+                     A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)
 #define PLK_LAUNCH(AKF, BKF)                                                  \
   do {                                                                        \
     if constexpr (sizeof(T) == 4) {                                           \
