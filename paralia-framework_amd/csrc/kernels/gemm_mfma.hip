@@ -557,7 +557,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   //    quarters of the global loads per MFMA), but a CU holds one such workgroup at a time, so nothing overlaps its
   //    prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K / (1 + g), a round of 512
   //    small ones 12 us + 0.1207 us * K, with g and f (beta == 0 / beta != 0) fitted per variant to 8192^3 and 16384^3
-  //    runs.  It pays from K of about 6000 on, for tile counts that fill whole rounds.
+  //    runs.  It pays from K of about 2000 (NT) / 6000 (TN) on, for tile counts that fill whole rounds.
   //  * 256 x 128 x 16 ("wide", NN): still two workgroups per CU, 3 % faster per k (measured with several streams in
   //    flight: +2.9 % at 4096^3, +4.7 % at 8192^3; for NN the large tile gains less, for NT the wide one loses 1 %).
   // TT keeps the small tile (K-major A costs the bigger tiles one LDS read per block: 137 against 138 TFLOP/s), and
