@@ -133,7 +133,7 @@ def main():
     ms = C.c_float()
     pkg.check(L.pl_event_elapsed_ms(e0, e1, C.byref(ms)), "elapsed")
     t_kernel = ms.value / reps / 1e3
-    roofline = {"bound": "mfma", "kernel": "plk::gemm_kernel<double,false,true> (fp64 NN tile GEMM), one launch of %d^3" % n,
+    roofline = {"bound": "mfma", "kernel": "plk::gemm_kernel<double,false,true,128,128,16> (fp64 NN tile GEMM), one launch of %d^3" % n,
                 "achieved": flops / t_kernel / 1e12, "peak": FP64_MFMA_PEAK / 1e12, "unit": "TFLOP/s",
                 "frac": flops / t_kernel / FP64_MFMA_PEAK, "avg_launch_ms": t_kernel * 1e3,
                 "flop_per_launch": flops, "traffic": GEMM_TRAFFIC_BYTES}
