@@ -123,6 +123,18 @@ long long pl_dgemv_workspace_doubles(char trans, long M, long N);
 int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
              double* y, long incy, double* workspace, void* stream);
 
+/* pl_dgemv for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): no workspace argument and no allocation of any kind inside the call.  It has no counterpart in the
+ * reference.  The partial sums go to a fixed array of PL_DGEMV_NOALLOC_MAX_DOUBLES doubles (4 MiB) that every GPU
+ * the library runs on holds until the process ends; kernels, chunking and summation order are those of pl_dgemv,
+ * so the results are bitwise the same.  A shape with pl_dgemv_workspace_doubles(trans, M, N) above that size is
+ * refused with PL_ERR_DIM (pl_last_error() says why).  All calls on one GPU share the array: calls that may
+ * overlap there (different streams, different threads) race; calls on one stream are safe. */
+#define PL_DGEMV_NOALLOC_MAX_DOUBLES 524288
+long long pl_dgemv_noalloc_max_doubles(void);
+int pl_dgemv_noalloc(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,
+                     double beta, double* y, long incy, void* stream);
+
 /* ---- routines: plain-C faces of Library_scheduler/include/PARALiA.hpp:33-72 ----
  * Operands may be host (pinned or pageable) or device pointers; the library detects which.  Calls return
  * after the result has reached the caller's buffer.  T > 0 / cache_limit > 0 preset the tile size and the

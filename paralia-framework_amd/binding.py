@@ -71,6 +71,8 @@ _SIGS = {
     "pl_ddot": (_i, [_l, _vp, _l, _vp, _l, _vp, _i, _vp, _vp]),
     "pl_dgemv_workspace_doubles": (_ll, [_c, _l, _l]),
     "pl_dgemv": (_i, [_c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _vp]),
+    "pl_dgemv_noalloc_max_doubles": (_ll, []),
+    "pl_dgemv_noalloc": (_i, [_c, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp]),
     "PARALiA_last_error": (C.c_char_p, []),
     "PARALiA_dgemm": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _l, _ll, C.POINTER(atc_info)]),
     "PARALiA_sgemm": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _l, _ll, C.POINTER(atc_info)]),

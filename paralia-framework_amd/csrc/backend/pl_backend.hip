@@ -11,6 +11,7 @@
 #include <string.h>
 
 #include "paralia_hip.h"
+#include "backend/pl_internal.h"
 
 namespace {
 thread_local char g_err[256] = "no error";
@@ -25,6 +26,12 @@ int fail(hipError_t e, const char* what) {
     if (e_ != hipSuccess) return fail(e_, #call); \
   } while (0)
 }  // namespace
+
+int pl_fail_hip(int hip_error, const char* what) { return fail((hipError_t)hip_error, what); }
+int pl_fail_msg(int code, const char* message) {
+  snprintf(g_err, sizeof(g_err), "%s", message);
+  return code;
+}
 
 extern "C" {
 

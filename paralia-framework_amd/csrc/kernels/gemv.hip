@@ -13,6 +13,9 @@
 // applies alpha and beta.  The summation order therefore depends only on (op, M, N), never on timing.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
+#include "backend/pl_internal.h"
 #include "paralia_hip.h"
 
 namespace plk {
@@ -164,24 +167,9 @@ __global__ __launch_bounds__(GEMV_WG) void gemv_final_kernel(long len, long chun
   *yp = beta == 0.0 ? alpha * s : fma(alpha, s, beta * *yp);
 }
 
-}  // namespace plk
-
-extern "C" {
-
-long long pl_dgemv_workspace_doubles(char trans, long M, long N) {
-  if (M <= 0 || N <= 0) return 0;
-  const bool t = !(trans == 'N' || trans == 'n');
-  // the chunk count depends on which load width the launch will pick (parity of M and lda, alignment of A):
-  // take the larger of the two
-  const plk::GemvShape wide = plk::gemv_shape(t, M + (M & 1), N, 2, nullptr);
-  const plk::GemvShape narrow = plk::gemv_shape(t, M, N, 1, nullptr);
-  const long chunks = wide.chunks > narrow.chunks ? wide.chunks : narrow.chunks;
-  return (long long)chunks * (wide.len_y + 1);
-}
-
-int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
-             double* y, long incy, double* workspace, void* stream) {
-  using namespace plk;
+// Launches the chunk kernel and the final kernel on `stream`; `workspace` receives the chunks' partial sums.
+static int launch_gemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
+                       double* y, long incy, double* workspace, void* stream) {
   const bool is_n = trans == 'N' || trans == 'n';
   const bool is_t = trans == 'T' || trans == 't' || trans == 'C' || trans == 'c';
   if (!is_n && !is_t) return PL_ERR_TRANS;
@@ -213,6 +201,70 @@ int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda
   }
   hipLaunchKernelGGL(gemv_final_kernel, dim3(fin_blocks), dim3(GEMV_WG), 0, st, len_y, s.chunks, (const double*)workspace, alpha, beta, ys, incy);
   return hipGetLastError() == hipSuccess ? 0 : PL_ERR_HIP;
+}
+
+// ---- scratch of the allocation-free entry point ----
+// The partial sums of pl_dgemv_noalloc go to this array instead of a caller-provided workspace.  Every GPU holds its
+// own copy, at its own address, from the moment the code object is loaded there until the process ends.  In host
+// code the name is only a handle for hipGetSymbolAddress; kernels get the address that call returned.
+static __device__ __align__(256) double scratch[PL_DGEMV_NOALLOC_MAX_DOUBLES];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static std::mutex scratch_mu;
+static double* scratch_ptr[NOALLOC_MAX_DEVICES];  // address of `scratch` on device d; null until the first call there
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+static int noalloc_scratch(double** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return pl_fail_hip((int)e, "pl_dgemv_noalloc: hipGetDevice");
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return pl_fail_msg(PL_ERR_ARG, "pl_dgemv_noalloc: device index beyond the per-device table");
+  std::lock_guard<std::mutex> lk(scratch_mu);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return pl_fail_hip((int)e, "pl_dgemv_noalloc: hipGetSymbolAddress(scratch)");
+    if (!p) return pl_fail_msg(PL_ERR_HIP, "pl_dgemv_noalloc: hipGetSymbolAddress(scratch) returned a null address");
+    scratch_ptr[dev] = (double*)p;
+  }
+  *out = scratch_ptr[dev];
+  return 0;
+}
+
+}  // namespace plk
+
+extern "C" {
+
+long long pl_dgemv_workspace_doubles(char trans, long M, long N) {
+  if (M <= 0 || N <= 0) return 0;
+  const bool t = !(trans == 'N' || trans == 'n');
+  // the chunk count depends on which load width the launch will pick (parity of M and lda, alignment of A):
+  // take the larger of the two
+  const plk::GemvShape wide = plk::gemv_shape(t, M + (M & 1), N, 2, nullptr);
+  const plk::GemvShape narrow = plk::gemv_shape(t, M, N, 1, nullptr);
+  const long chunks = wide.chunks > narrow.chunks ? wide.chunks : narrow.chunks;
+  return (long long)chunks * (wide.len_y + 1);
+}
+
+int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
+             double* y, long incy, double* workspace, void* stream) {
+  return plk::launch_gemv(trans, M, N, alpha, A, lda, x, incx, beta, y, incy, workspace, stream);
+}
+
+long long pl_dgemv_noalloc_max_doubles(void) { return PL_DGEMV_NOALLOC_MAX_DOUBLES; }
+
+// pl_dgemv without a workspace argument and without any allocation: same kernels, same chunking, same summation
+// order, partial sums in the per-device static array above.  Every chunk writes its whole slice before the final
+// kernel reads it, so nothing has to be cleared between calls.
+int pl_dgemv_noalloc(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
+                     double* y, long incy, void* stream) {
+  if (M > 0 && N > 0 && pl_dgemv_workspace_doubles(trans, M, N) > PL_DGEMV_NOALLOC_MAX_DOUBLES)
+    return pl_fail_msg(PL_ERR_DIM, "pl_dgemv_noalloc: this shape needs more partial sums than the fixed scratch holds "
+                                   "(pl_dgemv_workspace_doubles > pl_dgemv_noalloc_max_doubles); use pl_dgemv with a workspace");
+  double* ws = nullptr;
+  const int rc = plk::noalloc_scratch(&ws);
+  if (rc != 0) return rc;
+  return plk::launch_gemv(trans, M, N, alpha, A, lda, x, incx, beta, y, incy, ws, stream);
 }
 
 }  // extern "C"
