@@ -173,6 +173,19 @@ int PARALiA_dev_cache_free(int dev_id);
 /* metadata-cache and pool counters (PMD_cache, dgemm.cpp:342-368); reset drops the cached problems */
 int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries);
 int PARALiA_runtime_reset(void);
+/* releases everything the library holds: device block pool, streams, events, workspaces, pinned bounce buffers and
+ * the cached problems (CoCoPeLiaFreeResources, Subkernel.cpp:330, together with PARALiADevCacheFree); the next call
+ * creates what it needs again */
+int PARALiA_runtime_shutdown(void);
+/* per-command timeline of the streamed GEMM calls (what the reference's STEST / TTEST builds print per subkernel,
+ * Subkernel.cpp:498, dgemm.cpp:612-615).  While enabled, every command of a call's plan is bracketed by two timing
+ * events on its stream; PARALiA_trace_read copies the rows of the most recent such call, PL_TRACE_ROW doubles each:
+ * kind (0 fetch A, 1 fetch B, 2 fetch C, 3 tile GEMM, 4 lazy reduce, 5 write-back), mi, ni, ki, stream (0 H2D, 1 D2H,
+ * 2.. compute), start and end in milliseconds since the call's first command.  Returns the number of rows the call
+ * had (rows may be null to ask for the count).  Tracing costs a few percent; leave it off when timing. */
+#define PL_TRACE_ROW 7
+int PARALiA_trace_enable(int on);
+long PARALiA_trace_read(double* rows, long max_rows);
 /* which of the four stream-to-hardware-queue alignments the scheduler uses, and whether its start-up trial of
  * them (first four large streamed GEMM calls) is over; no counterpart in the reference */
 int PARALiA_stream_rotation(int* rotation, int* settled);

@@ -84,6 +84,9 @@ _SIGS = {
     "PARALiA_runtime_stats": (_i, [C.POINTER(_l), C.POINTER(_l), C.POINTER(_ll), C.POINTER(_l)]),
     "PARALiA_runtime_reset": (_i, []),
     "PARALiA_stream_rotation": (_i, [_pi, _pi]),
+    "PARALiA_runtime_shutdown": (_i, []),
+    "PARALiA_trace_enable": (_i, [_i]),
+    "PARALiA_trace_read": (_l, [C.POINTER(_d), _l]),
     "PARALiA_set_db_dir": (_i, [C.c_char_p]),
     "PARALiA_malloc": (_i, [C.POINTER(_vp), _ll, _i]),
     "PARALiA_free": (_i, [_vp, _i]),

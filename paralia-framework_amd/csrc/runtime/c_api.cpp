@@ -21,6 +21,9 @@ void cache_free_impl(short);
 void runtime_stats(long*, long*, long long*, long*);
 void runtime_reset();
 void stream_rotation(int*, int*);
+void runtime_shutdown();
+void trace_enable(int);
+long trace_read(double*, long);
 }  // namespace paralia
 paralia::StageTimes paralia_stage_times(const ATC* atc, long T);
 
@@ -125,6 +128,17 @@ int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_byte
 }
 int PARALiA_runtime_reset(void) {
   return guarded([&] { paralia::runtime_reset(); });
+}
+int PARALiA_runtime_shutdown(void) {
+  return guarded([&] { paralia::runtime_shutdown(); });
+}
+int PARALiA_trace_enable(int on) {
+  return guarded([&] { paralia::trace_enable(on); });
+}
+long PARALiA_trace_read(double* rows, long max_rows) {
+  long n = -1;
+  guarded([&] { n = paralia::trace_read(rows, max_rows); });
+  return n;
 }
 int PARALiA_stream_rotation(int* rotation, int* settled) {
   return guarded([&] { paralia::stream_rotation(rotation, settled); });

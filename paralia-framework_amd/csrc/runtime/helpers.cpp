@@ -48,14 +48,6 @@ double csecond() {
   return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
 }
 
-// The scheduler keeps four streams busy at once (H2D, D2H, two compute streams).  HIP multiplexes all streams of a
-// process, the default stream included, onto GPU_MAX_HW_QUEUES hardware queues (4 unless told otherwise); with
-// exactly four, which stream lands on which queue depends on how many streams the application created first, and
-// three of the four possible alignments cost 15-30% of the streamed GEMM's throughput (measured: 130 ms vs 148-169
-// ms for the 16384^3 fp64 case).  Eight queues remove the dependence.  The variable is read when the HIP runtime
-// initialises, so it is set when this library is loaded, and only if the user has not set it.
-__attribute__((constructor)) static void paralia_default_hw_queues() { setenv("GPU_MAX_HW_QUEUES", "8", 0); }
-
 static void hip_check(int rc, const char* what) {
   if (rc != 0) throw paralia_error(rc, std::string(what) + ": " + pl_last_error());
 }

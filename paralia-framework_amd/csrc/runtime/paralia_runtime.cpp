@@ -93,7 +93,7 @@ struct Resources {
         set_rotation(atoi(env));
         trials = 4;
       } else {
-        set_rotation(0);
+        set_rotation(trials >= 4 ? rotation : 0);  // a choice made before a teardown holds for the new ring
       }
     }
     for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
@@ -150,17 +150,54 @@ struct Resources {
     for (int q = 0; q < nexec; ++q) chk(pl_stream_sync(exec[q]), "stream sync");
     if (d2h) chk(pl_stream_sync(d2h), "stream sync");
   }
+  // Best effort, for error paths: whatever was enqueued before the failure must not outlive the call (it reads
+  // and writes the caller's operands and the pool blocks).
+  void drain() noexcept {
+    if (h2d) pl_stream_sync(h2d);
+    for (int q = 0; q < nexec; ++q) if (exec[q]) pl_stream_sync(exec[q]);
+    if (d2h) pl_stream_sync(d2h);
+  }
+  // Per-command timeline of a GEMM call (the reference's STEST / TTEST builds print one per subkernel,
+  // Subkernel.cpp:498, dgemm.cpp:612-615): when switched on, every command of the plan is bracketed by two timing
+  // events on its stream and the rows of the last call are kept for PARALiA_trace_read.
+  bool trace_on = false;
+  std::vector<void*> timing_events;
+  struct TraceRow { int kind, mi, ni, ki, stream; double t0_ms, t1_ms; };
+  std::vector<TraceRow> trace;
+  void ensure_timing_events(size_t n) {
+    while (timing_events.size() < n) {
+      void* e = nullptr;
+      chk(pl_event_create(&e, 1), "event create");
+      timing_events.push_back(e);
+    }
+  }
+  // The counterpart of CoCoPeLiaFreeResources (Subkernel.cpp:330): streams, events, workspaces and bounce buffers
+  // go; the next call creates them again.  The stream-alignment choice already made is kept.
   void destroy() {
+    drain();
     for (void* s : ring) if (s) pl_stream_destroy(s);
-    for (int q = 2; q < nexec; ++q) pl_stream_destroy(exec[q]);
+    for (int q = 2; q < nexec; ++q) if (exec[q]) pl_stream_destroy(exec[q]);
     for (void* e : events) pl_event_destroy(e);
+    for (void* e : timing_events) pl_event_destroy(e);
     if (dot_ws) pl_free_device(dot_ws);
     if (dot_host) pl_free_pinned(dot_host);
     gemv_x.release(); gemv_y.release(); gemv_ws.release();
     for (Scratch& w : gemm_ws) w.release();
     stager_.reset();
+    const int keep_rotation = rotation, keep_trials = trials;
+    const bool keep_trace = trace_on;
     *this = Resources();
+    rotation = keep_rotation;
+    trials = keep_trials;
+    trace_on = keep_trace;
   }
+};
+// Armed while a routine enqueues work; if the routine leaves by an exception the streams are drained first.
+struct DrainOnError {
+  Resources& res;
+  bool armed = true;
+  explicit DrainOnError(Resources& r) : res(r) {}
+  ~DrainOnError() { if (armed) res.drain(); }
 };
 
 // ------------------------------------------------------------------------------------ metadata cache
@@ -266,11 +303,18 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   void* ws[MAX_EXEC_QUEUES] = {nullptr};
   if (ws_bytes > 0)
     for (int q = 0; q < std::max(1, std::min(p.exec_queues, MAX_EXEC_QUEUES)); ++q) ws[q] = R.res.gemm_ws[q].ensure(ws_bytes);
+  const bool trace = R.res.trace_on;
+  if (trace) {
+    R.res.ensure_timing_events(2 * plan.cmds.size() + 1);
+    chk(pl_event_record(R.res.timing_events[0], R.res.h2d), "event record");  // time zero of the timeline
+  }
 
+  DrainOnError guard(R.res);
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
     void* s = R.res.stream(c.stream);
     for (int w = 0; w < c.nwait; ++w) chk(pl_stream_wait_event(s, ev[c.wait[w]]), "stream wait event");
+    if (trace) chk(pl_event_record(R.res.timing_events[1 + 2 * i], s), "event record");
     switch (c.kind) {
       case CMD_FETCH_A: {
         const long rows = at ? p.tk(c.ki) : p.tm(c.mi), cols = at ? p.tm(c.mi) : p.tk(c.ki);
@@ -321,13 +365,26 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         else chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
       } break;
     }
+    if (trace) chk(pl_event_record(R.res.timing_events[2 + 2 * i], s), "event record");
     if (c.signals) {
       ev[i] = R.res.events[next_ev++];
       chk(pl_event_record(ev[i], s), "event record");
     }
   }
   R.res.sync_all();
+  guard.armed = false;
   staged.finish();
+  if (trace) {
+    R.res.trace.clear();
+    R.res.trace.reserve(plan.cmds.size());
+    for (size_t i = 0; i < plan.cmds.size(); ++i) {
+      const Cmd& c = plan.cmds[i];
+      float t0 = 0, t1 = 0;
+      chk(pl_event_elapsed_ms(R.res.timing_events[0], R.res.timing_events[1 + 2 * i], &t0), "event elapsed");
+      chk(pl_event_elapsed_ms(R.res.timing_events[0], R.res.timing_events[2 + 2 * i], &t1), "event elapsed");
+      R.res.trace.push_back({c.kind, c.mi, c.ni, c.ki, c.stream, (double)t0, (double)t1});
+    }
+  }
 }
 
 template <typename T>
@@ -503,6 +560,7 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
   StagerScope staged(stager);
   std::vector<void*> ev_in(ring), ev_ex(ring), ev_out(ring);
   for (int r = 0; r < ring; ++r) { ev_in[r] = R.res.events[3 * r]; ev_ex[r] = R.res.events[3 * r + 1]; ev_out[r] = R.res.events[3 * r + 2]; }
+  DrainOnError guard(R.res);
   for (long t = 0; t < tiles; ++t) {
     const long len = std::min(T, N - t * T);
     const int r = (int)(t % ring);
@@ -534,6 +592,7 @@ static void blas1_stream(Runtime& R, long N, long T, double* x, long incx, int l
     }
   }
   R.res.sync_all();
+  guard.armed = false;
   staged.finish();
 }
 
@@ -705,6 +764,7 @@ ATC_p dgemv_impl(char TransA, long M, long N, double alpha, double* A, long ldA,
   double* yd = y;
   void* ev_vec = R.res.events[0];
   bool staged = false;
+  DrainOnError guard(R.res);
   if (locx < 0 && alpha != 0.0) {
     xd = (double*)R.res.gemv_x.ensure(span_x);
     chk(pl_copy_async(xd, x, span_x, s_in), "fetch x");
@@ -768,6 +828,7 @@ ATC_p dgemv_impl(char TransA, long M, long N, double alpha, double* A, long ldA,
     chk(pl_copy_async(y, yd, span_y, s_out), "write back y");
   }
   R.res.sync_all();
+  guard.armed = false;
   return atc_copy(atc);
 }
 
@@ -800,6 +861,36 @@ void runtime_reset() {
   std::lock_guard<std::mutex> lk(R.mu);
   R.pmd.clear();
   R.pmd_hits = R.pmd_misses = 0;
+}
+
+// Everything the library holds on the device goes: block pool, streams, events, workspaces, pinned bounce buffers,
+// cached problems (CoCoPeLiaFreeResources + PARALiADevCacheFree, Subkernel.cpp:330,488).  The next call starts cold.
+void runtime_shutdown() {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  R.res.drain();
+  R.pool.release();
+  R.res.destroy();
+  R.pmd.clear();
+}
+
+void trace_enable(int on) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  R.res.trace_on = on != 0;
+  if (!on) R.res.trace.clear();
+}
+
+long trace_read(double* rows, long max_rows) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  const long n = (long)R.res.trace.size();
+  for (long i = 0; rows && i < n && i < max_rows; ++i) {
+    const Resources::TraceRow& t = R.res.trace[i];
+    double* r = rows + i * 7;
+    r[0] = t.kind; r[1] = t.mi; r[2] = t.ni; r[3] = t.ki; r[4] = t.stream; r[5] = t.t0_ms; r[6] = t.t1_ms;
+  }
+  return n;
 }
 }  // namespace paralia
 
