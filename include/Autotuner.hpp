@@ -38,7 +38,10 @@ enum ModelType {
   COCOPELIA_DATALOC = 4,
   COCOPELIA_BIDIRECTIONAL = 5,
   COCOPELIA_REUSE = 6,
-  COCOPELIA_PIPELINE_EMULATE = 7,
+  // 7 is the reference's COCOPELIA_PIPELINE_EMULATE (ModelLvl3.cpp:554-650), left out on purpose: it multiplies its
+  // transfer times by the operands' location codes, which were 0 / 1 when it was written and are -1 for the host
+  // now, so its copy terms come out negative; the plan simulator of this runtime (runtime/gemm_plan.hpp) does that
+  // job, with both copy directions.
   FULL_OVERLAP = 9,
   NO_OVERLAP = 10
 };

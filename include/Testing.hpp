@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <vector>
 
 #include "PARALiA.hpp"
 #include "backend_wrappers.hpp"
@@ -26,6 +27,22 @@ inline std::string test_log_dir() {
   const char* d = getenv("PARALIA_TESTLIBDIR");
   return d && *d ? d : ".";
 }
+
+/// Names the reference's drivers build their log file names from (dgemm_runner.cpp:33-37:
+/// "%s/CoCoPeLiaDgemmRunner_%s_%s.log" with TESTLIBDIR, CoCoImplementationPrint() and VERSION).  There TESTLIBDIR and
+/// VERSION are compile definitions of its build; here they default to $PARALIA_TESTLIBDIR (or ".") and the driver
+/// version, and a build may still define them.
+inline const char* CoCoImplementationPrint() { return "MI355X"; }
+inline const char* paralia_testlibdir_cstr() {
+  static const std::string dir = test_log_dir();
+  return dir.c_str();
+}
+#ifndef TESTLIBDIR
+#define TESTLIBDIR (paralia_testlibdir_cstr())
+#endif
+#ifndef VERSION
+#define VERSION DRIVER_VERSION
+#endif
 
 inline ATC_p parse_control(const char* fn, const char* argv[]) {
   const int active_unit_num = atoi(argv[1]);
@@ -162,6 +179,47 @@ inline void StoreLogLvl3(const char* filename, ATC_p ctl, char TransA, char Tran
   fclose(fp);
 }
 
+/// The CHECKLOG step of the reference's drivers (testing.cpp:331-397): when the log already holds a row for exactly
+/// this configuration the benchmark is not repeated -- the program says so and exits with status 1.  A missing log
+/// file is created.  `ctl` is the preset controller before the run and the returned one after it.
+inline void paralia_check_log(const char* who, const char* filename, const char* search_string) {
+  FILE* fp = fopen(filename, "r");
+  if (!fp) {
+    fp = fopen(filename, "w+");
+    if (!fp) error("%s: LogFile %s failed to open\n", who, filename);
+    warning("%s: Generating Logfile %s...\n", who, filename);
+  }
+  char buffer[1024];
+  while (fgets(buffer, sizeof(buffer), fp) != NULL)
+    if (strstr(buffer, search_string) != NULL) {
+      fprintf(stderr, "%s: entry %s found. Quiting...\n", who, search_string);
+      fclose(fp);
+      exit(1);
+    }
+  fclose(fp);
+}
+inline void CheckLogLvl1(const char* filename, ATC_p ctl, double alpha, long int D1, long int inc1, long int inc2, short loc1,
+                         short loc2, short outloc1, short outloc2) {
+  char key[1024];
+  snprintf(key, sizeof key, "%s, %.5lf,%zu,%zu,%zu,%d,%d,%d,%d", ctl ? ctl->print_csv() : "-1,-1,-1,-1", alpha, (size_t)D1, (size_t)inc1,
+           (size_t)inc2, loc1, loc2, outloc1, outloc2);
+  paralia_check_log("CheckLogLvl1", filename, key);
+}
+inline void CheckLogLvl2(const char* filename, ATC_p ctl, char TransA, double alpha, double beta, long int D1, long int D2,
+                         long int inc1, long int inc2, short loc1, short loc2, short loc3, short outloc) {
+  char key[1024];
+  snprintf(key, sizeof key, "%s, %c,%.5lf,%.5lf,%zu,%zu,%zu,%zu,%d,%d,%d,%d", ctl ? ctl->print_csv() : "-1,-1,-1,-1", TransA, alpha, beta,
+           (size_t)D1, (size_t)D2, (size_t)inc1, (size_t)inc2, loc1, loc2, loc3, outloc);
+  paralia_check_log("CheckLogLvl2", filename, key);
+}
+inline void CheckLogLvl3(const char* filename, ATC_p ctl, char TransA, char TransB, double alpha, double beta, long int D1,
+                         long int D2, long int D3, short loc1, short loc2, short loc3, short outloc) {
+  char key[1024];
+  snprintf(key, sizeof key, "%s, %c,%c,%.5lf,%.5lf,%zu,%zu,%zu,%d,%d,%d,%d", ctl ? ctl->print_csv() : "-1,-1,-1,-1", TransA, TransB, alpha,
+           beta, (size_t)D1, (size_t)D2, (size_t)D3, loc1, loc2, loc3, outloc);
+  paralia_check_log("CheckLogLvl3", filename, key);
+}
+
 // ------------------------------------------------------------------------------------------------------------------
 // OpenBLAS, found at run time: $PARALIA_OPENBLAS_LIB, a system libopenblas, or the copy bundled with NumPy / SciPy
 // (symbols scipy_cblas_*64_ with 64-bit integers, or scipy_cblas_* / cblas_* with 32-bit ones).
@@ -199,6 +257,7 @@ struct OpenBlas {
   bool open() {
     if (h) return true;
     const char* env = getenv("PARALIA_OPENBLAS_LIB");
+    if (env && !strcmp(env, "none")) return false;  // run as on a machine without OpenBLAS (the host-computed references)
     if (env && *env && try_open(env)) return true;
     for (const char* p : {"libopenblas.so.0", "libopenblas.so", "libopenblas64_.so.0"})
       if (try_open(p)) return true;
@@ -244,6 +303,45 @@ struct OpenBlas {
     return ((double (*)(int, const double*, int, const double*, int))ddot)((int)n, x, (int)incx, y, (int)incy);
   }
 };
+
+/// Validation without OpenBLAS: `samples` entries of C, spread over the matrix by a fixed stride walk, are recomputed
+/// with a long double dot product from the same host copies of A, B and the original C, and the worst number of
+/// matching decimal digits is returned (differences are taken relative to max(|ref|, |x|, rms of the sampled refs), as
+/// Dtest_equality does).  A wrong tile index, a dropped k-step or a wrong beta schedule hits every sample of its tile.
+template <typename T>
+inline short sampled_gemm_digits(char ta, char tb, long M, long N, long K, T alpha, const T* A, long ldA, const T* B, long ldB, T beta,
+                                 const T* C0, const T* C, long ldC, int samples = 512) {
+  const bool at = ta == 'T' || ta == 't', bt = tb == 'T' || tb == 't';
+  const int cap = sizeof(T) == 8 ? 16 : 7;
+  std::vector<long double> ref(samples);
+  std::vector<double> got(samples);
+  uint64_t state = 0x9E3779B97F4A7C15ULL;
+  long double ss = 0;
+  for (int s = 0; s < samples; ++s) {
+    state = state * 6364136223846793005ULL + 1442695040888963407ULL;
+    const long i = (long)((state >> 33) % (uint64_t)M);
+    state = state * 6364136223846793005ULL + 1442695040888963407ULL;
+    const long j = (long)((state >> 33) % (uint64_t)N);
+    long double acc = 0;
+    for (long k = 0; k < K; ++k)
+      acc += (long double)(at ? A[k + i * ldA] : A[i + k * ldA]) * (long double)(bt ? B[j + k * ldB] : B[k + j * ldB]);
+    ref[s] = (long double)alpha * acc + (beta == T(0) ? 0.0L : (long double)beta * (long double)C0[i + j * ldC]);
+    got[s] = (double)C[i + j * ldC];
+    ss += ref[s] * ref[s];
+  }
+  const double rms = samples > 0 ? (double)sqrtl(ss / samples) : 0.0;
+  int worst = cap;
+  for (int s = 0; s < samples; ++s) {
+    const double d = fabs((double)ref[s] - got[s]);
+    if (d == 0) continue;
+    if (std::isnan(d)) return 0;
+    const double scale = fmax(fmax(fabs((double)ref[s]), fabs(got[s])), rms);
+    int digits = (int)floor(-log10(d / scale));
+    if (digits < 0) digits = 0;
+    if (digits < worst) worst = digits;
+  }
+  return (short)worst;
+}
 
 /// Host copy of a buffer at any location (caller frees with free()).
 template <typename T> inline T* host_copy(T* src, long long n, short loc) {

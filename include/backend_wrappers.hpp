@@ -52,9 +52,22 @@ inline long long gemv_flops(long M, long N) { return (long long)M * (2 * N + 1);
 inline long long axpy_flops(long N) { return 2LL * N; }
 inline long long dot_flops(long N) { return 2LL * N; }
 
-/// Leading dimension of a stored operand: rows of the matrix as stored (dgemm_runner.cpp:44-46).
+/// Leading dimension of a stored operand: rows of the matrix as stored.
 inline void TransposeTranslate(char TransChar, long* ldim, long dim1, long dim2) {
   *ldim = (TransChar == 'N' || TransChar == 'n') ? dim1 : dim2;
+}
+/// The call shape of the reference's drivers (dgemm_runner.cpp:44-46, dgemv_runner.cpp:47):
+///   TransposeTranslate(TransA, &cpu_op_A, &gpu_op_A, &ldA, M, K);
+/// The two operation out-parameters have the types of the host BLAS and of the device BLAS the driver was written
+/// for; here they are whatever enum or integer types the driver declares.  They receive the CBLAS codes
+/// (111 no-transpose, 112 transpose) and 0 / 1 respectively; nothing in this library reads them back.
+template <typename HostOp, typename DeviceOp>
+inline void TransposeTranslate(char TransChar, HostOp* host_op, DeviceOp* device_op, long* ldim, long dim1, long dim2) {
+  const bool n = (TransChar == 'N' || TransChar == 'n');
+  if (!n && TransChar != 'T' && TransChar != 't') error("TransposeTranslate: %c is an invalid Trans parameter\n", TransChar);
+  if (host_op) *host_op = static_cast<HostOp>(n ? 111 : 112);
+  if (device_op) *device_op = static_cast<DeviceOp>(n ? 0 : 1);
+  *ldim = n ? dim1 : dim2;
 }
 
 #endif

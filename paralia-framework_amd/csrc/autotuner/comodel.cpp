@@ -39,7 +39,6 @@ const char* printModel(ModelType mode) {
     case COCOPELIA_DATALOC: return "COCOPELIA_DATALOC";
     case COCOPELIA_BIDIRECTIONAL: return "COCOPELIA_BIDIRECTIONAL";
     case COCOPELIA_REUSE: return "COCOPELIA_REUSE";
-    case COCOPELIA_PIPELINE_EMULATE: return "COCOPELIA_PIPELINE_EMULATE";
     case FULL_OVERLAP: return "FULL_OVERLAP";
     case NO_OVERLAP: return "NO_OVERLAP";
   }

@@ -51,7 +51,20 @@ int main(const int argc, const char* argv[]) {
         if (Dtest_equality(ref, result, 1) < 9 && fabs(ref[0] - result[0]) > bound) error("Insufficient accuracy for benchmarks\n");
         free(hx); free(hy);
       } else {
-        warning("OpenBLAS absent: validation skipped\n");
+        // no OpenBLAS on this machine: a long double sum computed here
+        double* hx = host_copy(x, N * ax, x_loc);
+        double* hy = host_copy(y, N * ay, y_loc);
+        const double* xs = incx < 0 ? hx + (1 - N) * incx : hx;
+        const double* ys = incy < 0 ? hy + (1 - N) * incy : hy;
+        long double acc = 0, nx = 0, ny = 0;
+        for (long i = 0; i < N; ++i) {
+          acc += (long double)xs[i * incx] * ys[i * incy];
+          nx += (long double)xs[i * incx] * xs[i * incx];
+          ny += (long double)ys[i * incy] * ys[i * incy];
+        }
+        fprintf(stderr, "OpenBLAS absent: long double sum on the host -> %.15e, PARALiA -> %.15e\n", (double)acc, result[0]);
+        if (fabs((double)acc - result[0]) > 1e-13 * (double)sqrtl(nx * ny)) error("Insufficient accuracy for benchmarks\n");
+        free(hx); free(hy);
       }
     }
     for (int it = 0; it < 10; it++) return_values = call();

@@ -67,6 +67,10 @@ template <typename T> int run_gemm_runner(const int argc, const char* argv[]) {
     } else {
       snprintf(filename, sizeof filename, "%s/CoCoPeLia%sRunner_MI355X_%s.log", test_log_dir().c_str(), F::name, DRIVER_VERSION);
     }
+    // the reference builds its drivers with or without CHECKLOG (dgemm_runner.cpp:38-40,106-108); here it is a switch
+    const char* checklog_env = getenv("PARALIA_CHECKLOG");
+    const bool checklog = checklog_env && atoi(checklog_env);
+    if (checklog) CheckLogLvl3(filename, predef_control_values, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc);
 
     long int ldA, ldB, ldC = M;
     TransposeTranslate(TransA, &ldA, M, K);
@@ -122,7 +126,13 @@ template <typename T> int run_gemm_runner(const int argc, const char* argv[]) {
         if (digits < F::min_digits) error("Insufficient accuracy for benchmarks\n");
         free(hA); free(hB); free(C_ref);
       } else {
-        warning("OpenBLAS absent: result compared only with itself across calls\n");
+        // no OpenBLAS on this machine: sampled entries against a long double dot product instead
+        T* hA = host_copy(A, M * K, A_loc);
+        T* hB = host_copy(B, N * K, B_loc);
+        const short digits = sampled_gemm_digits<T>(TransA, TransB, M, N, K, (T)alpha, hA, ldA, hB, ldB, (T)beta, C_start, C_out, ldC);
+        fprintf(stderr, "OpenBLAS absent: 512 sampled entries against a long double dot product\nMatching digits vs long double samples: %d\n", digits);
+        if (digits < F::min_digits) error("Insufficient accuracy for benchmarks\n");
+        free(hA); free(hB);
       }
       CoCoMemcpy(C, C_start, M * N * sizeof(T), C_loc, -2);
       free(C_start); free(C_out); free(C_out1);
@@ -133,6 +143,7 @@ template <typename T> int run_gemm_runner(const int argc, const char* argv[]) {
     CoCoSyncCheckErr();
     cpu_timer = csecond() - cpu_timer;
     const double first_over_t = cpu_timer;
+    if (checklog) CheckLogLvl3(filename, return_values, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc);
 
     short warmup_bench_it = 10;
     if (M >= 20000 && N >= 20000 && K >= 20000) warmup_bench_it = 2;

@@ -42,8 +42,9 @@ template <typename T> int run_gemm_tester(const int argc, const char* argv[]) {
   int failures = 0, cases = 0;
   try {
     OpenBlas ob;
-    if (!ob.open()) { fprintf(stderr, "%s: OpenBLAS not found, nothing to compare with\n", F::name); return 2; }
-    fprintf(stderr, "%s: OpenBLAS = %s\n", F::name, ob.path.c_str());
+    const bool have_blas = ob.open();
+    if (have_blas) fprintf(stderr, "%s: OpenBLAS = %s\n", F::name, ob.path.c_str());
+    else fprintf(stderr, "%s: OpenBLAS not found: every case is checked on 512 sampled entries against a long double dot product\n", F::name);
     const long ld = 8192;
     const T alpha = (T)1.23, beta = (T)0.9876;
     T* hA = (T*)CoCoMalloc(ld * ld * ES, -1, 1);
@@ -70,17 +71,21 @@ template <typename T> int run_gemm_tester(const int argc, const char* argv[]) {
       t = csecond() - t;
       CoCoMemcpy(C_got, lc >= 0 ? dC : hC, ld * cols * ES, -2, lc >= 0 ? 0 : -1);
       double t_ref = csecond();
-      F::blas(ob, ta, tb, M, N, K, alpha, hA, ld, hB, ld, beta, C_ref, ld);
-      t_ref = csecond() - t_ref;
       short worst = F::cap;
-      for (long j = 0; j < N; ++j) worst = std::min(worst, F::digits(C_ref + j * ld, C_got + j * ld, M));
       bool pad_ok = true;  // rows M..ld of every column belong to the caller
       for (long j = 0; j < N && pad_ok; ++j)
         for (long i = M; i < ld && i < M + 4; ++i) pad_ok &= (C_got[i + j * ld] == C_ref[i + j * ld]);
+      if (have_blas) {
+        F::blas(ob, ta, tb, M, N, K, alpha, hA, ld, hB, ld, beta, C_ref, ld);
+        for (long j = 0; j < N; ++j) worst = std::min(worst, F::digits(C_ref + j * ld, C_got + j * ld, M));
+      } else {
+        worst = sampled_gemm_digits<T>(ta, tb, M, N, K, alpha, hA, ld, hB, ld, beta, C_ref, C_got, ld);
+      }
+      t_ref = csecond() - t_ref;
       ++cases;
       const bool ok = worst >= F::min_digits && pad_ok;
       if (!ok) ++failures;
-      fprintf(stderr, "%-22s %c%c M=%-5ld N=%-5ld K=%-5ld locs(%d,%d,%d): PARALiA %.1lf Gflops/s, OpenBLAS %.1lf, T=%ld, digits=%d %s\n", label, ta, tb,
+      fprintf(stderr, "%-22s %c%c M=%-5ld N=%-5ld K=%-5ld locs(%d,%d,%d): PARALiA %.1lf Gflops/s, reference %.1lf, T=%ld, digits=%d %s\n", label, ta, tb,
               M, N, K, la, lb, lc, Gval_per_s(gemm_flops(M, N, K), t), Gval_per_s(gemm_flops(M, N, K), t_ref), r->T, worst, ok ? "ok" : "FAIL");
       delete r;
     };

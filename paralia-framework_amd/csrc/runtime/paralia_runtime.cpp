@@ -27,25 +27,33 @@ static void chk(int rc, const char* what) {
 }
 
 // ------------------------------------------------------------------------------------------ block pool
-// Equal-size device blocks, kept between calls (the reference's Buffer with BUFFER_REUSE_ENABLE,
-// dgemm.cpp:95-117): reallocated only when the block size changes or more blocks are needed.
+// Equal-size device blocks carved from one allocation that is kept between calls (the reference's Buffer with
+// BUFFER_REUSE_ENABLE, dgemm.cpp:95-117).  The allocation is only replaced when a call needs more bytes than it
+// holds: a call with another block size re-partitions the memory it already has.  Freeing and re-allocating tens of
+// gigabytes between calls is not free on this device: for a few seconds after such a hipFree the host link runs
+// about 4 % slower (the link-bound 40000 x 40000 x 2048 product: 284 ms instead of 273 ms for its first ten calls).
 struct DevicePool {
   void* base = nullptr;
+  long long capacity = 0;  // bytes held
   long long block_sz = 0;
   long blocks = 0;
-  long long bytes() const { return block_sz * blocks; }
+  long long bytes() const { return capacity; }
   void* at(long b) const { return (char*)base + block_sz * b; }
-  void ensure(long need_blocks, long long need_block_sz) {
-    if (base && block_sz == need_block_sz && blocks >= need_blocks) return;
-    release();
-    chk(pl_malloc_device(&base, need_block_sz * need_blocks), "device block pool allocation");
+  // limit > 0: the caller's cache_limit; memory kept from an earlier, larger call is given back rather than held
+  void ensure(long need_blocks, long long need_block_sz, long long limit = 0) {
+    const long long need = need_block_sz * need_blocks;
+    if (!base || capacity < need || (limit > 0 && capacity > std::max(limit, need))) {
+      release();
+      chk(pl_malloc_device(&base, need), "device block pool allocation");
+      capacity = need;
+    }
     block_sz = need_block_sz;
-    blocks = need_blocks;
+    blocks = need_block_sz > 0 ? (long)(capacity / need_block_sz) : 0;
   }
   void release() {
     if (base) chk(pl_free_device(base), "device block pool free");
     base = nullptr;
-    block_sz = 0;
+    capacity = block_sz = 0;
     blocks = 0;
   }
 };
@@ -495,7 +503,7 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;
-    R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T));
+    R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T), atc->cache_limit);
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
     // a first call of a problem also pays for fresh pool memory and cold caches: it would misjudge its rotation
     const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab && !cold;
@@ -790,7 +798,7 @@ ATC_p dgemv_impl(char TransA, long M, long N, double alpha, double* A, long ldA,
     const long long blk = ((long long)std::min(T, M) * std::min(T, N) * 8 + 255) / 256 * 256;  // slots keep A's alignment
     long long budget = pool_budget(atc->cache_limit, R.pool.bytes());
     const int ring = (int)std::max<long long>(1, std::min<long long>(std::min<long>(tiles, 4), budget / blk));
-    R.pool.ensure(ring, blk);
+    R.pool.ensure(ring, blk, atc->cache_limit);
     // every tile has at most max(T, ...) outputs per chunk: size the workspace for the largest tile shape
     long long ws_doubles = 8;
     for (long mi : {0L, Mg - 1})

@@ -56,3 +56,23 @@ def sync(pkg):
 
 def gemm_denominator(alpha, opA_norm, opB_norm, beta, c0_norm):
     return abs(alpha) * opA_norm * opB_norm + abs(beta) * c0_norm
+
+
+def check_daxpy_against_blas(orc, got, blas_result, alpha, x, y0):
+    """The daxpy contract: every element within 1 ulp of the host BLAS.  A BLAS whose kernel uses a fused multiply-add
+    (the builds on these machines do) is held to that plainly.  Only a BLAS that is shown, bit for bit, to round
+    alpha*x before adding may differ more where the sum cancels; then the bound is 1.5 units in the last place of the
+    larger operand (half a unit for the rounded product, half for each final rounding).  Prints which case applied."""
+    import oracle_binding as ob
+    worst = int(orc.orc_max_ulp_f64(ob.ptr(got), ob.ptr(blas_result), got.size))
+    if worst <= 1:
+        print("  daxpy vs host BLAS: worst distance %d ulp (plain 1-ulp contract)" % worst, flush=True)
+        return worst
+    unfused = y0.copy()
+    orc.orc_daxpy_mul_add(got.size, alpha, ob.ptr(x), 1, ob.ptr(unfused), 1)
+    assert np.array_equal(blas_result, unfused), "host BLAS result is neither within 1 ulp nor the unfused evaluation: %d ulp" % worst
+    scale = np.maximum(np.maximum(np.abs(alpha * x), np.abs(y0)), np.maximum(np.abs(got), np.abs(blas_result)))
+    scaled = float(np.max(np.abs(got - blas_result) / np.spacing(scale)))
+    print("  daxpy vs host BLAS without fused multiply-add: worst %d ulp of the result, %.2f units of the larger operand" % (worst, scaled), flush=True)
+    assert scaled <= 1.5
+    return worst

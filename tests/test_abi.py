@@ -131,3 +131,35 @@ def test_runner_row_is_readable_by_the_reference_plotters(pkg, tmp_path):
     assert list(df["T"]) == [2048, 1024] and list(df["TransA"]) == ["N", "T"] and list(df["TransB"]) == ["T", "N"]
     assert list(df["M"]) == [8192, 4096] and list(df["N"]) == [4096, 4096] and list(df["K"]) == [2048, 4096]
     assert list(df["Bloc"]) == [0, -1] and (df["t1"] > 0).all()
+
+
+def test_driver_written_against_the_reference_call_shapes_compiles_and_links(pkg, tmp_path):
+    """tests/golden/reference_call_shapes.cpp uses the helper surface the way the reference's drivers do (six-argument
+    TransposeTranslate with the caller's own operation enums, CoCoMalloc / CoCoVecInit / CoCoMemcpy, PARALiADgemm and its
+    Controled twin, CheckLogLvl3 / StoreLogLvl3 with TESTLIBDIR, CoCoImplementationPrint() and VERSION).  It must compile
+    against include/ alone and link libparalia.so; its host mode (no GPU call) must run and leave one 18-column row."""
+    import subprocess
+    src = os.path.join(ROOT, "tests", "golden", "reference_call_shapes.cpp")
+    exe = str(tmp_path / "reference_call_shapes")
+    libdir = os.path.dirname(pkg.LIB_PATH)
+    cmd = ["g++", "-O1", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "include"), src, "-o", exe, "-L", libdir, "-lparalia",
+           "-Wl,-rpath," + libdir, "-ldl", "-lpthread"]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-3000:]
+    env = dict(os.environ, PARALIA_TESTLIBDIR=str(tmp_path))
+    run = subprocess.run([exe, "host"], env=env, capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0, (run.returncode, run.stderr[-2000:])
+    log = next(tmp_path.glob("CoCoPeLiaDgemmRunner_MI355X_*.log"))
+    parts = [p.strip() for p in log.read_text().strip().split(",")]
+    assert len(parts) == 18 and parts[:6] == ["128", "1", "1", "0", "N", "T"] and [int(p) for p in parts[8:11]] == [300, 200, 100]
+    # the row is in the log now: the CHECKLOG helper refuses to repeat the configuration once it is given the
+    # returned controller (exit status 1, as in the reference)
+    probe = tmp_path / "probe.cpp"
+    probe.write_text('#include "Testing.hpp"\nint main() { ATC c; c.T = 128; c.active_unit_num = 1; c.active_unit_id_list[0] = 0;\n'
+                     ' CheckLogLvl3("%s", &c, \'N\', \'T\', 1.2, 1.1, 300, 200, 100, -1, -1, -1, -1); return 0; }\n' % log)
+    exe2 = str(tmp_path / "probe")
+    run = subprocess.run(["g++", "-std=c++17", "-I", os.path.join(ROOT, "include"), str(probe), "-o", exe2, "-L", libdir, "-lparalia",
+                          "-Wl,-rpath," + libdir, "-ldl", "-lpthread"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-3000:]
+    run = subprocess.run([exe2], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 1 and "found. Quiting" in run.stderr

@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from gpu_util import Buf, sync
+from gpu_util import Buf, sync, check_daxpy_against_blas
 from oracle_binding import ptr, rand_f32, rand_f64
 
 pytestmark = pytest.mark.gpu
@@ -230,11 +230,6 @@ def test_dgemm_large_checksum(pkg, L):
         assert d / (abs(alpha) * np.linalg.norm(Am[i:i + 64, :]) * np.linalg.norm(Bm[:, j:j + 64]) + abs(beta) * np.linalg.norm(Cm[i:i + 64, j:j + 64])) < TOL64
 
 
-def scaled_ulp(a, b, alpha, x, y0):
-    scale = np.maximum(np.maximum(np.abs(alpha * x), np.abs(y0)), np.maximum(np.abs(a), np.abs(b)))
-    return float(np.max(np.abs(a - b) / np.spacing(scale)))
-
-
 @pytest.mark.parametrize("locs", [(0, 0), (-1, -1), (-1, 0), (0, -1), (-2, -2)])
 @pytest.mark.parametrize("T", [-1, 1000, 1 << 16])
 def test_daxpy_routine(pkg, L, orc, openblas, locs, T):
@@ -250,7 +245,7 @@ def test_daxpy_routine(pkg, L, orc, openblas, locs, T):
     assert np.array_equal(got, fused)
     ref = y0.copy()
     assert openblas.orc_openblas_daxpy(n, alpha, ptr(x), 1, ptr(ref), 1) == 0
-    assert orc.orc_max_ulp_f64(ptr(got), ptr(ref), n) <= 1 or scaled_ulp(got, ref, alpha, x, y0) <= 1.5
+    check_daxpy_against_blas(orc, got, ref, alpha, x, y0)
     assert np.array_equal(bx.get(), x)
     if T > 0 and min(locs) < 0:
         assert info.T == T and info.subkernel_num == -(-n // T)
@@ -381,3 +376,67 @@ def test_random_blas1_cases(pkg, L, orc, seed):
     orc.orc_daxpy(n, alpha, ptr(x), incx, ptr(ref), incy)
     assert np.array_equal(by.get(), ref)
     assert np.array_equal(bx.get(), x)
+
+
+def test_command_timeline_of_a_streamed_call(pkg, L, orc, openblas):
+    """PARALiA_trace_enable: every command of the plan comes back with its stream and its start / end time.  The rows
+    must be the plan (one tile GEMM per subkernel, one fetch per tile of A and B, one write-back per C tile), ordered in
+    time on each stream, with every GEMM starting after the fetches of its two tiles ended; and tracing must not
+    change the result."""
+    M, N, K, T = 700, 600, 500, 256
+    A, B, C0 = rand_f64(M * K, 1), rand_f64(K * N, 2), rand_f64(M * N, 3)
+    ref = openblas_ref(openblas, np.float64, "N", "N", M, N, K, 1.0, 0.0, A, M, B, K, C0, M)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
+    pkg.check(L.PARALiA_trace_enable(1), "trace on")
+    try:
+        info = call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=T)
+        n = int(L.PARALiA_trace_read(None, 0))
+        buf = (C.c_double * (7 * n))()
+        assert L.PARALiA_trace_read(buf, n) == n
+    finally:
+        pkg.check(L.PARALiA_trace_enable(0), "trace off")
+    assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.0, 0.0, A, M, K, M, B, K, N, K, C0) < TOL64
+    rows = [tuple(buf[7 * i:7 * i + 7]) for i in range(n)]
+    Mg, Ng, Kg = -(-M // T), -(-N // T), -(-K // T)
+    kinds = [int(r[0]) for r in rows]
+    assert kinds.count(3) == Mg * Ng * Kg == info.subkernel_num
+    assert kinds.count(0) == Mg * Kg and kinds.count(1) == Kg * Ng and kinds.count(2) == 0 and kinds.count(5) == Mg * Ng
+    fetch_end = {}
+    last_on_stream = {}
+    for kind, mi, ni, ki, stream, t0, t1 in rows:
+        assert 0.0 <= t0 <= t1
+        assert t0 >= last_on_stream.get(stream, 0.0) - 1e-3        # a stream runs its commands in order
+        last_on_stream[stream] = t1
+        if kind == 0:
+            fetch_end[("A", int(mi), int(ki))] = t1
+        elif kind == 1:
+            fetch_end[("B", int(ki), int(ni))] = t1
+        elif kind == 3:
+            assert t0 >= fetch_end[("A", int(mi), int(ki))] - 1e-3 and t0 >= fetch_end[("B", int(ki), int(ni))] - 1e-3
+    assert int(L.PARALiA_trace_read(None, 0)) == 0                  # switched off: the rows are gone
+
+
+def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg, L, orc, openblas):
+    """PARALiA_runtime_shutdown (the reference's CoCoPeLiaFreeResources + PARALiADevCacheFree): pool, streams, events and
+    cached problems go; device memory returns; the routines work again afterwards, every kind of them."""
+    M, N, K = 640, 512, 384
+    A, B, C0 = rand_f64(M * K, 4), rand_f64(K * N, 5), rand_f64(M * N, 6)
+    ref = openblas_ref(openblas, np.float64, "N", "T", M, N, K, 1.5, 0.5, A, M, B, N, C0, M)
+    free0, free1, total = C.c_longlong(), C.c_longlong(), C.c_longlong()
+    for rep in range(2):
+        bA, bB, bC = place(pkg, A, -1), place(pkg, B, -2), place(pkg, C0, -1)
+        call_gemm(pkg, L, np.float64, "N", "T", M, N, K, 1.5, 0.5, bA, M, bB, N, bC, M, T=128)
+        assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.5, 0.5, A, M, K, M, B, N, K, N, C0) < TOL64
+        x, y = place(pkg, rand_f64(100000, 7), -1), place(pkg, rand_f64(100000, 8), -1)
+        r = C.c_double(0.0)
+        pkg.check(L.PARALiA_ddot(100000, x.ptr, 1, y.ptr, 1, C.byref(r), -1, None), "ddot")
+        pool, entries = C.c_longlong(), C.c_long()
+        L.PARALiA_runtime_stats(None, None, C.byref(pool), C.byref(entries))
+        assert pool.value > 0 and entries.value >= 2
+        pkg.check(L.pl_mem_info(C.byref(free0), C.byref(total)), "mem info")
+        pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
+        pkg.check(L.pl_mem_info(C.byref(free1), C.byref(total)), "mem info")
+        L.PARALiA_runtime_stats(None, None, C.byref(pool), C.byref(entries))
+        assert pool.value == 0 and entries.value == 0
+        assert free1.value >= free0.value                            # the pool and the workspaces went back
+    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown twice is harmless")
