@@ -217,7 +217,7 @@ int PARALiA_autotune(const char* db_dir, const char* func, long D1, long D2, lon
                      int beta_zero, long T_in, long long pool_budget_bytes, pl_atc_info* info);
 /* static GEMM plan (CreateSubkernelsDgemm + request_data + run_operation, dgemm.cpp:123-205, Subkernel.cpp:90-247) */
 #define PL_PLAN_MAX_WAITS 12
-#define PL_PLAN_ROW (10 + PL_PLAN_MAX_WAITS)
+#define PL_PLAN_ROW (11 + PL_PLAN_MAX_WAITS)
 long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
                        int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]);
 /* makespan of one order (order_id >= 0) or of the best candidate (< 0) on the simulated H2D / compute / D2H pipeline;

@@ -255,6 +255,22 @@ paralia::StageTimes nominal_stage_times(const ProblemDesc& d, long T) {
 
 }  // namespace
 
+// What one launch over several k tiles of a C tile saves against one launch per k tile, per launch saved.  The fp32
+// kernel's larger macro tiles leave no room for a second workgroup on a compute unit, so nothing overlaps a
+// workgroup's prologue (first panels) and epilogue (the read-modify-write of its part of C): measured on sgemm
+// 32768^3 N/T at T = 4096, 336 launches fewer took 13.5 ms less = 40 us each, for one round of 256 tiles of 256 x 256
+// per launch.  The fp64 kernel runs two workgroups per compute unit that cover each other's ends: joining its launches
+// changed nothing (124.0 against 124.3 ms on dgemm 16384^3), so there the planner is not offered the choice.
+static double paralia_merge_saving(const ProblemDesc& d, long T) {
+  const char* env = getenv("PARALIA_MERGE_CHAINS");  // "0": never merge, "1": offer it for every type
+  if (env && *env && atoi(env) == 0) return 0.0;
+  if (d.dtype_sz != 4 && !(env && atoi(env) == 1)) return 0.0;
+  // a launch with fewer workgroups than compute units wastes that much less of the device: scale by the rounds of 256
+  // workgroups it amounts to, as a fraction
+  const double rounds = (double)((T + 255) / 256) * (double)((T + 255) / 256) / 256.0;
+  return 40e-6 * rounds;
+}
+
 paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   const ProblemDesc& d = atc->problem;
   if (!atc->has_db || !atc->unit_modeler_list[0]) return nominal_stage_times(d, T);
@@ -271,6 +287,7 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.d2h_ti = d2h->ti; st.d2h_tb = d2h->tb;
   st.h2d_sl = std::max(1.0, h2d->sl); st.d2h_sl = std::max(1.0, d2h->sl);
   st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
+  st.merge_saving = paralia_merge_saving(d, T);
   return st;
 }
 

@@ -242,7 +242,8 @@ static paralia::GemmProblem gp_of(long M, long N, long K, long T, int a_remote, 
 }
 
 // Builds the static plan and writes it as rows of PL_PLAN_ROW ints:
-// kind, mi, ni, ki, stream, block, a_block, b_block, beta_mode, nwait, wait[0..PL_PLAN_MAX_WAITS-1].
+// kind, mi, ni, ki, stream, block, a_block, b_block, beta_mode, nwait, wait[0..PL_PLAN_MAX_WAITS-1], kn (k tiles of a
+// GEMM launch; more than 1 only for order ids of 80000 and above, the merged K chains).
 // stats: [blocks_used, fetch_A, fetch_B, fetch_C, evictions, subkernels].  Returns the number of commands.
 long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
                        int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]) {
@@ -261,6 +262,7 @@ long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remot
         r[0] = c.kind; r[1] = c.mi; r[2] = c.ni; r[3] = c.ki; r[4] = c.stream; r[5] = c.block; r[6] = c.a_block; r[7] = c.b_block;
         r[8] = c.beta_mode; r[9] = c.nwait;
         for (int w = 0; w < PL_PLAN_MAX_WAITS; ++w) r[10 + w] = w < c.nwait ? c.wait[w] : -1;
+        r[10 + PL_PLAN_MAX_WAITS] = c.kn;
       }
   });
   return n;

@@ -13,7 +13,8 @@ namespace paralia {
 
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
-  order_id %= 40000;                       // the eviction policy does not change the order
+  order_id %= ORDER_MERGE_CHAINS;          // merging launches does not change the order
+  order_id %= 40000;                       // nor does the eviction policy
   const bool repeat = order_id >= 20000;  // every panel k-outer, not only the first
   const int orient = (order_id % 20000) / 10000;
   int w = order_id % 10000;
@@ -67,7 +68,7 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   return order;
 }
 
-std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe) {
+std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool merge) {
   std::vector<int> ids;
   ids.push_back(order_id_of(1, 0));  // the reference's index order; needs the fewest blocks
   if (!(p.a_remote || p.b_remote || p.c_remote)) return ids;
@@ -103,6 +104,11 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe) {
   if (limited) {
     const size_t n = ids.size();
     for (size_t i = 0; i < n; ++i) ids.push_back(40000 + ids[i]);
+  } else if (merge && p.Kg() > 1) {
+    // the whole working set fits: the orders that run K chains back to back also with those chains as one launch
+    const size_t n = ids.size();
+    for (size_t i = 0; i < n; ++i)
+      if (ids[i] < 20000) ids.push_back(ORDER_MERGE_CHAINS + ids[i]);
   }
   return ids;
 }
@@ -127,8 +133,14 @@ struct Block {
 void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w) {
   if (w < 0) return;
   if (cmds[w].stream == c.stream) return;  // stream order already covers it
-  for (int i = 0; i < c.nwait; ++i)
+  for (int i = 0; i < c.nwait; ++i) {
     if (c.wait[i] == w) return;
+    if (cmds[c.wait[i]].stream == cmds[w].stream) {
+      // streams run their commands in order: the later of two commands of one stream covers the earlier
+      if (w > c.wait[i]) { c.wait[i] = w; cmds[w].signals = true; }
+      return;
+    }
+  }
   if (c.nwait >= MAX_WAITS) throw std::runtime_error("gemm plan: too many dependencies on one command");
   c.wait[c.nwait++] = w;
   cmds[w].signals = true;
@@ -142,6 +154,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
   plan.p = p;
   plan.order_id = order_id;
   plan.task_order = gemm_task_order(p, order_id);
+  const bool merge = order_id >= ORDER_MERGE_CHAINS;
+  order_id %= ORDER_MERGE_CHAINS;
   const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
   const int NQ = std::max(1, std::min(p.exec_queues, MAX_EXEC_QUEUES));
   const bool any_remote = p.a_remote || p.b_remote || p.c_remote;
@@ -163,7 +177,17 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
   // FIFO: never-used blocks first, then released blocks oldest first, so a recycled block's previous users
   // (a write-back still in flight, say) have had the longest time to finish before its new writer waits on them
   std::deque<int> free_list;
-  for (int b = 0; b < (int)blocks.size(); ++b) free_list.push_back(b);
+  int first_dynamic = 0;
+  if (merge) {
+    // panel layout: every tile of A and B has its own block for the whole call, the k tiles of a panel side by side
+    plan.panels = true;
+    if (p.a_remote) { plan.a_first = first_dynamic; first_dynamic += Mg * Kg; }
+    if (p.b_remote) { plan.b_first = first_dynamic; first_dynamic += Kg * Ng; }
+    const int c_min = p.c_remote ? (p.beta_zero ? 1 : 2) : 0;
+    if (any_remote && (long)first_dynamic + c_min > p.pool_blocks)
+      throw std::runtime_error("PARALiA gemm: device block pool too small for the panel layout of merged K chains");
+  }
+  for (int b = first_dynamic; b < (int)blocks.size(); ++b) free_list.push_back(b);
   int c_seq = 0;
   const bool slack_policy = order_id >= 40000;
   int cur_pos = 0;
@@ -189,6 +213,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     // simulation decides.
     int b = -1;
     int best_next = -1, best_touch = INT_MAX;
+    if (plan.panels && free_list.empty())  // the tiles of A and B keep their blocks for the whole call: nothing to evict
+      throw std::runtime_error("PARALiA gemm: device block pool too small for the panel layout of merged K chains");
     if (free_list.empty() || slack_policy) {
       for (int i = 0; i < (int)blocks.size(); ++i) {
         if (i == pin1 || i == pin2) continue;
@@ -240,6 +266,21 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     pend.push_back(cmd_idx);
   };
 
+  struct OpenChain {
+    bool active = false;
+    int ci = -1, mi = -1, ni = -1, ki0 = -1, kn = 0, ablk = -1, bblk = -1, beta_mode = BETA_ONE;
+    std::vector<int> waits;
+  } open;
+  auto close_chain = [&]() -> int {
+    Cmd c;
+    c.kind = CMD_GEMM; c.mi = open.mi; c.ni = open.ni; c.ki = open.ki0; c.kn = open.kn; c.stream = STREAM_EXEC0 + queue_of[open.ci];
+    c.block = p.c_remote ? c_blk[open.ci] : -1; c.a_block = open.ablk; c.b_block = open.bblk; c.beta_mode = open.beta_mode;
+    cmds.push_back(c);
+    for (int x : open.waits) add_wait(cmds, cmds.back(), x);
+    open.active = false;
+    return (int)cmds.size() - 1;
+  };
+
   for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
     const int t = plan.task_order[pos];
     const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
@@ -253,7 +294,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     if (p.a_remote) {
       if (a_blk[ai] < 0) {
         std::vector<int> w;
-        const int b = alloc(p.b_remote ? b_blk[bi] : -1, -1, w);
+        const int b = plan.panels ? plan.a_first + mi * Kg + ki : alloc(p.b_remote ? b_blk[bi] : -1, -1, w);
+        blocks[b].ever_used = true;
         Cmd c;
         c.kind = CMD_FETCH_A; c.mi = mi; c.ki = ki; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
@@ -268,7 +310,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
     if (p.b_remote) {
       if (b_blk[bi] < 0) {
         std::vector<int> w;
-        const int b = alloc(ablk, -1, w);
+        const int b = plan.panels ? plan.b_first + ni * Kg + ki : alloc(ablk, -1, w);
+        blocks[b].ever_used = true;
         Cmd c;
         c.kind = CMD_FETCH_B; c.ki = ki; c.ni = ni; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
@@ -294,31 +337,41 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
         beta_mode = BETA_USER;  // resident C: plain read-modify-write (dgemm.cpp:259-260)
       }
     }
-    {
-      Cmd c;
-      c.kind = CMD_GEMM; c.mi = mi; c.ni = ni; c.ki = ki; c.stream = STREAM_EXEC0 + queue_of[ci];
-      c.block = p.c_remote ? c_blk[ci] : -1; c.a_block = ablk; c.b_block = bblk; c.beta_mode = beta_mode;
-      cmds.push_back(c);
-      for (int x : gemm_waits) add_wait(cmds, cmds.back(), x);
+    // The launch of this subkernel.  With merged K chains a subkernel that continues the chain of the previous one in
+    // the order (same C tile, next k tile) joins its launch, which is only written out when the chain ends: by then
+    // every fetch it depends on is already in the command list.
+    if (merge && open.active && open.ci == ci && open.ki0 + open.kn == ki) {
+      ++open.kn;
+      open.waits.insert(open.waits.end(), gemm_waits.begin(), gemm_waits.end());
+    } else {
+      if (open.active) close_chain();
+      open.active = true;
+      open.ci = ci; open.mi = mi; open.ni = ni; open.ki0 = ki; open.kn = 1;
+      open.ablk = ablk; open.bblk = bblk; open.beta_mode = beta_mode;
+      open.waits = gemm_waits;
     }
-    const int gemm_idx = (int)cmds.size() - 1;
-    if (ablk >= 0) note_reader(ablk, gemm_idx);
-    if (bblk >= 0) note_reader(bblk, gemm_idx);
-    // A tile that no later subkernel reads gives its block back at once (its readers stay pending on the block): the
-    // FIFO then hands out the longest-dead block first, so the fetch that reuses it rarely waits and the copy stream
-    // can run a whole k-step ahead of the subkernels even when the pool is much smaller than the operands.
-    if (ablk >= 0 && a_ptr[ai] == (int)a_uses[ai].size()) {
-      blocks[ablk].kind = -1; blocks[ablk].idx = -1;
-      a_blk[ai] = -1;
-      free_list.push_back(ablk);
-    }
-    if (bblk >= 0 && b_ptr[bi] == (int)b_uses[bi].size()) {
-      blocks[bblk].kind = -1; blocks[bblk].idx = -1;
-      b_blk[bi] = -1;
-      free_list.push_back(bblk);
+    int gemm_idx = -1;
+    if (!merge) {
+      gemm_idx = close_chain();
+      if (ablk >= 0) note_reader(ablk, gemm_idx);
+      if (bblk >= 0) note_reader(bblk, gemm_idx);
+      // A tile that no later subkernel reads gives its block back at once (its readers stay pending on the block): the
+      // FIFO then hands out the longest-dead block first, so the fetch that reuses it rarely waits and the copy stream
+      // can run a whole k-step ahead of the subkernels even when the pool is much smaller than the operands.
+      if (ablk >= 0 && a_ptr[ai] == (int)a_uses[ai].size()) {
+        blocks[ablk].kind = -1; blocks[ablk].idx = -1;
+        a_blk[ai] = -1;
+        free_list.push_back(ablk);
+      }
+      if (bblk >= 0 && b_ptr[bi] == (int)b_uses[bi].size()) {
+        blocks[bblk].kind = -1; blocks[bblk].idx = -1;
+        b_blk[bi] = -1;
+        free_list.push_back(bblk);
+      }
     }
 
     if (++fired[ci] == Kg && p.c_remote) {
+      if (open.active) gemm_idx = close_chain();
       const int accb = c_blk[ci];
       int last = gemm_idx;
       if (!p.beta_zero) {
@@ -347,7 +400,14 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
       c_blk[ci] = -1;
     }
   }
-  for (const Block& b : blocks) plan.blocks_used += b.ever_used ? 1 : 0;
+  if (open.active) close_chain();
+  // with panels the pool is addressed by block number up to the last one in use
+  if (plan.panels) {
+    for (int b = 0; b < (int)blocks.size(); ++b)
+      if (blocks[b].ever_used) plan.blocks_used = b + 1;
+  } else {
+    for (const Block& b : blocks) plan.blocks_used += b.ever_used ? 1 : 0;
+  }
   return plan;
 }
 
@@ -428,7 +488,10 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
         case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
         case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
         case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
-        case CMD_GEMM: dur = st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(c.ki)); break;
+        case CMD_GEMM:
+          for (int k = c.ki; k < c.ki + c.kn; ++k) dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
+          if (c.kn > 1) dur = std::max(0.5 * dur, dur - (c.kn - 1) * st.merge_saving * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2);
+          break;
         case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
         case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
       }
@@ -461,7 +524,7 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   int best_id = -1;
   PipelineResult best;
   std::string last_err;
-  for (int id : gemm_candidate_orders(p, probe)) {
+  for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0)) {
     try {
       GemmPlan plan = build_gemm_plan(p, id);
       PipelineResult r = simulate_plan(plan, st);

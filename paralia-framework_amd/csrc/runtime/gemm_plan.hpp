@@ -47,6 +47,7 @@ struct Cmd {
   int block = -1;     // block written by a FETCH; accumulator block of GEMM / REDUCE / WRITEBACK (-1: caller's C)
   int a_block = -1;   // GEMM: block of the A tile (-1: caller's memory); REDUCE: block holding the fetched source C
   int b_block = -1;   // GEMM: block of the B tile (-1: caller's memory)
+  int kn = 1;         // GEMM: number of consecutive k tiles ki .. ki + kn - 1 multiplied by this one launch
   int beta_mode = BETA_ONE;
   int nwait = 0;
   int wait[MAX_WAITS];  // earlier commands on other streams that must have completed
@@ -56,6 +57,13 @@ struct Cmd {
 struct GemmPlan {
   GemmProblem p;
   int order_id = 0;
+  // Panel layout: the k tiles of an A row panel (and of a B column panel) sit in consecutive blocks, block
+  // a_first + mi * Kg + ki for A(mi, ki) and b_first + ni * Kg + ki for B(ki, ni), and inside a panel the tiles are
+  // placed so that the panel is ONE matrix with one leading dimension (for an operand that is contiguous along m or
+  // n: dense tiles one after the other; for an operand contiguous along k: the tiles stacked in a K x tile matrix).
+  // A launch can then multiply several k tiles at once.  Only when the pool holds every tile of A and B.
+  bool panels = false;
+  int a_first = -1, b_first = -1;
   std::vector<int> task_order;  // subkernel ids mi*Ng*Kg + ni*Kg + ki in firing order
   std::vector<Cmd> cmds;
   long blocks_used = 0;
@@ -71,10 +79,16 @@ struct GemmPlan {
 // one after the other; this is the family for block pools smaller than the working set.
 // + 40000: same order, but evictions prefer the tile untouched for longest among those not needed soon (instead of
 // the one needed farthest in the future), which lets fetches run ahead of the subkernels.
+// + 80000: panel layout (GemmPlan::panels) and merged K chains: wherever the order runs consecutive k-steps of one C
+// tile back to back, they become one launch over the joined k range.  That saves the launch's fixed cost -- for the
+// large fp32 tiles, whose workgroups hold a compute unit alone, the prologue and epilogue nothing else overlaps -- at
+// the price of starting only when all its tiles have arrived.  Needs a pool that holds the whole working set.
+constexpr int ORDER_MERGE_CHAINS = 80000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
 // probe = true: a handful of representative orders, enough to rank tile sizes before the full search
-std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe = false);
+// merge = true: also the variants with merged K chains (when the pool holds the whole working set)
+std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe = false, bool merge = false);
 
 // Throws std::runtime_error when pool_blocks cannot hold the minimum working set (3 blocks, dgemm.cpp:90-93).
 GemmPlan build_gemm_plan(const GemmProblem& p, int order_id);
@@ -93,6 +107,9 @@ struct StageTimes {
   double d2h_ti = 0, d2h_tb = 0;
   double h2d_sl = 1, d2h_sl = 1;     // how much slower a copy runs while the opposite direction is busy (>= 1)
   double t_reduce = 0;               // one T^2 scale-add
+  // seconds a launch over kn k tiles of a full T x T C tile takes less than kn separate launches, per launch saved
+  // (0: merging K chains is not worth considering for this kernel)
+  double merge_saving = 0;
 };
 struct PipelineResult {
   double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource

@@ -137,14 +137,15 @@ void HostStager::reserve(long long tile_bytes) {
   slot_bytes_ = tile_bytes;
 }
 
-void HostStager::fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream) {
+void HostStager::fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream, long ld_dst) {
   if (rows <= 0 || cols <= 0) return;
   const long long bytes = (long long)rows * cols * elem;
   reserve(bytes);
   const int s = (int)(in_next_++ % SLOTS);
   if (in_used_[s]) chk(pl_event_sync(in_ev_[s]), "event sync");  // the slot's previous tile has left for the device
   threads()->copy2d(in_[s], (size_t)rows * elem, src, (size_t)ld_src * elem, (size_t)rows * elem, cols);
-  chk(pl_copy_async(dst, in_[s], bytes, stream), "staged tile copy");
+  if (ld_dst <= 0 || ld_dst == rows) chk(pl_copy_async(dst, in_[s], bytes, stream), "staged tile copy");
+  else chk(pl_copy2d_async(dst, ld_dst, in_[s], rows, rows, cols, elem, stream), "staged tile copy");
   chk(pl_event_record(in_ev_[s], stream), "event record");
   in_used_[s] = true;
 }

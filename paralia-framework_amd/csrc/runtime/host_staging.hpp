@@ -55,8 +55,9 @@ class HostStager {
   ~HostStager();
   HostStager(const HostStager&) = delete;
   HostStager& operator=(const HostStager&) = delete;
-  // dst (device, dense, leading dimension = rows)  <-  src (pageable host, leading dimension ld_src), on `stream`.
-  void fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream);
+  // dst (device, leading dimension ld_dst; 0 = dense, i.e. rows)  <-  src (pageable host, leading dimension ld_src), on
+  // `stream`.
+  void fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream, long ld_dst = 0);
   // dst (pageable host, leading dimension ld_dst)  <-  src (device, dense) on `stream`; the host-side scatter happens
   // when the slot is needed again or in finish().
   void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream);

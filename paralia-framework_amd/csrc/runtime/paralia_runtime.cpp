@@ -317,6 +317,26 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
     chk(pl_event_record(R.res.timing_events[0], R.res.h2d), "event record");  // time zero of the timeline
   }
 
+  // Where a fetched tile of A / B lives on the device and with which leading dimension.  Without panels: its own
+  // block, dense.  With panels (GemmPlan::panels) the Kg blocks of a row panel of op(A) / column panel of op(B) hold one
+  // matrix: tiles one after the other when the operand is contiguous along m / n (leading dimension = tile rows), or a
+  // K x tile matrix with leading dimension K when it is contiguous along k.
+  const int Kg = p.Kg();
+  auto a_tile = [&](int block, int mi, int ki, long* ld) -> T* {
+    if (!plan.panels) { *ld = at ? p.tk(ki) : p.tm(mi); return (T*)R.pool.at(block); }
+    T* base = (T*)R.pool.at(plan.a_first + (long)mi * Kg);
+    if (at) { *ld = std::max(1L, p.K); return base + (long)ki * Tt; }
+    *ld = p.tm(mi);
+    return base + (long)ki * Tt * p.tm(mi);
+  };
+  auto b_tile = [&](int block, int ni, int ki, long* ld) -> T* {
+    if (!plan.panels) { *ld = bt ? p.tn(ni) : p.tk(ki); return (T*)R.pool.at(block); }
+    T* base = (T*)R.pool.at(plan.b_first + (long)ni * Kg);
+    if (!bt) { *ld = std::max(1L, p.K); return base + (long)ki * Tt; }
+    *ld = p.tn(ni);
+    return base + (long)ki * Tt * p.tn(ni);
+  };
+
   DrainOnError guard(R.res);
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
@@ -327,14 +347,18 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       case CMD_FETCH_A: {
         const long rows = at ? p.tk(c.ki) : p.tm(c.mi), cols = at ? p.tm(c.mi) : p.tk(c.ki);
         const T* src = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda;
-        if (pageable[0]) stager.fetch(R.pool.at(c.block), src, lda, rows, cols, sizeof(T), s);
-        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, lda, rows, cols, sizeof(T), s), "fetch A tile");
+        long ld_dst;
+        T* dst = a_tile(c.block, c.mi, c.ki, &ld_dst);
+        if (pageable[0]) stager.fetch(dst, src, lda, rows, cols, sizeof(T), s, ld_dst);
+        else chk(pl_copy2d_async(dst, ld_dst, src, lda, rows, cols, sizeof(T), s), "fetch A tile");
       } break;
       case CMD_FETCH_B: {
         const long rows = bt ? p.tn(c.ni) : p.tk(c.ki), cols = bt ? p.tk(c.ki) : p.tn(c.ni);
         const T* src = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb;
-        if (pageable[1]) stager.fetch(R.pool.at(c.block), src, ldb, rows, cols, sizeof(T), s);
-        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
+        long ld_dst;
+        T* dst = b_tile(c.block, c.ni, c.ki, &ld_dst);
+        if (pageable[1]) stager.fetch(dst, src, ldb, rows, cols, sizeof(T), s, ld_dst);
+        else chk(pl_copy2d_async(dst, ld_dst, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
       } break;
       case CMD_FETCH_C: {
         const long rows = p.tm(c.mi), cols = p.tn(c.ni);
@@ -343,14 +367,16 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
       } break;
       case CMD_GEMM: {
-        const long m = p.tm(c.mi), n = p.tn(c.ni), k = p.tk(c.ki);
+        const long m = p.tm(c.mi), n = p.tn(c.ni);
+        long k = 0;  // one launch over the k tiles ki .. ki + kn - 1 (kn > 1 only with the panel layout)
+        for (int kt = c.ki; kt < c.ki + c.kn; ++kt) k += p.tk(kt);
         const T* a;
         long la;
-        if (c.a_block >= 0) { a = (const T*)R.pool.at(c.a_block); la = at ? k : m; }
+        if (c.a_block >= 0) a = a_tile(c.a_block, c.mi, c.ki, &la);
         else { a = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda; la = lda; }
         const T* b;
         long lb;
-        if (c.b_block >= 0) { b = (const T*)R.pool.at(c.b_block); lb = bt ? n : k; }
+        if (c.b_block >= 0) b = b_tile(c.b_block, c.ni, c.ki, &lb);
         else { b = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb; lb = ldb; }
         T* cc;
         long lc;

@@ -24,12 +24,14 @@ int main(int argc, char** argv) {
     p.pool_blocks = pools[rng() % 9];
     if (p.subkernels() > 6000) continue;
     StageTimes st; st.t_exec = 1e-4; st.h2d_ti = 1e-5; st.h2d_tb = 2e-11; st.d2h_ti = 1e-5; st.d2h_tb = 2e-11; st.t_reduce = 1e-5; st.h2d_sl = 1.01; st.d2h_sl = 1.2;
+    st.merge_saving = (rng() % 2) ? 4e-6 : 0.0;
     try {
       if (rng() % 4 == 0) {
         PipelineResult r; pick_gemm_order(p, st, &r, rng() % 2);
       } else {
         const int orient = rng() % 2, w = rng() % 40;
-        const int id = orient * 10000 + w + ((w > 0 && rng() % 2) ? 20000 : 0) + ((rng() % 2) ? 40000 : 0);
+        int id = orient * 10000 + w + ((w > 0 && rng() % 2) ? 20000 : 0) + ((rng() % 2) ? 40000 : 0);
+        if (rng() % 3 == 0) id = ORDER_MERGE_CHAINS + orient * 10000 + w;  // merged K chains (refused unless the pool holds everything)
         GemmPlan plan = build_gemm_plan(p, id);
         PipelineResult r = simulate_plan(plan, st);
         if (!(r.t_total >= 0)) { printf("bad makespan\n"); return 1; }

@@ -440,3 +440,47 @@ def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg,
         assert pool.value == 0 and entries.value == 0
         assert free1.value >= free0.value                            # the pool and the workspaces went back
     pkg.check(L.PARALiA_runtime_shutdown(), "shutdown twice is harmless")
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("order", [80000, 80002, 90003])
+@pytest.mark.parametrize("locs", [(-1, -1, -1), (-1, -1, 0), (-2, -2, -1), (0, -1, -1)])
+def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs, monkeypatch):
+    """Order ids of 80000 and above: the k tiles of every A row panel and B column panel lie side by side on the device
+    and each K chain that the order runs back to back is ONE launch over the joined k range.  Integer-valued operands,
+    ragged tiles in all three dimensions (289 x 353 x 307 at T = 64: 5 x 6 x 5 tiles), every transpose (the panel of
+    an operand that is contiguous along k is a K x tile matrix, the other kind a row of dense tiles), operands pinned,
+    pageable or already on the device, beta = 0 over NaN and beta != 0 (fetched C, lazy reduce): bit for bit the
+    untiled result, in fp64 and fp32."""
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+    M, N, K, T = 289, 353, 307 + {80000: 0, 80002: 1, 90003: 2}[order], 64   # a new problem for the metadata cache per order
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    rng = np.random.default_rng(order + 7 * len(ta + tb))
+    for dtype, brute in ((np.float64, orc.orc_dgemm_bruteforce), (np.float32, orc.orc_sgemm_bruteforce)):
+        A = rng.integers(-4, 5, ra * ca).astype(dtype)
+        B = rng.integers(-4, 5, rb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, M * N).astype(dtype)
+        for beta in (0.0, 2.0):
+            ref = C0.copy()
+            brute(ta.encode(), tb.encode(), M, N, K, 3.0, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M)
+            start = np.full(M * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+            bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
+            info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 3.0, beta, bA, ra, bB, rb, bC, M, T=T)
+            assert info.order_id == order and info.subkernel_num == 5 * 6 * 5
+            assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
+
+
+def test_sgemm_autotuned_call_merges_k_chains(pkg, L, orc, openblas):
+    """No pin: for fp32 with A and B on the host the planner is offered the merged variants and its simulator takes
+    one when the product is bound by compute and the chains are long (12288 x 12288 x 16384 here); parity against
+    OpenBLAS."""
+    M = N = 12288
+    K = 16384
+    A, B, C0 = rand_f32(M * K, 1), rand_f32(N * K, 2), rand_f32(M * N, 3)
+    ref = openblas_ref(openblas, np.float32, "N", "T", M, N, K, 1.0, 1.0, A, M, B, N, C0, M)
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, 0)
+    info = call_gemm(pkg, L, np.float32, "N", "T", M, N, K, 1.0, 1.0, bA, M, bB, N, bC, M)
+    print("  T", info.T, "order", info.order_id, "predicted ms", info.pred_t * 1e3, flush=True)
+    assert info.order_id >= 80000
+    assert normwise(orc, np.float32, bC.get(), ref, M, N, M, 1.0, 1.0, A, M, K, M, B, N, K, N, C0) < TOL32

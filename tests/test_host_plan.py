@@ -320,3 +320,74 @@ def test_random_plans_are_safe_and_correct(pkg, seed):
     check_plan(rows, stats, M, N, K, T, a_r, b_r, c_r, beta_zero, eff_pool, nq)
     assert np.array_equal(replay(rows, M, N, K, T, alpha, beta, A, B, C, eff_pool), alpha * (A @ B) + beta * C)
     check_async_safety(rows)
+
+
+def expand_merged(rows):
+    """A plan with merged K chains (order ids of 80000 and above) rewritten as the equivalent plan with one GEMM row per
+    k tile, so that the checks above apply unchanged: the k tiles of a launch sit in consecutive blocks of its panels,
+    the launch's waits guard its first k-step, later k-steps follow on the same stream, and whoever waited for the
+    launch waits for its last k-step."""
+    out, new_index = [], {}
+    for i, r in enumerate(rows):
+        if r["kind"] == GEMM and r["kn"] > 1:
+            for s in range(r["kn"]):
+                e = dict(r, ki=r["ki"] + s, kn=1, waits=list(r["waits"]) if s == 0 else [],
+                         a_block=r["a_block"] + s if r["a_block"] >= 0 else -1, b_block=r["b_block"] + s if r["b_block"] >= 0 else -1,
+                         beta_mode=r["beta_mode"] if s == 0 else BETA_ONE)
+                out.append(e)
+        else:
+            out.append(dict(r, waits=list(r["waits"])))
+        new_index[i] = len(out) - 1
+    for e in out:
+        e["waits"] = [new_index[w] for w in e["waits"]]
+    return out
+
+
+@pytest.mark.parametrize("order", [80000, 80001, 80002, 90000, 90002])
+@pytest.mark.parametrize("locs", [(1, 1, 1), (1, 1, 0), (0, 1, 1), (1, 0, 0)])
+@pytest.mark.parametrize("beta_zero", [0, 1])
+def test_merged_chain_plans(pkg, order, locs, beta_zero):
+    """Merged K chains: fewer GEMM launches than subkernels, every (mi, ni, ki) still covered exactly once, the tiles of
+    A and B in their fixed panel blocks (A(mi, ki) in block mi * Kg + ki, B(ki, ni) behind them in ni * Kg + ki), each
+    fetched once, and the expanded plan keeps every invariant, replays exactly and orders every hazard."""
+    M, N, K, T = 90, 70, 110, 32
+    a_r, b_r, c_r = locs
+    Mg, Ng, Kg = grids(M, N, K, T)
+    rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
+    gemms = [r for r in rows if r["kind"] == GEMM]
+    assert sum(g["kn"] for g in gemms) == Mg * Ng * Kg and len(gemms) < Mg * Ng * Kg
+    assert any(g["kn"] == Kg for g in gemms)                  # the tile-by-tile part of the order runs whole chains
+    a_first = 0
+    b_first = Mg * Kg if a_r else 0
+    for r in rows:
+        if r["kind"] == FETCH_A:
+            assert r["block"] == a_first + r["mi"] * Kg + r["ki"]
+        if r["kind"] == FETCH_B:
+            assert r["block"] == b_first + r["ni"] * Kg + r["ki"]
+    full = 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
+    flat = expand_merged(rows)
+    check_plan(flat, stats, M, N, K, T, a_r, b_r, c_r, beta_zero, full, 2)
+    assert stats[1] == (Mg * Kg if a_r else 0) and stats[2] == (Kg * Ng if b_r else 0) and stats[4] == 0
+    rng = np.random.default_rng(order + beta_zero)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64)
+    B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C = rng.integers(-5, 6, (M, N)).astype(np.float64)
+    alpha, beta = 2.0, (0.0 if beta_zero else 3.0)
+    assert np.array_equal(replay(flat, M, N, K, T, alpha, beta, A, B, C, full), alpha * (A @ B) + beta * C)
+    check_async_safety(flat)
+
+
+def test_merged_chains_need_the_whole_working_set_and_pay_only_with_a_saving(pkg, L):
+    import ctypes as C
+    with pytest.raises(pkg.ParaliaError, match="panel layout"):
+        pkg.plan_rows(100, 100, 100, 32, 1, 1, 1, 0, 8, 2, 12, 80000)     # 4 x 4 tiles of A and of B do not fit 12 blocks
+    # simulator: the same order with and without merging costs the same when a merged launch saves nothing ...
+    args = (4096, 4096, 4096, 512, 1, 1, 0, 0, 4, 2, 0)
+    st = (1e-3, 1e-5, 2e-11, 1e-5, 2e-11, 1e-5, 1.0, 1.0)
+    picked, busy = C.c_int(), (C.c_double * 3)()
+    plain = L.PARALiA_gemm_plan_simulate(*args, 2, *st, C.byref(picked), busy)
+    merged = L.PARALiA_gemm_plan_simulate(*args, 80002, *st, C.byref(picked), busy)
+    assert plain > 0 and abs(merged - plain) <= 1e-9 * plain
+    # ... and the search offers merged orders only to a kernel with such a saving (none through this entry point)
+    best = L.PARALiA_gemm_plan_simulate(*args, -1, *st, C.byref(picked), busy)
+    assert picked.value < 80000 and best <= plain
