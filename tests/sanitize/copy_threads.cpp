@@ -17,6 +17,10 @@ int pl_event_destroy(void* e) { free(e); return 0; }
 int pl_event_record(void*, void*) { return 0; }
 int pl_event_sync(void*) { return 0; }
 int pl_copy_async(void* d, const void* s, long long b, void*) { memcpy(d, s, b); return 0; }
+int pl_copy2d_async(void* d, long ldd, const void* s, long lds, long rows, long cols, int elem, void*) {
+  for (long c = 0; c < cols; ++c) memcpy((char*)d + c * ldd * elem, (const char*)s + c * lds * elem, rows * elem);
+  return 0;
+}
 }
 int main() {
   using namespace paralia;
