@@ -29,6 +29,9 @@
 #ifndef PLK_F32_BK
 #define PLK_F32_BK 16
 #endif
+#ifndef PLK_F64_PAIR
+#define PLK_F64_PAIR 0
+#endif
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
 #endif
@@ -259,7 +262,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // rows a lane needs for its NB blocks are adjacent in LDS and come with one 8- or 16-byte read instead of NB 4-byte
   // ones (every operand read issued between MFMAs costs MFMA issue slots: 1 read per MFMA loses 8 % of the pipe rate,
   // 1 per 2 about half of that).  The epilogue maps the accumulators back with the same rule.
-  constexpr bool A_PAIR = sizeof(T) == 4 && !AK, B_PAIR = sizeof(T) == 4 && !BKM;
+  constexpr bool PAIRED = sizeof(T) == 4 || PLK_F64_PAIR;
+  constexpr bool A_PAIR = PAIRED && !AK, B_PAIR = PAIRED && !BKM;
   const T* const lane_a = smem + LA::at(kk, wm + (A_PAIR ? NBM * idx : idx));         // this lane's A operand of k-step 0, block 0
   const T* const lane_b = smem + ASZ + LB::at(kk, wn + (B_PAIR ? NBN * idx : idx));  // this lane's B operand
   constexpr int A_KS = LA::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : LA::at(0, BLK);    // strides per k-step / per block
