@@ -10,7 +10,9 @@
 //   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2 or 4 x 4);
 //   * A and B k-panels (16 elements deep, 32 for the large tile) are staged global -> registers -> LDS,
 //     double-buffered, one barrier per k-panel; the next panel's global loads are in flight while the current one is
-//     multiplied;
+//     multiplied; when both operands are MN-major (NT) and a panel row is exactly 1 KiB (fp64 128 x 128, fp32
+//     256 x 256) the rows go global -> LDS directly instead (fp64 NT 72.8 -> 73.7, fp32 NT 148.7 -> 149.9 TFLOP/s at
+//     8192^3);
 //   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
 //     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
@@ -31,6 +33,15 @@
 #endif
 #ifndef PLK_F64_PAIR
 #define PLK_F64_PAIR 0
+#endif
+// Bit 0: fp64, bit 1: fp32 -- MN-major operand panels whose rows are exactly 1 KiB go global -> LDS without passing
+// registers (see dma_row).
+#ifndef PLK_DIRECT
+#define PLK_DIRECT 3
+#endif
+// scheduling class the compiler's instruction-group pass files the LDS-DMA loads under (all DS instructions)
+#ifndef PLK_DMA_MASK
+#define PLK_DMA_MASK 0x080
 #endif
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
@@ -170,6 +181,18 @@ __device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Tra
   for (int i = 0; i < L::NV; ++i) lds_put<T, KMAJOR>(xs + L::slot_offset(tid, i), regs[i]);
 }
 
+// Row `row` of an MN-major panel straight from global memory into LDS (global_load_lds_dwordx4): the 64 lanes of a wave
+// fetch 16 bytes each and the hardware puts lane l's at the wave's LDS base + 16 l, so one instruction moves one 1 KiB
+// row (256 floats or 128 doubles) and neither staging registers nor LDS store instructions are spent on it.  The LDS
+// base is wave-uniform, which is why the row stride of the padded layout can stay.
+template <typename T>
+__device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs, int row, int lane, int s_mn) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const T* p = g + (16 / (int)sizeof(T)) * lane + (long)row * ld;
+  __builtin_amdgcn_global_load_lds(p, xs + row * s_mn, 16, 0, 0);
+#endif
+}
+
 // Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
 // give each XCD a contiguous range of logical ids, then walk that range in groups of 8 block rows.
 __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, int& bn) {
@@ -301,46 +324,79 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     // where the MFMA queue still has a k-step of work behind it.  The loop body has no branches: past the end, the
     // loads re-read the last panel and the stores fill a buffer nobody reads.
     T am[2][KV][NBM], bnv[2][KV][NBN];
-    auto fetch_fast = [&](int kt) {
-      gload<LA, T, false>(Ab + kt * a_kstep, lda, 0, 0, true, ra, tid);
-      gload<LB, T, false>(Bb + kt * b_kstep, ldb, 0, 0, true, rb, tid);
-    };
-    fetch_fast(0);
-    lds_store<LA, T, AK>(smem, ra, tid);
-    lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
-    fetch_fast(min(1, nkt - 1));
+    // MN-major operands whose panel rows are 1 KiB skip the registers (dma_row): panel kt+1 is requested while panel kt
+    // is multiplied and must have landed (vmcnt) before the panel's barrier; operands staged through registers are
+    // loaded two panels ahead as before.
+    constexpr bool DIR_T = ((PLK_DIRECT >> (sizeof(T) == 4 ? 1 : 0)) & 1) != 0;
+    // only when both operands qualify: with one operand direct and one staged the wait in front of the barrier also
+    // covers the staged operand's newer loads (fp32 256 x 128 NN: 143.8 -> 137.4 TFLOP/s)
+    constexpr bool A_DIR = DIR_T && !AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024;
+    constexpr bool B_DIR = A_DIR;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    if constexpr (A_DIR) {
+#pragma unroll
+      for (int i = 0; i < NVA; ++i) dma_row<T>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
+    } else {
+      gload<LA, T, false>(Ab, lda, 0, 0, true, ra, tid);
+      lds_store<LA, T, AK>(smem, ra, tid);
+      gload<LA, T, false>(Ab + min(1, nkt - 1) * a_kstep, lda, 0, 0, true, ra, tid);
+    }
+    if constexpr (B_DIR) {
+#pragma unroll
+      for (int i = 0; i < NVB; ++i) dma_row<T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
+    } else {
+      gload<LB, T, false>(Bb, ldb, 0, 0, true, rb, tid);
+      lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
+      gload<LB, T, false>(Bb + min(1, nkt - 1) * b_kstep, ldb, 0, 0, true, rb, tid);
+    }
+    if constexpr (A_DIR || B_DIR) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the requested rows are in LDS
     __syncthreads();
     read_ops(0, 0, am[0], bnv[0]);
-    constexpr int NVS = NVA + NVB, SIDE = 2 * NVS;           // NVS LDS stores and NVS global loads per panel
+    // side instructions of a panel, in issue order: the row requests of the direct operands, then for the staged ones
+    // NREG LDS stores and NREG global loads
+    constexpr int NDIR = (A_DIR ? NVA : 0) + (B_DIR ? NVB : 0), NREG = NVA + NVB - NDIR;
+    constexpr int SIDE = NDIR + 2 * NREG;
     constexpr int PER_STEP = (SIDE + KS - 2) / (KS - 1);     // side instructions placed in each pre-barrier k-step
     constexpr int MFMAS = KV * NBM * NBN;
     constexpr bool ALT = sizeof(T) == 8;
+    // staged vector number r -> index into (A vectors, then B vectors)
+    constexpr int REG0 = A_DIR ? NVA : 0;
+    // one side instruction of the panel (row request, LDS store or global load), by its number in issue order
+    auto side_item = [&](int slot, T* nxt_a, T* nxt_b, const T* ga, const T* gb) {
+      if (slot < NDIR) {
+        const int vec = (A_DIR ? 0 : NVA) + slot;  // direct rows: A's first when both are direct
+        if (vec < NVA) dma_row<T>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
+        else dma_row<T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
+        return;
+      }
+      // staged side instruction number r of the panel: fp64 alternates store / load vector by vector (the load
+      // refills the registers the store has just read), fp32 issues all stores first, then all loads;
+      // measured at 8192^3: fp64 73.5 against 72.0 TFLOP/s, fp32 141.3 against 139.9 the other way round
+      const int r = slot - NDIR;
+      const bool is_store = ALT ? (r % 2 == 0) : (r < NREG);
+      const int vec = REG0 + (ALT ? r / 2 : (r < NREG ? r : r - NREG));  // 0 .. NVA-1: A, NVA .. : B
+      if (is_store) {
+        if (vec < NVA) lds_store_one<LA, T, AK>(nxt_a, ra[vec], tid, vec);
+        else lds_store_one<LB, T, BKM>(nxt_b, rb[vec - NVA], tid, vec - NVA);
+      } else {
+        if (vec < NVA) gload_one<LA, T>(ga, lda, ra[vec], tid, vec);
+        else gload_one<LB, T>(gb, ldb, rb[vec - NVA], tid, vec - NVA);
+      }
+    };
     for (int kt = 0; kt < nkt; ++kt) {
       const int cur = kt & 1;
       T* const nxt_a = smem + (cur ^ 1) * STAGE;
       T* const nxt_b = nxt_a + ASZ;
-      const int kt2 = min(kt + 2, nkt - 1);
-      const T* const ga = Ab + kt2 * a_kstep;
-      const T* const gb = Bb + kt2 * b_kstep;
+      const int kt2 = min(kt + 2, nkt - 1), kt1 = min(kt + 1, nkt - 1);
+      const T* const ga = Ab + (A_DIR ? kt1 : kt2) * a_kstep;
+      const T* const gb = Bb + (B_DIR ? kt1 : kt2) * b_kstep;
 #pragma unroll
       for (int ks = 0; ks < KS - 1; ++ks) {
         read_ops(cur, ks + 1, am[(ks + 1) & 1], bnv[(ks + 1) & 1]);
 #pragma unroll
         for (int q = 0; q < PER_STEP; ++q) {
           const int slot = ks * PER_STEP + q;
-          if (slot >= SIDE) continue;
-          // side instruction number "slot" of the panel: fp64 alternates store / load vector by vector (the load
-          // refills the registers the store has just read), fp32 issues all stores first, then all loads;
-          // measured at 8192^3: fp64 73.5 against 72.0 TFLOP/s, fp32 141.3 against 139.9 the other way round
-          const bool is_store = ALT ? (slot % 2 == 0) : (slot < NVS);
-          const int vec = ALT ? slot / 2 : (slot < NVS ? slot : slot - NVS);  // 0 .. NVA-1: A, NVA .. NVS-1: B
-          if (is_store) {
-            if (vec < NVA) lds_store_one<LA, T, AK>(nxt_a, ra[vec], tid, vec);
-            else lds_store_one<LB, T, BKM>(nxt_b, rb[vec - NVA], tid, vec - NVA);
-          } else {
-            if (vec < NVA) gload_one<LA, T>(ga, lda, ra[vec], tid, vec);
-            else gload_one<LB, T>(gb, ldb, rb[vec - NVA], tid, vec - NVA);
-          }
+          if (slot < SIDE) side_item(slot, nxt_a, nxt_b, ga, gb);
         }
         mfma_step(am[ks & 1], bnv[ks & 1]);
         // Issue order: the NREADS operand reads of the next step and the PER_STEP side instructions alternate and are
@@ -361,8 +417,10 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
             } else {
               const int slot = ks * PER_STEP + (e < BOTH ? e / 2 : e - NREADS);
               if (slot >= SIDE) continue;
-              const bool is_store = ALT ? (slot % 2 == 0) : (slot < NVS);
-              const int vec = ALT ? slot / 2 : (slot < NVS ? slot : slot - NVS);
+              if (slot < NDIR) { __builtin_amdgcn_sched_group_barrier(PLK_DMA_MASK, 1, 0); continue; }
+              const int r = slot - NDIR;
+              const bool is_store = ALT ? (r % 2 == 0) : (r < NREG);
+              const int vec = REG0 + (ALT ? r / 2 : (r < NREG ? r : r - NREG));
               if (!is_store) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
               else if (vec < NVA) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
               else __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
@@ -371,6 +429,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (A_DIR || B_DIR) __builtin_amdgcn_s_waitcnt(0x0F70);  // the rows requested during this panel are in LDS
       __syncthreads();
       read_ops(cur ^ 1, 0, am[KS & 1], bnv[KS & 1]);
       mfma_step(am[(KS - 1) & 1], bnv[(KS - 1) & 1]);
