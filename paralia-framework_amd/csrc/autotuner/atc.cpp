@@ -233,7 +233,7 @@ paralia::GemmProblem gemm_problem_of(const ProblemDesc& d, long T, int exec_queu
   gp.beta_zero = d.beta_is_zero;
   gp.elem = d.dtype_sz;
   gp.exec_queues = exec_queues;
-  const long full = paralia::gemm_full_block_num(gp);
+  const long full = paralia::gemm_max_block_num(gp);
   gp.pool_blocks = full;
   if (d.pool_budget_bytes > 0) {
     const long long blk = (long long)T * T * d.dtype_sz;
@@ -439,6 +439,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     pipeline.t_d2h_busy = r.t_d2h; pipeline.order_id = order_id;
     pred_t = r.t_total;
     pred_t_pesimistic = r.t_h2d + r.t_exec + r.t_d2h;
+    gp.k_split = 1 << (order_id / paralia::ORDER_K_SPLIT);  // a thin start adds k tiles
     update_sk_num(gp.subkernels());
     distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
   } else if (problem.problem == BLAS2) {

@@ -237,7 +237,7 @@ static paralia::GemmProblem gp_of(long M, long N, long K, long T, int a_remote, 
   gp.M = M; gp.N = N; gp.K = K; gp.T = T;
   gp.a_remote = a_remote; gp.b_remote = b_remote; gp.c_remote = c_remote; gp.beta_zero = beta_zero;
   gp.elem = elem; gp.exec_queues = exec_queues;
-  gp.pool_blocks = pool_blocks > 0 ? pool_blocks : paralia::gemm_full_block_num(gp);
+  gp.pool_blocks = pool_blocks > 0 ? pool_blocks : paralia::gemm_max_block_num(gp);
   return gp;
 }
 

@@ -12,7 +12,8 @@
 namespace paralia {
 
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
-  const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
+  const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();   // p.k_split is the caller's business (build_gemm_plan sets it)
+  order_id %= ORDER_K_SPLIT;
   order_id %= ORDER_MERGE_CHAINS;          // merging launches does not change the order
   order_id %= 40000;                       // nor does the eviction policy
   const bool repeat = order_id >= 20000;  // every panel k-outer, not only the first
@@ -72,7 +73,9 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
   std::vector<int> ids;
   ids.push_back(order_id_of(1, 0));  // the reference's index order; needs the fewest blocks
   if (!(p.a_remote || p.b_remote || p.c_remote)) return ids;
-  const bool limited = p.pool_blocks < gemm_full_block_num(p);
+  GemmProblem unsplit = p;
+  unsplit.k_split = 1;
+  const bool limited = p.pool_blocks < gemm_full_block_num(unsplit);
   static const int widths[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 48, 64};
   static const int probe_widths[] = {2, 4};
   for (int orient = 0; orient < 2; ++orient) {
@@ -119,6 +122,12 @@ long gemm_full_block_num(const GemmProblem& p) {
   return 1 + a + b + 2 * c;
 }
 
+long gemm_max_block_num(const GemmProblem& p) {
+  GemmProblem q = p;
+  q.k_split = 4;
+  return gemm_full_block_num(q);
+}
+
 namespace {
 
 struct Block {
@@ -148,12 +157,16 @@ void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w) {
 
 }  // namespace
 
-GemmPlan build_gemm_plan(const GemmProblem& p, int order_id) {
-  if (p.T <= 0 || p.M <= 0 || p.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
+GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
+  if (p_in.T <= 0 || p_in.M <= 0 || p_in.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
   GemmPlan plan;
-  plan.p = p;
+  plan.p = p_in;
+  plan.p.k_split = 1 << (order_id / ORDER_K_SPLIT);
+  const GemmProblem& p = plan.p;
+  if (order_id >= ORDER_K_SPLIT && p.slabs() == 1) throw std::runtime_error("gemm plan: this problem has no thin start");
   plan.order_id = order_id;
   plan.task_order = gemm_task_order(p, order_id);
+  order_id %= ORDER_K_SPLIT;
   const bool merge = order_id >= ORDER_MERGE_CHAINS;
   order_id %= ORDER_MERGE_CHAINS;
   const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();
@@ -489,7 +502,10 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
         case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
         case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
         case CMD_GEMM:
-          for (int k = c.ki; k < c.ki + c.kn; ++k) dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
+          for (int k = c.ki; k < c.ki + c.kn; ++k) {
+            if (k < p.slabs() && p.slabs() > 1) dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.T) / p.slabs() + st.slab_fixed;
+            else dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
+          }
           if (c.kn > 1) dur = std::max(0.5 * dur, dur - (c.kn - 1) * st.merge_saving * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2);
           break;
         case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
@@ -537,6 +553,23 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
     }
   }
   if (best_id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
+  // the best order also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link
+  GemmProblem unsplit = p;
+  unsplit.k_split = 1;
+  if ((p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit)) {
+    const int base_id = best_id;
+    for (int s = 1; s <= 2; ++s) {
+      try {
+        GemmPlan plan = build_gemm_plan(p, base_id + s * ORDER_K_SPLIT);
+        PipelineResult r = simulate_plan(plan, st);
+        if (plan.n_evictions == 0 && r.t_total < best.t_total * (1.0 - 1e-3)) {
+          best = r;
+          best_id = base_id + s * ORDER_K_SPLIT;
+        }
+      } catch (const std::runtime_error&) {
+      }
+    }
+  }
   if (best_out) *best_out = best;
   return best_id;
 }

@@ -27,12 +27,22 @@ struct GemmProblem {
   int elem = 8;                                              // bytes per element
   int exec_queues = 2;
   long pool_blocks = 0;                                      // device blocks available (>= 3 when anything is remote)
+  // Thin start: the first k tile is cut into k_split slabs of T / k_split (each its own k tile, fetched and multiplied
+  // separately), so the first subkernels can start after a fraction of the first tiles has crossed the link.  Taken
+  // as 1 when it does not apply (K < T, T not divisible, slabs under 16).
+  int k_split = 1;
+  int slabs() const { return (k_split > 1 && K >= T && T % k_split == 0 && T / k_split >= 16) ? k_split : 1; }
   int Mg() const { return (int)((M + T - 1) / T); }
   int Ng() const { return (int)((N + T - 1) / T); }
-  int Kg() const { return K > 0 ? (int)((K + T - 1) / T) : 1; }
+  int Kg() const { return K > 0 ? (int)((K + T - 1) / T) + slabs() - 1 : 1; }
   long tm(int mi) const { return mi == Mg() - 1 ? M - (long)mi * T : T; }
   long tn(int ni) const { return ni == Ng() - 1 ? N - (long)ni * T : T; }
-  long tk(int ki) const { return K <= 0 ? 0 : (ki == Kg() - 1 ? K - (long)ki * T : T); }
+  long k0(int ki) const { const int s = slabs(); return ki < s ? (long)ki * (T / s) : (long)(ki - s + 1) * T; }  // first k of tile ki
+  long tk(int ki) const {
+    if (K <= 0) return 0;
+    if (ki < slabs() && slabs() > 1) return T / slabs();
+    return ki == Kg() - 1 ? K - k0(ki) : T;
+  }
   long subkernels() const { return (long)Mg() * Ng() * Kg(); }
 };
 
@@ -84,6 +94,8 @@ struct GemmPlan {
 // large fp32 tiles, whose workgroups hold a compute unit alone, the prologue and epilogue nothing else overlaps -- at
 // the price of starting only when all its tiles have arrived.  Needs a pool that holds the whole working set.
 constexpr int ORDER_MERGE_CHAINS = 80000;
+// + 160000 * s: thin start (GemmProblem::k_split) with 2^s slabs, s = 1 or 2.
+constexpr int ORDER_K_SPLIT = 160000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
 // probe = true: a handful of representative orders, enough to rank tile sizes before the full search
@@ -95,6 +107,9 @@ GemmPlan build_gemm_plan(const GemmProblem& p, int order_id);
 
 // Block pool size the reference would ask for (dgemm.cpp:23-36,80-82).
 long gemm_full_block_num(const GemmProblem& p);
+// The same with the most slabs a thin start may add: what a caller may offer as pool_blocks at most (the pool is
+// allocated for the blocks the chosen plan uses, not for this number).
+long gemm_max_block_num(const GemmProblem& p);
 
 // Stage costs of a full T x T (x T) tile; edge tiles scale with their area / volume.
 struct StageTimes {
@@ -110,6 +125,8 @@ struct StageTimes {
   // seconds a launch over kn k tiles of a full T x T C tile takes less than kn separate launches, per launch saved
   // (0: merging K chains is not worth considering for this kernel)
   double merge_saving = 0;
+  // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch
+  double slab_fixed = 2e-6;  // measured: 2048 x 2048 x 1024 119.9 us, x 512 61.2 us against 236.7 us for the whole tile
 };
 struct PipelineResult {
   double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource

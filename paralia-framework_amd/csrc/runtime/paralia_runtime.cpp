@@ -303,9 +303,10 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   // what the tile kernel can use to split K when a tile product has too few workgroups (small T): the largest need
   // over the full and the ragged tile extents
   long ws_bytes = 0;
-  for (int e = 0; e < 8; ++e) {
+  for (int e = 0; e < 12; ++e) {
     const long m = (e & 1) ? p.tm(p.Mg() - 1) : std::min<long>(Tt, p.M), n = (e & 2) ? p.tn(p.Ng() - 1) : std::min<long>(Tt, p.N);
-    const long k = p.Kg() > 0 ? ((e & 4) ? p.tk(p.Kg() - 1) : std::min<long>(Tt, p.K)) : 0;
+    // a full k tile, the last one, or a slab of the thin start
+    const long k = p.Kg() > 0 ? (e / 4 == 1 ? p.tk(p.Kg() - 1) : e / 4 == 2 ? p.tk(0) : std::min<long>(Tt, p.K)) : 0;
     ws_bytes = std::max(ws_bytes, pl_gemm_tile_workspace_bytes(m, n, k, (int)sizeof(T)));
   }
   void* ws[MAX_EXEC_QUEUES] = {nullptr};
@@ -325,16 +326,16 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   auto a_tile = [&](int block, int mi, int ki, long* ld) -> T* {
     if (!plan.panels) { *ld = at ? p.tk(ki) : p.tm(mi); return (T*)R.pool.at(block); }
     T* base = (T*)R.pool.at(plan.a_first + (long)mi * Kg);
-    if (at) { *ld = std::max(1L, p.K); return base + (long)ki * Tt; }
+    if (at) { *ld = std::max(1L, p.K); return base + p.k0(ki); }
     *ld = p.tm(mi);
-    return base + (long)ki * Tt * p.tm(mi);
+    return base + p.k0(ki) * p.tm(mi);
   };
   auto b_tile = [&](int block, int ni, int ki, long* ld) -> T* {
     if (!plan.panels) { *ld = bt ? p.tn(ni) : p.tk(ki); return (T*)R.pool.at(block); }
     T* base = (T*)R.pool.at(plan.b_first + (long)ni * Kg);
-    if (!bt) { *ld = std::max(1L, p.K); return base + (long)ki * Tt; }
+    if (!bt) { *ld = std::max(1L, p.K); return base + p.k0(ki); }
     *ld = p.tn(ni);
-    return base + (long)ki * Tt * p.tn(ni);
+    return base + p.k0(ki) * p.tn(ni);
   };
 
   DrainOnError guard(R.res);
@@ -346,7 +347,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
     switch (c.kind) {
       case CMD_FETCH_A: {
         const long rows = at ? p.tk(c.ki) : p.tm(c.mi), cols = at ? p.tm(c.mi) : p.tk(c.ki);
-        const T* src = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda;
+        const T* src = at ? A + p.k0(c.ki) + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + p.k0(c.ki) * lda;
         long ld_dst;
         T* dst = a_tile(c.block, c.mi, c.ki, &ld_dst);
         if (pageable[0]) stager.fetch(dst, src, lda, rows, cols, sizeof(T), s, ld_dst);
@@ -354,7 +355,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       } break;
       case CMD_FETCH_B: {
         const long rows = bt ? p.tn(c.ni) : p.tk(c.ki), cols = bt ? p.tk(c.ki) : p.tn(c.ni);
-        const T* src = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb;
+        const T* src = bt ? B + (long)c.ni * Tt + p.k0(c.ki) * ldb : B + p.k0(c.ki) + (long)c.ni * Tt * ldb;
         long ld_dst;
         T* dst = b_tile(c.block, c.ni, c.ki, &ld_dst);
         if (pageable[1]) stager.fetch(dst, src, ldb, rows, cols, sizeof(T), s, ld_dst);
@@ -373,11 +374,11 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         const T* a;
         long la;
         if (c.a_block >= 0) a = a_tile(c.a_block, c.mi, c.ki, &la);
-        else { a = at ? A + (long)c.ki * Tt + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + (long)c.ki * Tt * lda; la = lda; }
+        else { a = at ? A + p.k0(c.ki) + (long)c.mi * Tt * lda : A + (long)c.mi * Tt + p.k0(c.ki) * lda; la = lda; }
         const T* b;
         long lb;
         if (c.b_block >= 0) b = b_tile(c.b_block, c.ni, c.ki, &lb);
-        else { b = bt ? B + (long)c.ni * Tt + (long)c.ki * Tt * ldb : B + (long)c.ki * Tt + (long)c.ni * Tt * ldb; lb = ldb; }
+        else { b = bt ? B + (long)c.ni * Tt + p.k0(c.ki) * ldb : B + p.k0(c.ki) + (long)c.ni * Tt * ldb; lb = ldb; }
         T* cc;
         long lc;
         if (c.block >= 0) { cc = (T*)R.pool.at(c.block); lc = m; }
@@ -501,7 +502,7 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
       gp.a_remote = key.loc[0] < 0; gp.b_remote = key.loc[1] < 0; gp.c_remote = key.loc[2] < 0;
       gp.beta_zero = key.beta_zero; gp.elem = sizeof(T); gp.exec_queues = atc->exec_queues;
       const long long blk = (long long)atc->T * atc->T * (long long)sizeof(T);
-      gp.pool_blocks = (long)std::min<long long>(gemm_full_block_num(gp), d.pool_budget_bytes / blk);
+      gp.pool_blocks = (long)std::min<long long>(gemm_max_block_num(gp), d.pool_budget_bytes / blk);
       try {
         ne->plan = build_gemm_plan(gp, atc->order_id);
       } catch (const std::runtime_error&) {
@@ -510,8 +511,8 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
         catch (const std::runtime_error& e2) { error("%s\n", e2.what()); }
         atc->order_id = order_id_of(1, 0);
       }
-      atc->update_sk_num(gp.subkernels());
-      atc->distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
+      atc->update_sk_num(ne->plan.p.subkernels());  // the plan's own problem: a thin start adds k tiles
+      atc->distribute_subkernels(ne->plan.p.Mg(), ne->plan.p.Ng(), ne->plan.p.Kg());
     }
     if ((int)R.pmd.size() >= PROBLEM_MD_CACHE) R.pmd.erase(R.pmd.begin());
     R.pmd.push_back(std::move(ne));

@@ -76,3 +76,10 @@ def check_daxpy_against_blas(orc, got, blas_result, alpha, x, y0):
     print("  daxpy vs host BLAS without fused multiply-add: worst %d ulp of the result, %.2f units of the larger operand" % (worst, scaled), flush=True)
     assert scaled <= 1.5
     return worst
+
+
+def k_tiles(info, K, T=None):
+    """k tiles of a streamed GEMM plan: ceil(K / T), plus the extra slabs of a thin start (order id 160000 * s + ...:
+    the first k tile is cut into 2^s slabs that are fetched and multiplied separately)."""
+    T = T or info.T
+    return -(-K // T) + (1 << (info.order_id // 160000)) - 1

@@ -20,7 +20,7 @@ int main(int argc, char** argv) {
     p.a_remote = rng() % 2; p.b_remote = rng() % 2; p.c_remote = rng() % 2;
     p.beta_zero = rng() % 2; p.elem = (rng() % 2) ? 8 : 4; p.exec_queues = 1 + rng() % 4;
     const long full = gemm_full_block_num(p);
-    const long pools[] = {full, full, 3, 4, 5, 8, std::max(3L, full / 2), std::max(3L, full / 3), std::max(3L, full / 8)};
+    const long pools[] = {gemm_max_block_num(p), full, 3, 4, 5, 8, std::max(3L, full / 2), std::max(3L, full / 3), std::max(3L, full / 8)};
     p.pool_blocks = pools[rng() % 9];
     if (p.subkernels() > 6000) continue;
     StageTimes st; st.t_exec = 1e-4; st.h2d_ti = 1e-5; st.h2d_tb = 2e-11; st.d2h_ti = 1e-5; st.d2h_tb = 2e-11; st.t_reduce = 1e-5; st.h2d_sl = 1.01; st.d2h_sl = 1.2;
@@ -32,6 +32,7 @@ int main(int argc, char** argv) {
         const int orient = rng() % 2, w = rng() % 40;
         int id = orient * 10000 + w + ((w > 0 && rng() % 2) ? 20000 : 0) + ((rng() % 2) ? 40000 : 0);
         if (rng() % 3 == 0) id = ORDER_MERGE_CHAINS + orient * 10000 + w;  // merged K chains (refused unless the pool holds everything)
+        if (rng() % 3 == 0) id += ORDER_K_SPLIT * (1 + rng() % 2);  // thin start: first k tile in 2 or 4 slabs (refused when it does not apply)
         GemmPlan plan = build_gemm_plan(p, id);
         PipelineResult r = simulate_plan(plan, st);
         if (!(r.t_total >= 0)) { printf("bad makespan\n"); return 1; }

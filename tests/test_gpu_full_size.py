@@ -9,7 +9,7 @@ import time
 import numpy as np
 import pytest
 
-from gpu_util import Buf, check_daxpy_against_blas
+from gpu_util import Buf, check_daxpy_against_blas, k_tiles
 from oracle_binding import rand_f64
 
 pytestmark = pytest.mark.gpu
@@ -96,7 +96,8 @@ def check_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, locs, T=-1, tol=TOL6
 def test_dgemm_16384_host_operands(pkg, L):
     """dgemm 16384^3, alpha = 1, beta = 0, all operands in pinned host memory, T picked by the autotuner."""
     info = check_gemm(pkg, L, np.float64, "N", "N", 16384, 16384, 16384, 1.0, 0.0, (-1, -1, -1))
-    assert info.subkernel_num == (-(-16384 // info.T)) ** 3
+    g = -(-16384 // info.T)
+    assert info.subkernel_num == g * g * k_tiles(info, 16384)
 
 
 @pytest.mark.timeout(600)

@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from gpu_util import Buf, sync, check_daxpy_against_blas
+from gpu_util import Buf, sync, check_daxpy_against_blas, k_tiles
 from oracle_binding import ptr, rand_f32, rand_f64
 
 pytestmark = pytest.mark.gpu
@@ -66,7 +66,7 @@ def test_dgemm_placements_and_transposes(pkg, L, orc, openblas, locs, ta, tb):
     pad = np.ones(ldc * N, dtype=bool)
     pad.reshape(N, ldc)[:, :M] = False
     assert np.array_equal(got[pad], C0[pad])
-    assert info.T == 128 and info.selected_by == b"user" and info.subkernel_num == 27
+    assert info.T == 128 and info.selected_by == b"user" and info.subkernel_num == 9 * k_tiles(info, K)
     assert np.array_equal(bA.get(), A) and np.array_equal(bB.get(), B)  # inputs are never written
 
 
@@ -121,7 +121,7 @@ def test_dgemm_pool_sweep_picks_different_orders(pkg, L, orc, openblas, blocks, 
     bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, C0, -1)
     info = call_gemm(pkg, L, np.float64, "T", "N", M, N, K, -0.7, beta, bA, K, bB, K, bC, M, T=T, cache_limit=blocks * T * T * 8)
     print("  order", info.order_id, "subkernels", info.subkernel_num, flush=True)
-    assert info.subkernel_num == 6 * 5 * 7
+    assert info.subkernel_num == 6 * 5 * k_tiles(info, K)
     assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 0.7, beta, A, K, M, K, B, K, N, K, C0) < TOL64
 
 
@@ -397,7 +397,7 @@ def test_command_timeline_of_a_streamed_call(pkg, L, orc, openblas):
         pkg.check(L.PARALiA_trace_enable(0), "trace off")
     assert normwise(orc, np.float64, bC.get(), ref, M, N, M, 1.0, 0.0, A, M, K, M, B, K, N, K, C0) < TOL64
     rows = [tuple(buf[7 * i:7 * i + 7]) for i in range(n)]
-    Mg, Ng, Kg = -(-M // T), -(-N // T), -(-K // T)
+    Mg, Ng, Kg = -(-M // T), -(-N // T), k_tiles(info, K)
     kinds = [int(r[0]) for r in rows]
     assert kinds.count(3) == Mg * Ng * Kg == info.subkernel_num
     assert kinds.count(0) == Mg * Kg and kinds.count(1) == Kg * Ng and kinds.count(2) == 0 and kinds.count(5) == Mg * Ng
@@ -443,7 +443,7 @@ def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg,
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
-@pytest.mark.parametrize("order", [80000, 80002, 90003])
+@pytest.mark.parametrize("order", [80000, 80002, 90003, 160002, 320003, 240002, 330000])
 @pytest.mark.parametrize("locs", [(-1, -1, -1), (-1, -1, 0), (-2, -2, -1), (0, -1, -1)])
 def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs, monkeypatch):
     """Order ids of 80000 and above: the k tiles of every A row panel and B column panel lie side by side on the device
@@ -451,9 +451,12 @@ def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs
     ragged tiles in all three dimensions (289 x 353 x 307 at T = 64: 5 x 6 x 5 tiles), every transpose (the panel of
     an operand that is contiguous along k is a K x tile matrix, the other kind a row of dense tiles), operands pinned,
     pageable or already on the device, beta = 0 over NaN and beta != 0 (fetched C, lazy reduce): bit for bit the
-    untiled result, in fp64 and fp32."""
+    untiled result, in fp64 and fp32.  Order ids of 160000 and above add the thin start: the first k tile is cut into 2
+    (160000 +) or 4 (320000 +) slabs that are fetched and multiplied as k tiles of their own (7 or 9 k tiles here), alone
+    or together with merged chains (240002)."""
     monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
-    M, N, K, T = 289, 353, 307 + {80000: 0, 80002: 1, 90003: 2}[order], 64   # a new problem for the metadata cache per order
+    orders = [80000, 80002, 90003, 160002, 320003, 240002, 330000]
+    M, N, K, T = 289, 353, 307 + orders.index(order), 64   # a new problem for the metadata cache per order
     ra, ca = (M, K) if ta == "N" else (K, M)
     rb, cb = (K, N) if tb == "N" else (N, K)
     rng = np.random.default_rng(order + 7 * len(ta + tb))
@@ -467,7 +470,8 @@ def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs
             start = np.full(M * N, np.nan, dtype=dtype) if beta == 0.0 else C0
             bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
             info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 3.0, beta, bA, ra, bB, rb, bC, M, T=T)
-            assert info.order_id == order and info.subkernel_num == 5 * 6 * 5
+            assert info.order_id == order and info.subkernel_num == 5 * 6 * k_tiles(info, K)
+            assert k_tiles(info, K) == 5 + (1 << (order // 160000)) - 1
             assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
 
 

@@ -8,15 +8,27 @@ import pytest
 FETCH_A, FETCH_B, FETCH_C, GEMM, REDUCE, WRITEBACK = range(6)
 BETA_ZERO, BETA_ONE, BETA_USER = 0, 1, 2
 H2D, D2H, EXEC0 = 0, 1, 2
+K_AXIS = object()   # marks a slice request along k, whose tiles need not be uniform
 
 
-def grids(M, N, K, T):
+def kbounds(K, T, slabs=1):
+    """First k of every k tile, and K: tiles of T, the first one cut into `slabs` equal slabs by a thin start (order ids
+    of 160000 and above) when K >= T and the slabs are whole and at least 16 deep."""
+    if K <= 0:
+        return [0, 0]
+    b = list(range(0, K, T)) + [K]
+    if slabs > 1 and K >= T and T % slabs == 0 and T // slabs >= 16:
+        b = [i * (T // slabs) for i in range(slabs)] + b[1:]
+    return b
+
+
+def grids(M, N, K, T, slabs=1):
     c = lambda a: -(-a // T)
-    return c(M), c(N), (c(K) if K > 0 else 1)
+    return c(M), c(N), len(kbounds(K, T, slabs)) - 1
 
 
-def check_plan(rows, stats, M, N, K, T, a_remote, b_remote, c_remote, beta_zero, pool_blocks, nq):
-    Mg, Ng, Kg = grids(M, N, K, T)
+def check_plan(rows, stats, M, N, K, T, a_remote, b_remote, c_remote, beta_zero, pool_blocks, nq, slabs=1):
+    Mg, Ng, Kg = grids(M, N, K, T, slabs)
     gemms = [r for r in rows if r["kind"] == GEMM]
     # every subkernel fired exactly once
     assert sorted((g["mi"], g["ni"], g["ki"]) for g in gemms) == sorted(itertools.product(range(Mg), range(Ng), range(Kg)))
@@ -52,19 +64,19 @@ def check_plan(rows, stats, M, N, K, T, a_remote, b_remote, c_remote, beta_zero,
     assert stats[0] <= pool_blocks
 
 
-def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks):
+def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks, slabs=1):
     """Execute the plan sequentially in plan order with numpy tiles; checks along the way that every block is read
     only while it holds the tile the command expects (i.e. eviction never clobbers live data in plan order)."""
-    Mg, Ng, Kg = grids(M, N, K, T)
-    sl = lambda i, D: slice(i * T, min((i + 1) * T, D))
+    kb = kbounds(K, T, slabs)
+    sl = lambda i, D: slice(kb[i], kb[i + 1]) if D is K_AXIS else slice(i * T, min((i + 1) * T, D))
     blocks = [None] * pool_blocks
     out = C.copy()
     for r in rows:
         k = r["kind"]
         if k == FETCH_A:
-            blocks[r["block"]] = ("A", r["mi"], r["ki"], A[sl(r["mi"], M), sl(r["ki"], K)].copy())
+            blocks[r["block"]] = ("A", r["mi"], r["ki"], A[sl(r["mi"], M), sl(r["ki"], K_AXIS)].copy())
         elif k == FETCH_B:
-            blocks[r["block"]] = ("B", r["ki"], r["ni"], B[sl(r["ki"], K), sl(r["ni"], N)].copy())
+            blocks[r["block"]] = ("B", r["ki"], r["ni"], B[sl(r["ki"], K_AXIS), sl(r["ni"], N)].copy())
         elif k == FETCH_C:
             blocks[r["block"]] = ("S", r["mi"], r["ni"], C[sl(r["mi"], M), sl(r["ni"], N)].copy())
         elif k == GEMM:
@@ -72,12 +84,12 @@ def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks):
                 tag, i, j, a = blocks[r["a_block"]]
                 assert (tag, i, j) == ("A", r["mi"], r["ki"])
             else:
-                a = A[sl(r["mi"], M), sl(r["ki"], K)]
+                a = A[sl(r["mi"], M), sl(r["ki"], K_AXIS)]
             if r["b_block"] >= 0:
                 tag, i, j, b = blocks[r["b_block"]]
                 assert (tag, i, j) == ("B", r["ki"], r["ni"])
             else:
-                b = B[sl(r["ki"], K), sl(r["ni"], N)]
+                b = B[sl(r["ki"], K_AXIS), sl(r["ni"], N)]
             prod = alpha * (a @ b)
             if r["block"] >= 0:
                 if r["beta_mode"] == BETA_ZERO:
@@ -233,7 +245,14 @@ def test_pipeline_simulation(pkg, L):
     args = (16384, 16384, 16384, 2048, 1, 1, 1, 1, 8, 2, 0)
     st = (0.24e-3, 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.0, 0.6e-3 / (2048 * 2048 * 8), 0.02e-3, 1.0, 1.0)
     best = L.PARALiA_gemm_plan_simulate(*args, -1, *st, C.byref(picked), busy)
-    assert abs(busy[1] - 512 * 0.24e-3) < 1e-9 and abs(busy[0] - 128 * 0.6e-3) < 1e-9 and abs(busy[2] - 64 * 0.6e-3) < 1e-9
+    # a thin start (order id 160000 * s + ...: first k tile in 2^s slabs) multiplies the same flops in more launches,
+    # every slab priced at 2 us on top of its share of the tile time
+    slabs = 1 << (picked.value // 160000)
+    assert slabs in (1, 2, 4)
+    assert abs(busy[1] - (512 * 0.24e-3 + (64 * slabs * 2e-6 if slabs > 1 else 0.0))) < 1e-9
+    assert abs(busy[0] - 128 * 0.6e-3) < 1e-9 and abs(busy[2] - 64 * 0.6e-3) < 1e-9
+    unsplit = L.PARALiA_gemm_plan_simulate(*args, picked.value % 160000, *st, None, None)
+    assert best <= unsplit                              # and is only taken when the simulated call gets shorter
     assert best >= busy[1] and best < busy[1] * 1.04
     ref_order = L.PARALiA_gemm_plan_simulate(*args, 10000, *st, None, None)
     k_outer = L.PARALiA_gemm_plan_simulate(*args, 8, *st, None, None)
@@ -390,4 +409,38 @@ def test_merged_chains_need_the_whole_working_set_and_pay_only_with_a_saving(pkg
     assert plain > 0 and abs(merged - plain) <= 1e-9 * plain
     # ... and the search offers merged orders only to a kernel with such a saving (none through this entry point)
     best = L.PARALiA_gemm_plan_simulate(*args, -1, *st, C.byref(picked), busy)
-    assert picked.value < 80000 and best <= plain
+    assert picked.value % 160000 < 80000 and best <= plain
+
+
+@pytest.mark.parametrize("order", [160000, 160002, 170001, 320000, 320003, 330002, 240002, 410001, 180002])
+@pytest.mark.parametrize("locs", [(1, 1, 1), (1, 1, 0), (0, 1, 1), (1, 0, 0)])
+@pytest.mark.parametrize("beta_zero", [0, 1])
+def test_thin_start_plans(pkg, order, locs, beta_zero):
+    """Order ids of 160000 * s and above: the first k tile is cut into 2^s slabs, each a k tile of its own (fetched into
+    its own block, multiplied by its own launch, beta' = 0 on a C tile's first slab only).  Every subkernel of the
+    finer k grid fires once, every tile is fetched once, and the plan -- with merged K chains expanded -- keeps the
+    invariants, replays to the exact result on integers and orders every hazard.  K = 110 with T = 32: 4 k tiles become
+    5 (two slabs of 16); four slabs of 8 are too thin, so ids of 320000 and above are refused here, as they are when K < T."""
+    M, N, K, T = 90, 70, 110, 32
+    a_r, b_r, c_r = locs
+    slabs = 1 << (order // 160000)
+    if slabs == 4:
+        with pytest.raises(pkg.ParaliaError, match="thin start"):
+            pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
+        T = 64                                                   # 2 k tiles become 5: slabs of 16, 16, 16, 16 and 46
+    Mg, Ng, Kg = grids(M, N, K, T, slabs)
+    assert Kg == -(-K // T) + slabs - 1
+    rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
+    flat = expand_merged(rows)
+    full = 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
+    check_plan(flat, stats, M, N, K, T, a_r, b_r, c_r, beta_zero, full, 2, slabs)
+    assert stats[1] == (Mg * Kg if a_r else 0) and stats[2] == (Kg * Ng if b_r else 0) and stats[4] == 0
+    rng = np.random.default_rng(order + beta_zero)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64)
+    B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C = rng.integers(-5, 6, (M, N)).astype(np.float64)
+    alpha, beta = 2.0, (0.0 if beta_zero else 3.0)
+    assert np.array_equal(replay(flat, M, N, K, T, alpha, beta, A, B, C, full, slabs), alpha * (A @ B) + beta * C)
+    check_async_safety(flat)
+    with pytest.raises(pkg.ParaliaError, match="thin start"):
+        pkg.plan_rows(M, N, 20, 32, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)     # K < T: nothing to cut
