@@ -34,10 +34,18 @@
 #ifndef PLK_F64_PAIR
 #define PLK_F64_PAIR 0
 #endif
-// Bit 0: fp64, bit 1: fp32 -- MN-major operand panels whose rows are exactly 1 KiB go global -> LDS without passing
-// registers (see dma_row).
+// Bit 0: fp64, bit 1: fp32 -- operand panels go global -> LDS without passing registers where every panel of the tile
+// can (see dma_row, dma_krows).
 #ifndef PLK_DIRECT
 #define PLK_DIRECT 3
+#endif
+// Bit 0: fp64, bit 1: fp32 -- K-major panels in the swizzled, unpadded LDS layout that an LDS-DMA load can write.
+#ifndef PLK_SWZ
+#define PLK_SWZ 3
+#endif
+// 1: the permuted k order of gemm_kernel's V2 (fp32 256 x 256 tiles with a K-major operand)
+#ifndef PLK_V2
+#define PLK_V2 1
 #endif
 // scheduling class the compiler's instruction-group pass files the LDS-DMA loads under (all DS instructions)
 #ifndef PLK_DMA_MASK
@@ -96,12 +104,23 @@ template <> struct Traits<float> {
 // [mn][k] layout (K-major operands): rows BK + 2 elements apart.  fp32: lane (idx, kk) of an operand read sits in bank
 // ((BK + 2) * idx + kk) mod 64, all distinct; rows are then only 8-byte aligned, so a 16-byte vector goes to LDS as two
 // 8-byte stores (lds_put).  A 16-byte aligned stride costs two-way conflicts on every operand read.
-template <typename T, bool KMAJOR, int EXT, int BK> struct Lds {
+template <typename T, bool KMAJOR, int EXT, int BK, bool SWZ = false> struct Lds {
   using Tr = Traits<T>;
-  static constexpr int S_K = BK + 2, S_MN = EXT + Tr::PAD_MN;
+  // SWZ (K-major only): rows exactly BK elements apart, no padding, and the 16-byte chunks of row mn stored at chunk
+  // position c ^ swz(mn).  That is the layout an LDS-DMA load can write (a wave instruction fills 1 KiB of consecutive
+  // LDS, lane by lane, while every lane picks its own global address), and the XOR keeps the 16-byte operand reads of
+  // eight consecutive rows in eight different bank groups.
+  static constexpr int NC = BK / Tr::VEC;                         // 16-byte chunks per K-major row
+  static constexpr int RPB = 256 / (BK * (int)sizeof(T)) > 0 ? 256 / (BK * (int)sizeof(T)) : 1;  // rows per 256 B (all 64 banks)
+  static constexpr __host__ __device__ __forceinline__ int swz(int mn) { return (mn / RPB) % NC; }
+  static constexpr int S_K = (KMAJOR && SWZ) ? BK : BK + 2, S_MN = EXT + Tr::PAD_MN;
   static constexpr int SIZE = KMAJOR ? EXT * S_K : BK * S_MN;  // elements, padding included
   static constexpr int NV = EXT * BK / Tr::VEC / NTHREADS;     // 16-byte vectors per thread per panel
-  static constexpr __host__ __device__ __forceinline__ int at(int k, int mn) { return KMAJOR ? mn * S_K + k : k * S_MN + mn; }
+  static constexpr bool SPLIT_PUT = KMAJOR && !SWZ && sizeof(T) == 4;  // rows only 8-byte aligned: a vector goes as two halves
+  static constexpr __host__ __device__ __forceinline__ int at(int k, int mn) {
+    if (KMAJOR && SWZ) return mn * S_K + (((k / Tr::VEC) ^ swz(mn)) * Tr::VEC) + k % Tr::VEC;
+    return KMAJOR ? mn * S_K + k : k * S_MN + mn;
+  }
   // Vector i of thread tid: "c" runs along the memory-contiguous dimension (mn for MN-major operands, k for K-major
   // ones), "s" along the leading-dimension stride.
   static constexpr int CVECS = (KMAJOR ? BK : EXT) / Tr::VEC;  // vectors per contiguous run
@@ -113,7 +132,7 @@ template <typename T, bool KMAJOR, int EXT, int BK> struct Lds {
   static __device__ __forceinline__ int slot_offset(int tid, int i) {
     int c, s;
     coords(tid, i, c, s);
-    return KMAJOR ? at(c, s) : at(s, c);  // the contiguous run is also contiguous in LDS for both layouts
+    return KMAJOR ? at(c, s) : at(s, c);  // a 16-byte vector stays together in LDS in every layout
   }
 };
 
@@ -156,11 +175,11 @@ __device__ __forceinline__ void gload_one(const T* __restrict__ base, long ld, t
 }
 typedef float fvec2 __attribute__((ext_vector_type(2)));
 
-// One 16-byte vector into LDS; PUTS<T, KMAJOR> is the number of store instructions that takes.
-template <typename T, bool KMAJOR> constexpr int PUTS = (KMAJOR && sizeof(T) == 4) ? 2 : 1;
-template <typename T, bool KMAJOR>
+// One 16-byte vector into LDS; PUTS<L> is the number of store instructions that takes.
+template <typename L> constexpr int PUTS = L::SPLIT_PUT ? 2 : 1;
+template <typename L, typename T>
 __device__ __forceinline__ void lds_put(T* __restrict__ p, const typename Traits<T>::vec_t& v) {
-  if constexpr (KMAJOR && sizeof(T) == 4) {
+  if constexpr (L::SPLIT_PUT) {
     fvec2 lo, hi;
     lo.x = v[0]; lo.y = v[1]; hi.x = v[2]; hi.y = v[3];
     *reinterpret_cast<fvec2*>(p) = lo;
@@ -170,15 +189,15 @@ __device__ __forceinline__ void lds_put(T* __restrict__ p, const typename Traits
   }
 }
 
-template <typename L, typename T, bool KMAJOR>
+template <typename L, typename T>
 __device__ __forceinline__ void lds_store_one(T* __restrict__ xs, const typename Traits<T>::vec_t& reg, int tid, int i) {
-  lds_put<T, KMAJOR>(xs + L::slot_offset(tid, i), reg);
+  lds_put<L, T>(xs + L::slot_offset(tid, i), reg);
 }
 
-template <typename L, typename T, bool KMAJOR>
+template <typename L, typename T>
 __device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Traits<T>::vec_t (&regs)[L::NV], int tid) {
 #pragma unroll
-  for (int i = 0; i < L::NV; ++i) lds_put<T, KMAJOR>(xs + L::slot_offset(tid, i), regs[i]);
+  for (int i = 0; i < L::NV; ++i) lds_put<L, T>(xs + L::slot_offset(tid, i), regs[i]);
 }
 
 // Row `row` of an MN-major panel straight from global memory into LDS (global_load_lds_dwordx4): the 64 lanes of a wave
@@ -190,6 +209,20 @@ __device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs,
 #if defined(__HIP_DEVICE_COMPILE__)
   const T* p = g + (16 / (int)sizeof(T)) * lane + (long)row * ld;
   __builtin_amdgcn_global_load_lds(p, xs + row * s_mn, 16, 0, 0);
+#endif
+}
+
+// Rows of a K-major panel (each BK elements = NC 16-byte chunks) straight into the swizzled layout of Lds<.., SWZ>: wave
+// instruction number `inst` of the panel fills 64 / NC consecutive rows; lane l fills chunk position l % NC of row
+// l / NC with the global chunk (l % NC) ^ swz(row).
+template <typename L, typename T>
+__device__ __forceinline__ void dma_krows(const T* __restrict__ g, long ld, T* xs, int inst, int lane) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int NC = L::NC, RPI = 64 / NC;
+  const int row = inst * RPI + lane / NC;
+  const int gc = (lane % NC) ^ L::swz(row);
+  const T* p = g + (long)row * ld + gc * Traits<T>::VEC;
+  __builtin_amdgcn_global_load_lds(p, xs + inst * RPI * L::S_K, 16, 0, 0);
 #endif
 }
 
@@ -221,8 +254,22 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
   using acc_t = typename Tr::acc_t;
-  using LA = Lds<T, AK, BM, BK>;
-  using LB = Lds<T, BKM, BN, BK>;
+  // SWZL (the tiles whose MN-major panel rows are exactly 1 KiB: fp64 128 x 128, fp32 256 x 256): K-major panels in the
+  // swizzled, unpadded layout (Lds<.., SWZ>), so every panel, K-major or MN-major, can be loaded global -> LDS directly
+  // and all four transposes run without staging registers and LDS stores.
+  // V2 (fp32 256 x 256 with a K-major operand) adds a k order.  Which k of a panel an MFMA step multiplies is free as
+  // long as A and B agree.  Inside every 16-deep group of k, lane group kk (k index of the MFMA) takes the SPG
+  // consecutive values kk * SPG .. kk * SPG + SPG - 1, one per step, instead of every KSTEP-th value.  A K-major
+  // operand then has the values of KV = VEC = 4 consecutive steps side by side in LDS: ONE 16-byte read per block
+  // serves four steps, where the plain order needs a read per block and two steps.  MN-major operands do not care which
+  // row a step reads.  (For fp64 the same order was slower than the plain one: 71.3 against 73.0 TFLOP/s NN.)
+  // fp64: only with a K-major A (TN 73.2 -> 74.0, TT 72.6 -> 73.6 TFLOP/s at 8192^3); NN measured the same either way
+  // (73.55 / 73.45) and keeps the register path.
+  constexpr bool SWZL = ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
+                        ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16 && AK) || (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
+  constexpr bool V2 = PLK_V2 && SWZL && sizeof(T) == 4 && (AK || BKM);
+  using LA = Lds<T, AK, BM, BK, SWZL>;
+  using LB = Lds<T, BKM, BN, BK, SWZL>;
   constexpr int BLK = Tr::BLK, WM = BM / 2, WN = BN / 2, NBM = WM / BLK, NBN = WN / BLK;
   if (kchunk > 0) {
     // split K: the workgroups of grid row y multiply k in [y * kchunk, (y + 1) * kchunk) and leave their plain partial
@@ -235,7 +282,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   }
   constexpr int ASZ = LA::SIZE, BSZ = LB::SIZE;
 
-  __shared__ __attribute__((aligned(16))) T smem[2 * (ASZ + BSZ)];
+  __shared__ __attribute__((aligned(32))) T smem[2 * (ASZ + BSZ)];
   constexpr int STAGE = ASZ + BSZ;  // buffer b holds A at smem + b*STAGE and B right behind it
 
   const int tid = threadIdx.x;
@@ -287,21 +334,78 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // 1 per 2 about half of that).  The epilogue maps the accumulators back with the same rule.
   constexpr bool PAIRED = sizeof(T) == 4 || PLK_F64_PAIR;
   constexpr bool A_PAIR = PAIRED && !AK, B_PAIR = PAIRED && !BKM;
-  const T* const lane_a = smem + LA::at(kk, wm + (A_PAIR ? NBM * idx : idx));         // this lane's A operand of k-step 0, block 0
-  const T* const lane_b = smem + ASZ + LB::at(kk, wn + (B_PAIR ? NBN * idx : idx));  // this lane's B operand
+  constexpr int G = 16, SPG = G / Tr::KSTEP;   // V2: k group depth, MFMA steps per group
+  // this lane's A / B operand of k-step 0, block 0 (V2: of the first step of a group)
+  const T* const lane_a = smem + LA::at(V2 ? kk * SPG : kk, wm + (A_PAIR ? NBM * idx : idx));
+  const T* const lane_b = smem + ASZ + LB::at(V2 ? kk * SPG : kk, wn + (B_PAIR ? NBN * idx : idx));
   constexpr int A_KS = LA::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : LA::at(0, BLK);    // strides per k-step / per block
   constexpr int B_KS = LB::at(Tr::KSTEP, 0), B_BL = B_PAIR ? 1 : LB::at(0, BLK);
-  constexpr int NREADS = (A_PAIR ? 1 : NBM) + (B_PAIR ? 1 : NBN);  // LDS read instructions per k-step
-  constexpr int KV = Tr::KV;
+  constexpr int KV = V2 ? SPG / 2 : Tr::KV;    // V2: == VEC, the steps one 16-byte read of a K-major operand serves
+  static_assert(!V2 || KV == Tr::VEC, "a 16-byte chunk of a K-major row must hold exactly KV steps");
   constexpr int KS = BK / (Tr::KSTEP * KV);  // operand refreshes ("steps") per panel
+  // LDS read instructions per refresh
+  constexpr int RD_A = V2 ? (AK ? NBM : KV * (NBM * (int)sizeof(T) > 16 ? 2 : 1)) : (A_PAIR ? 1 : NBM);
+  constexpr int RD_B = V2 ? (BKM ? NBN : KV * (NBN * (int)sizeof(T) > 16 ? 2 : 1)) : (B_PAIR ? 1 : NBN);
+  constexpr int NREADS = RD_A + RD_B;
+  // K-major operand in the swizzled layout: where this lane finds its values in its row of block 0 (the same place in
+  // every block: a block is a multiple of the swizzle period).  V2: the chunk of refresh (g, h) -- group g of the panel,
+  // half h of the lane's SPG steps -- is chunk g * (16 / VEC) + 2 kk + h, moved by the row's swizzle.  Plain order: the
+  // value of k-step t is element t * KSTEP + kk of the row, its chunk moved likewise.
+  constexpr int NKP = !SWZL ? 1 : V2 ? (BK / G) * 2 : BK / Tr::KSTEP;
+  const T* a_kp[NKP];
+  const T* b_kp[NKP];
+#pragma unroll
+  for (int q = 0; q < NKP; ++q) {
+    const int k_q = V2 ? ((q / 2) * (G / Tr::VEC) + 2 * kk + q % 2) * Tr::VEC : q * Tr::KSTEP + kk;
+    a_kp[q] = smem + LA::at(k_q, wm + idx);
+    b_kp[q] = smem + ASZ + LB::at(k_q, wn + idx);
+  }
 
   auto read_ops = [&](int buf, int ks, T (&am)[KV][NBM], T (&bnv)[KV][NBN]) {
+    if constexpr (V2) {
+      const int g = (ks * KV) / SPG, h = ((ks * KV) % SPG) / KV;
+      if constexpr (AK) {
+#pragma unroll
+        for (int j = 0; j < NBM; ++j) {
+          const vec_t x = *reinterpret_cast<const vec_t*>(a_kp[2 * g + h] + buf * STAGE + j * BLK * LA::S_K);
+#pragma unroll
+          for (int v = 0; v < KV; ++v) am[v][j] = x[v];
+        }
+      } else {
+        typedef T opv_t __attribute__((ext_vector_type(NBM)));
+#pragma unroll
+        for (int v = 0; v < KV; ++v) {
+          const opv_t x = *reinterpret_cast<const opv_t*>(lane_a + buf * STAGE + (g * G + h * KV + v) * LA::S_MN);
+#pragma unroll
+          for (int j = 0; j < NBM; ++j) am[v][j] = x[j];
+        }
+      }
+      if constexpr (BKM) {
+#pragma unroll
+        for (int i = 0; i < NBN; ++i) {
+          const vec_t x = *reinterpret_cast<const vec_t*>(b_kp[2 * g + h] + buf * STAGE + i * BLK * LB::S_K);
+#pragma unroll
+          for (int v = 0; v < KV; ++v) bnv[v][i] = x[v];
+        }
+      } else {
+        typedef T opv_t __attribute__((ext_vector_type(NBN)));
+#pragma unroll
+        for (int v = 0; v < KV; ++v) {
+          const opv_t x = *reinterpret_cast<const opv_t*>(lane_b + buf * STAGE + (g * G + h * KV + v) * LB::S_MN);
+#pragma unroll
+          for (int i = 0; i < NBN; ++i) bnv[v][i] = x[i];
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
 #pragma unroll
-      for (int j = 0; j < NBM; ++j) am[v][j] = lane_a[buf * STAGE + (ks * KV + v) * A_KS + j * A_BL];
+      for (int j = 0; j < NBM; ++j)
+        am[v][j] = (SWZL && AK) ? a_kp[ks * KV + v][buf * STAGE + j * BLK * LA::S_K] : lane_a[buf * STAGE + (ks * KV + v) * A_KS + j * A_BL];
 #pragma unroll
-      for (int i = 0; i < NBN; ++i) bnv[v][i] = lane_b[buf * STAGE + (ks * KV + v) * B_KS + i * B_BL];
+      for (int i = 0; i < NBN; ++i)
+        bnv[v][i] = (SWZL && BKM) ? b_kp[ks * KV + v][buf * STAGE + i * BLK * LB::S_K] : lane_b[buf * STAGE + (ks * KV + v) * B_KS + i * B_BL];
     }
   };
   auto mfma_step = [&](const T (&am)[KV][NBM], const T (&bnv)[KV][NBN]) {
@@ -329,24 +433,30 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     // loaded two panels ahead as before.
     constexpr bool DIR_T = ((PLK_DIRECT >> (sizeof(T) == 4 ? 1 : 0)) & 1) != 0;
     // only when both operands qualify: with one operand direct and one staged the wait in front of the barrier also
-    // covers the staged operand's newer loads (fp32 256 x 128 NN: 143.8 -> 137.4 TFLOP/s)
-    constexpr bool A_DIR = DIR_T && !AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024;
+    // covers the staged operand's newer loads (fp32 256 x 128 NN: 143.8 -> 137.4 TFLOP/s).  SWZL: every operand does.
+    constexpr bool A_DIR = DIR_T && (SWZL || (!AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024));
     constexpr bool B_DIR = A_DIR;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     if constexpr (A_DIR) {
 #pragma unroll
-      for (int i = 0; i < NVA; ++i) dma_row<T>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
+      for (int i = 0; i < NVA; ++i) {
+        if constexpr (AK) dma_krows<LA, T>(Ab, lda, smem, wave_u + 4 * i, lane);
+        else dma_row<T>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
+      }
     } else {
       gload<LA, T, false>(Ab, lda, 0, 0, true, ra, tid);
-      lds_store<LA, T, AK>(smem, ra, tid);
+      lds_store<LA, T>(smem, ra, tid);
       gload<LA, T, false>(Ab + min(1, nkt - 1) * a_kstep, lda, 0, 0, true, ra, tid);
     }
     if constexpr (B_DIR) {
 #pragma unroll
-      for (int i = 0; i < NVB; ++i) dma_row<T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
+      for (int i = 0; i < NVB; ++i) {
+        if constexpr (BKM) dma_krows<LB, T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane);
+        else dma_row<T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
+      }
     } else {
       gload<LB, T, false>(Bb, ldb, 0, 0, true, rb, tid);
-      lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
+      lds_store<LB, T>(smem + ASZ, rb, tid);
       gload<LB, T, false>(Bb + min(1, nkt - 1) * b_kstep, ldb, 0, 0, true, rb, tid);
     }
     if constexpr (A_DIR || B_DIR) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the requested rows are in LDS
@@ -365,8 +475,13 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     auto side_item = [&](int slot, T* nxt_a, T* nxt_b, const T* ga, const T* gb) {
       if (slot < NDIR) {
         const int vec = (A_DIR ? 0 : NVA) + slot;  // direct rows: A's first when both are direct
-        if (vec < NVA) dma_row<T>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
-        else dma_row<T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
+        if (vec < NVA) {
+          if constexpr (AK) dma_krows<LA, T>(ga, lda, nxt_a, wave_u + 4 * vec, lane);
+          else dma_row<T>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
+        } else {
+          if constexpr (BKM) dma_krows<LB, T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane);
+          else dma_row<T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
+        }
         return;
       }
       // staged side instruction number r of the panel: fp64 alternates store / load vector by vector (the load
@@ -376,8 +491,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
       const bool is_store = ALT ? (r % 2 == 0) : (r < NREG);
       const int vec = REG0 + (ALT ? r / 2 : (r < NREG ? r : r - NREG));  // 0 .. NVA-1: A, NVA .. : B
       if (is_store) {
-        if (vec < NVA) lds_store_one<LA, T, AK>(nxt_a, ra[vec], tid, vec);
-        else lds_store_one<LB, T, BKM>(nxt_b, rb[vec - NVA], tid, vec - NVA);
+        if (vec < NVA) lds_store_one<LA, T>(nxt_a, ra[vec], tid, vec);
+        else lds_store_one<LB, T>(nxt_b, rb[vec - NVA], tid, vec - NVA);
       } else {
         if (vec < NVA) gload_one<LA, T>(ga, lda, ra[vec], tid, vec);
         else gload_one<LB, T>(gb, ldb, rb[vec - NVA], tid, vec - NVA);
@@ -422,8 +537,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
               const bool is_store = ALT ? (r % 2 == 0) : (r < NREG);
               const int vec = REG0 + (ALT ? r / 2 : (r < NREG ? r : r - NREG));
               if (!is_store) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-              else if (vec < NVA) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, AK>, 0);
-              else __builtin_amdgcn_sched_group_barrier(0x200, PUTS<T, BKM>, 0);
+              else if (vec < NVA) __builtin_amdgcn_sched_group_barrier(0x200, PUTS<LA>, 0);
+              else __builtin_amdgcn_sched_group_barrier(0x200, PUTS<LB>, 0);
             }
           }
         }
@@ -446,8 +561,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     // General loop: edge workgroups, ragged K, unaligned operands.  Same double buffering, loads guarded.
     if (nkt > 0) {
       fetch(0);
-      lds_store<LA, T, AK>(smem, ra, tid);
-      lds_store<LB, T, BKM>(smem + ASZ, rb, tid);
+      lds_store<LA, T>(smem, ra, tid);
+      lds_store<LB, T>(smem + ASZ, rb, tid);
     }
     __syncthreads();
     for (int kt = 0; kt < nkt; ++kt) {
@@ -460,8 +575,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         mfma_step(am, bnv);
       }
       if (kt + 1 < nkt) {
-        lds_store<LA, T, AK>(smem + (cur ^ 1) * STAGE, ra, tid);
-        lds_store<LB, T, BKM>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
+        lds_store<LA, T>(smem + (cur ^ 1) * STAGE, ra, tid);
+        lds_store<LB, T>(smem + (cur ^ 1) * STAGE + ASZ, rb, tid);
       }
       __syncthreads();
     }
@@ -616,29 +731,36 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   int splits = workspace ? pick_splits<T>(M, N, K, &kchunk) : 1;
   if (splits > 1 && (long)splits * M * N * (long)sizeof(T) > workspace_bytes) splits = 1, kchunk = 0;
   // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
-  //  * 256 x 256 x 32 ("large", NT and TN): its inner loop runs 4 - 6 % faster per k (half the operand reads and three
-  //    quarters of the global loads per MFMA), but a CU holds one such workgroup at a time, so nothing overlaps its
-  //    prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K / (1 + g), a round of 512
-  //    small ones 12 us + 0.1207 us * K, with g and f (beta == 0 / beta != 0) fitted per variant to 8192^3 and 16384^3
-  //    runs.  It pays from K of about 2000 (NT) / 6000 (TN) on, for tile counts that fill whole rounds.
-  //  * 256 x 128 x 16 ("wide", NN): still two workgroups per CU, 3 % faster per k (measured with several streams in
-  //    flight: +2.9 % at 4096^3, +4.7 % at 8192^3; for NN the large tile gains less, for NT the wide one loses 1 %).
-  // TT keeps the small tile (K-major A costs the bigger tiles one LDS read per block: 137 against 138 TFLOP/s), and
-  // so does split K.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs) measured 70.7
-  // against 73.4 TFLOP/s.
+  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 7 - 9 % faster per k (all panels global -> LDS
+  //    directly, a 16-byte operand read per block and four k-steps), but a CU holds one such workgroup at a time, so
+  //    nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K / (1 + g),
+  //    with g and f (beta == 0 / beta != 0) fitted per transpose to single-stream runs at M = N = 8192, K = 512 .. 8192
+  //    (148 - 150 TFLOP/s at K = 8192, beta = 0, for all four).
+  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 4 % faster per k than the small tile with a
+  //    small fixed cost: (5 | 10.6) us + 2 * 0.1207 us * K / 1.042 per round of 512; ahead of the large tile for
+  //    beta != 0 up to K of about 5000.
+  //  * a round of 512 small tiles: 6 us + 0.1207 us * K.
+  // Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs)
+  // measured 70.7 against 73.4 TFLOP/s.
   struct LargeTileFit { double g, f0, f1; };
-  const LargeTileFit fit = at ? LargeTileFit{0.045, 77.0, 114.0} : LargeTileFit{0.042, 23.0, 34.0};
+  const LargeTileFit fit = an ? (bnn ? LargeTileFit{0.072, 10.0, 46.0} : LargeTileFit{0.088, 10.0, 44.0})
+                              : (bnn ? LargeTileFit{0.073, 9.0, 52.0} : LargeTileFit{0.076, 10.0, 55.0});
   auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
   const double k_us = 0.1207 * (double)K;
-  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (12.0 + k_us);
+  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (6.0 + k_us);
   const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * k_us / (1.0 + fit.g));
-  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (12.0 + 2.0 * k_us / 1.026);
-  const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");  // "0": never, "1": wherever it exists, unset: the model
-  const bool pinned = pin && *pin, other = sizeof(T) == 4 && splits == 1 && !(at && bt) && (!pinned || atoi(pin) != 0);
+  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * ((beta == T(0) ? 5.0 : 10.6) + 2.0 * k_us / 1.042);
+  // PARALIA_GEMM_LARGE_TILE: "0" small tiles only, "1" the large tile for every call, "2" the wide tile wherever it
+  // exists (NN), unset: the model
+  const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");
+  const int pinv = (pin && *pin) ? atoi(pin) : -1;
+  const bool other = sizeof(T) == 4 && splits == 1 && pinv != 0;
   // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
   auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
-  const bool wide = other && an && bnn && (pinned || (wide_us < small_us && fills(tiles_of(256, 128), 512)));
-  const bool big = other && !(an && bnn) && (pinned || (large_us < small_us && fills(tiles_of(256, 256), 256)));
+  const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
+  const bool big_ok = other && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
+  const bool big = big_ok && (pinv == 1 || (large_us < small_us && (!wide_ok || large_us <= wide_us)));
+  const bool wide = !big && wide_ok && (pinv == 2 || wide_us < small_us);
   const int TM_RT = big || wide ? 256 : 128, TN_RT = big ? 256 : 128;
   const int gm = (int)((M + TM_RT - 1) / TM_RT), gn = (int)((N + TN_RT - 1) / TN_RT);
   if ((long)gm * gn > INT32_MAX) return 2;

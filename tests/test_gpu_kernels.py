@@ -21,8 +21,9 @@ _LARGE_TILE_BITS = {}
 
 @contextlib.contextmanager
 def large_tile(pin):
-    """PARALIA_GEMM_LARGE_TILE for the calls inside: "1" forces the 256 x 256 fp32 tile, "0" forbids it, None leaves the
-    choice to the kernel's cost model.  The library reads the variable at every launch."""
+    """PARALIA_GEMM_LARGE_TILE for the calls inside: "1" forces the 256 x 256 fp32 tile (every transpose), "2" the
+    256 x 128 one where it exists (NN), "0" forbids both, None leaves the choice to the kernel's cost model.  The library
+    reads the variable at every launch."""
     old = os.environ.pop("PARALIA_GEMM_LARGE_TILE", None)
     if pin is not None:
         os.environ["PARALIA_GEMM_LARGE_TILE"] = pin
@@ -151,11 +152,14 @@ def test_sgemm_tile_exact_and_unaligned(pkg, L, orc):
     assert np.array_equal(got, ref)
 
 
-@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
-@pytest.mark.parametrize("dims,off", [((4096, 4096, 64), 0), ((4000, 4100, 77), 0), ((8192 + 256, 2048, 33), 0), ((4096, 4096, 40), 1)])
-def test_sgemm_large_tile_exact_on_integers(pkg, L, openblas, ta, tb, dims, off):
-    """The 256 x 256 macro tile of fp32 (TT keeps the small one), forced for shapes the cost model would give to the
-    small tile: interior tiles, partial tiles on both edges, k not a multiple of the panel depth, and operands one
+@pytest.mark.parametrize("ta,tb,pin", [("N", "N", "1"), ("N", "T", "1"), ("T", "N", "1"), ("T", "T", "1"), ("N", "N", "2")])
+@pytest.mark.parametrize("dims,off", [((4096, 4096, 64), 0), ((4000, 4100, 77), 0), ((8192 + 256, 2048, 33), 0), ((4096, 4096, 40), 1),
+                                      ((2048, 2304, 1056), 0)])
+def test_sgemm_large_tile_exact_on_integers(pkg, L, openblas, ta, tb, dims, off, pin):
+    """The 256 x 256 macro tile of fp32 (pin "1": all panels loaded straight into LDS, K-major ones in the swizzled layout
+    and read in the permuted k order) and the 256 x 128 one (pin "2", NN), forced for shapes the cost model would give to
+    the small tile: interior tiles, partial tiles on both edges, k not a multiple of the panel depth (the guarded loop
+    writes the same LDS layouts through registers), a long k with whole panels (the pipelined loop), and operands one
     element off the 16-byte alignment (the element-load path).  Small-integer data, so OpenBLAS gives the exact bits."""
     M, N, K = dims
     rng = np.random.default_rng(11)
@@ -165,20 +169,21 @@ def test_sgemm_large_tile_exact_on_integers(pkg, L, openblas, ta, tb, dims, off)
     A = rng.integers(-4, 5, lda * ca + off).astype(np.float32)
     B = rng.integers(-4, 5, ldb * cb + off).astype(np.float32)
     C0 = rng.integers(-4, 5, ldc * N + off).astype(np.float32)
-    with large_tile("1"):
+    with large_tile(pin):
         got = run_gemm(pkg, L, np.float32, ta, tb, M, N, K, 2.0, -1.0, A, lda, B, ldb, C0, ldc, off, off, off)
     ref = C0.copy()
     assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A[off:]), lda, ptr(B[off:]), ldb, -1.0, ptr(ref[off:]), ldc) == 0
     assert np.array_equal(got, ref)  # includes the padding between columns, which both leave alone
 
 
-@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N")])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
 @pytest.mark.parametrize("beta", [0.5, 0.0])
-@pytest.mark.parametrize("pin", ["1", "0", None])
+@pytest.mark.parametrize("pin", ["1", "2", "0", None])
 def test_sgemm_large_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, pin, beta):
-    """Random data at 4096 x 4096 x 8192, where the kernel's cost model picks the large tile by itself (pin None) for
-    beta = 0 and for NT also with beta != 0.  The summation order over k does not depend on the tile, so the three
-    runs give the same bits."""
+    """Random data at 4096 x 4096 x 8192, where the kernel's cost model picks the large tile by itself (pin None).  Every
+    tile is held to OpenBLAS within the fp32 tolerance.  Tiles that multiply k in the same order give the same bits:
+    for NT (no K-major operand) all of them; with a K-major operand the large tile walks each 16-deep group of k in
+    its own order, so there only runs on the same tile are compared."""
     M, N, K = 4096, 4096, 8192
     ra, ca = (M, K) if ta == "N" else (K, M)
     rb, cb = (K, N) if tb == "N" else (N, K)
@@ -189,7 +194,8 @@ def test_sgemm_large_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, pin, beta):
     assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 1.5, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M) == 0
     d = 1.5 * orc.orc_fro_norm_f32(ptr(A), ra, ca, ra) * orc.orc_fro_norm_f32(ptr(B), rb, cb, rb) + beta * orc.orc_fro_norm_f32(ptr(C0), M, N, M)
     assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
-    key = (ta, tb, beta)
+    same_order = "all" if (ta, tb) == ("N", "T") else ("large" if pin in ("1", None) else "small")
+    key = (ta, tb, beta, same_order)
     if key in _LARGE_TILE_BITS:
         assert np.array_equal(got, _LARGE_TILE_BITS[key])
     _LARGE_TILE_BITS[key] = got
