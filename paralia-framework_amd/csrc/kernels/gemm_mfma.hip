@@ -247,7 +247,10 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 // for two workgroups per CU (two waves per SIMD that fill each other's gaps); larger ones run one workgroup per CU with
 // the whole register file and fewer operand reads and global loads per MFMA.
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
-template <typename T, bool AK, bool BKM, int BM, int BN, int BK>
+// DIR = false: every panel through registers, plain layouts (what the launcher picks for short k: a panel requested
+// straight into LDS is asked for one panel ahead, one staged through registers two, and on the cold first panels of a
+// short k chunk that is the difference: fp64 1024^3 split four ways ran 7 - 12 % slower with direct panels).
+template <typename T, bool AK, bool BKM, int BM, int BN, int BK, bool DIR = true>
 __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 8 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
                                                           long ldc, int gm, int gn, int vecA, int vecB, int vecC, int kchunk) {
@@ -265,7 +268,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // row a step reads.  (For fp64 the same order was slower than the plain one: 71.3 against 73.0 TFLOP/s NN.)
   // fp64: only with a K-major A (TN 73.2 -> 74.0, TT 72.6 -> 73.6 TFLOP/s at 8192^3); NN measured the same either way
   // (73.55 / 73.45) and keeps the register path.
-  constexpr bool SWZL = ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
+  constexpr bool SWZL = DIR && ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
                         ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16 && AK) || (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
   constexpr bool V2 = PLK_V2 && SWZL && sizeof(T) == 4 && (AK || BKM);
   using LA = Lds<T, AK, BM, BK, SWZL>;
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     // MN-major operands whose panel rows are 1 KiB skip the registers (dma_row): panel kt+1 is requested while panel kt
     // is multiplied and must have landed (vmcnt) before the panel's barrier; operands staged through registers are
     // loaded two panels ahead as before.
-    constexpr bool DIR_T = ((PLK_DIRECT >> (sizeof(T) == 4 ? 1 : 0)) & 1) != 0;
+    constexpr bool DIR_T = DIR && ((PLK_DIRECT >> (sizeof(T) == 4 ? 1 : 0)) & 1) != 0;
     // only when both operands qualify: with one operand direct and one staged the wait in front of the barrier also
     // covers the staged operand's newer loads (fp32 256 x 128 NN: 143.8 -> 137.4 TFLOP/s).  SWZL: every operand does.
     constexpr bool A_DIR = DIR_T && (SWZL || (!AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024));
@@ -774,16 +777,21 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   T* const k_C = splits > 1 ? workspace : C;
   const long k_ldc = splits > 1 ? M : ldc;
   constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
-#define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK)                                                                            \
-  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
+  // fp64 with direct panels (every transpose but NN) only where the k extent of a workgroup is long
+  const bool stage = sizeof(T) == 8 && (splits > 1 ? kchunk : K) < 1536;
+#define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK, DIRF)                                                                            \
+  hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK, DIRF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
                      A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)
-#define PLK_LAUNCH(AKF, BKF)                                                  \
-  do {                                                                        \
-    if constexpr (sizeof(T) == 4) {                                           \
-      if (big) { PLK_LAUNCH_T(AKF, BKF, 256, 256, PLK_F32_BIG_BK); break; }   \
-      if (wide) { PLK_LAUNCH_T(AKF, BKF, 256, 128, PLK_F32_BK); break; }      \
-    }                                                                         \
-    PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL);                               \
+#define PLK_LAUNCH(AKF, BKF)                                                        \
+  do {                                                                              \
+    if constexpr (sizeof(T) == 4) {                                                 \
+      if (big) { PLK_LAUNCH_T(AKF, BKF, 256, 256, PLK_F32_BIG_BK, true); break; }   \
+      if (wide) { PLK_LAUNCH_T(AKF, BKF, 256, 128, PLK_F32_BK, true); break; }      \
+    }                                                                               \
+    if constexpr (sizeof(T) == 8 && !(!AKF && BKF)) {                               \
+      if (stage) { PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, false); break; }      \
+    }                                                                               \
+    PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, true);                               \
   } while (0)
   // op(A) K-major <=> TransA == 'T'; op(B) K-major <=> TransB == 'N'
   if (an && bnn) PLK_LAUNCH(false, true);
