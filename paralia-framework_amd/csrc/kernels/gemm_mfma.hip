@@ -204,11 +204,13 @@ __device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Tra
 // fetch 16 bytes each and the hardware puts lane l's at the wave's LDS base + 16 l, so one instruction moves one 1 KiB
 // row (256 floats or 128 doubles) and neither staging registers nor LDS store instructions are spent on it.  The LDS
 // base is wave-uniform, which is why the row stride of the padded layout can stay.
-template <typename T>
-__device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs, int row, int lane, int s_mn) {
+template <typename T, int EXT>
+__device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs, int inst, int lane, int s_mn) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  const T* p = g + (16 / (int)sizeof(T)) * lane + (long)row * ld;
-  __builtin_amdgcn_global_load_lds(p, xs + row * s_mn, 16, 0, 0);
+  constexpr int PER = 1024 / (int)sizeof(T), PARTS = EXT / PER > 0 ? EXT / PER : 1;  // elements per instruction, instructions per row
+  const int row = inst / PARTS, part = inst % PARTS;
+  const T* p = g + (16 / (int)sizeof(T)) * lane + part * PER + (long)row * ld;
+  __builtin_amdgcn_global_load_lds(p, xs + row * s_mn + part * PER, 16, 0, 0);
 #endif
 }
 
@@ -269,7 +271,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // fp64: only with a K-major A (TN 73.2 -> 74.0, TT 72.6 -> 73.6 TFLOP/s at 8192^3); NN measured the same either way
   // (73.55 / 73.45) and keeps the register path.
   constexpr bool SWZL = DIR && ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
-                        ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16 && AK) || (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
+                        ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16 && AK) ||
+                         (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
   constexpr bool V2 = PLK_V2 && SWZL && sizeof(T) == 4 && (AK || BKM);
   using LA = Lds<T, AK, BM, BK, SWZL>;
   using LB = Lds<T, BKM, BN, BK, SWZL>;
@@ -337,18 +340,25 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // 1 per 2 about half of that).  The epilogue maps the accumulators back with the same rule.
   constexpr bool PAIRED = sizeof(T) == 4 || PLK_F64_PAIR;
   constexpr bool A_PAIR = PAIRED && !AK, B_PAIR = PAIRED && !BKM;
+  // rows of an MN-major operand a lane holds side by side: all its blocks' (8 or 16 bytes).  Block j of a lane is row
+  // (j / PF) * BLK * PF + PF * idx + j % PF of the wave's part -- with PF = 1 the plain rule.
+  constexpr int PFA = A_PAIR ? NBM : 1, PFB = B_PAIR ? NBN : 1;
+  auto row_a = [&](int j) { return wm + (j / PFA) * (BLK * PFA) + PFA * idx + j % PFA; };
+  auto row_b = [&](int i, int r) { return wn + (i / PFB) * (BLK * PFB) + PFB * r + i % PFB; };
   constexpr int G = 16, SPG = G / Tr::KSTEP;   // V2: k group depth, MFMA steps per group
   // this lane's A / B operand of k-step 0, block 0 (V2: of the first step of a group)
-  const T* const lane_a = smem + LA::at(V2 ? kk * SPG : kk, wm + (A_PAIR ? NBM * idx : idx));
-  const T* const lane_b = smem + ASZ + LB::at(V2 ? kk * SPG : kk, wn + (B_PAIR ? NBN * idx : idx));
-  constexpr int A_KS = LA::at(Tr::KSTEP, 0), A_BL = A_PAIR ? 1 : LA::at(0, BLK);    // strides per k-step / per block
-  constexpr int B_KS = LB::at(Tr::KSTEP, 0), B_BL = B_PAIR ? 1 : LB::at(0, BLK);
+  const T* const lane_a = smem + LA::at(V2 ? kk * SPG : kk, wm + PFA * idx);
+  const T* const lane_b = smem + ASZ + LB::at(V2 ? kk * SPG : kk, wn + PFB * idx);
+  constexpr int A_KS = LA::at(Tr::KSTEP, 0), B_KS = LB::at(Tr::KSTEP, 0);    // strides per k-step
+  // where block j sits relative to block 0 of the lane
+  auto a_blk = [](int j) { return AK ? LA::at(0, j * BLK) : (j / PFA) * (BLK * PFA) + j % PFA; };
+  auto b_blk = [](int i) { return BKM ? LB::at(0, i * BLK) : (i / PFB) * (BLK * PFB) + i % PFB; };
   constexpr int KV = V2 ? SPG / 2 : Tr::KV;    // V2: == VEC, the steps one 16-byte read of a K-major operand serves
   static_assert(!V2 || KV == Tr::VEC, "a 16-byte chunk of a K-major row must hold exactly KV steps");
   constexpr int KS = BK / (Tr::KSTEP * KV);  // operand refreshes ("steps") per panel
   // LDS read instructions per refresh
-  constexpr int RD_A = V2 ? (AK ? NBM : KV * (NBM * (int)sizeof(T) > 16 ? 2 : 1)) : (A_PAIR ? 1 : NBM);
-  constexpr int RD_B = V2 ? (BKM ? NBN : KV * (NBN * (int)sizeof(T) > 16 ? 2 : 1)) : (B_PAIR ? 1 : NBN);
+  constexpr int RD_A = V2 ? (AK ? NBM : KV * (NBM / PFA)) : (A_PAIR ? 1 : NBM);
+  constexpr int RD_B = V2 ? (BKM ? NBN : KV * (NBN / PFB)) : (B_PAIR ? 1 : NBN);
   constexpr int NREADS = RD_A + RD_B;
   // K-major operand in the swizzled layout: where this lane finds its values in its row of block 0 (the same place in
   // every block: a block is a multiple of the swizzle period).  V2: the chunk of refresh (g, h) -- group g of the panel,
@@ -375,13 +385,15 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
           for (int v = 0; v < KV; ++v) am[v][j] = x[v];
         }
       } else {
-        typedef T opv_t __attribute__((ext_vector_type(NBM)));
+        typedef T opv_t __attribute__((ext_vector_type(PFA)));
 #pragma unroll
-        for (int v = 0; v < KV; ++v) {
-          const opv_t x = *reinterpret_cast<const opv_t*>(lane_a + buf * STAGE + (g * G + h * KV + v) * LA::S_MN);
+        for (int v = 0; v < KV; ++v)
 #pragma unroll
-          for (int j = 0; j < NBM; ++j) am[v][j] = x[j];
-        }
+          for (int q = 0; q < NBM / PFA; ++q) {
+            const opv_t x = *reinterpret_cast<const opv_t*>(lane_a + buf * STAGE + (g * G + h * KV + v) * LA::S_MN + q * BLK * PFA);
+#pragma unroll
+            for (int e = 0; e < PFA; ++e) am[v][q * PFA + e] = x[e];
+          }
       }
       if constexpr (BKM) {
 #pragma unroll
@@ -391,13 +403,15 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
           for (int v = 0; v < KV; ++v) bnv[v][i] = x[v];
         }
       } else {
-        typedef T opv_t __attribute__((ext_vector_type(NBN)));
+        typedef T opv_t __attribute__((ext_vector_type(PFB)));
 #pragma unroll
-        for (int v = 0; v < KV; ++v) {
-          const opv_t x = *reinterpret_cast<const opv_t*>(lane_b + buf * STAGE + (g * G + h * KV + v) * LB::S_MN);
+        for (int v = 0; v < KV; ++v)
 #pragma unroll
-          for (int i = 0; i < NBN; ++i) bnv[v][i] = x[i];
-        }
+          for (int q = 0; q < NBN / PFB; ++q) {
+            const opv_t x = *reinterpret_cast<const opv_t*>(lane_b + buf * STAGE + (g * G + h * KV + v) * LB::S_MN + q * BLK * PFB);
+#pragma unroll
+            for (int e = 0; e < PFB; ++e) bnv[v][q * PFB + e] = x[e];
+          }
       }
       return;
     }
@@ -405,10 +419,10 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     for (int v = 0; v < KV; ++v) {
 #pragma unroll
       for (int j = 0; j < NBM; ++j)
-        am[v][j] = (SWZL && AK) ? a_kp[ks * KV + v][buf * STAGE + j * BLK * LA::S_K] : lane_a[buf * STAGE + (ks * KV + v) * A_KS + j * A_BL];
+        am[v][j] = (SWZL && AK) ? a_kp[ks * KV + v][buf * STAGE + j * BLK * LA::S_K] : lane_a[buf * STAGE + (ks * KV + v) * A_KS + a_blk(j)];
 #pragma unroll
       for (int i = 0; i < NBN; ++i)
-        bnv[v][i] = (SWZL && BKM) ? b_kp[ks * KV + v][buf * STAGE + i * BLK * LB::S_K] : lane_b[buf * STAGE + (ks * KV + v) * B_KS + i * B_BL];
+        bnv[v][i] = (SWZL && BKM) ? b_kp[ks * KV + v][buf * STAGE + i * BLK * LB::S_K] : lane_b[buf * STAGE + (ks * KV + v) * B_KS + b_blk(i)];
     }
   };
   auto mfma_step = [&](const T (&am)[KV][NBM], const T (&bnv)[KV][NBN]) {
@@ -444,7 +458,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
 #pragma unroll
       for (int i = 0; i < NVA; ++i) {
         if constexpr (AK) dma_krows<LA, T>(Ab, lda, smem, wave_u + 4 * i, lane);
-        else dma_row<T>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
+        else dma_row<T, BM>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
       }
     } else {
       gload<LA, T, false>(Ab, lda, 0, 0, true, ra, tid);
@@ -455,7 +469,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
 #pragma unroll
       for (int i = 0; i < NVB; ++i) {
         if constexpr (BKM) dma_krows<LB, T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane);
-        else dma_row<T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
+        else dma_row<T, BN>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
       }
     } else {
       gload<LB, T, false>(Bb, ldb, 0, 0, true, rb, tid);
@@ -480,10 +494,10 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         const int vec = (A_DIR ? 0 : NVA) + slot;  // direct rows: A's first when both are direct
         if (vec < NVA) {
           if constexpr (AK) dma_krows<LA, T>(ga, lda, nxt_a, wave_u + 4 * vec, lane);
-          else dma_row<T>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
+          else dma_row<T, BM>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
         } else {
           if constexpr (BKM) dma_krows<LB, T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane);
-          else dma_row<T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
+          else dma_row<T, BN>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
         }
         return;
       }
@@ -585,28 +599,32 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     }
   }
 
-  // Interior tile: no guards, so the compiler can batch the reads of C.  With the paired row rule (fp32, MN-major A) a
-  // lane's NBM accumulators of one column are adjacent in memory and go out as one 8- or 16-byte access when C is
-  // aligned for it.  Same arithmetic per element as the guarded loop below.
+  // Interior tile: no guards, so the compiler can batch the reads of C.  With the paired row rule (MN-major A) a lane's
+  // PFA accumulators of one column are adjacent in memory and go out as one 8- or 16-byte access when C is aligned for
+  // it.  Same arithmetic per element as the guarded loop below.
+  // acc[i][j][r] is C(m0 + row_a(j), n0 + row_b(i, drow(r, kk))).
   if (mrem == BM && nrem == BN) {
-    if constexpr (A_PAIR) {
-      typedef T cvec_t __attribute__((ext_vector_type(NBM)));
+    if constexpr (PFA > 1) {
+      typedef T cvec_t __attribute__((ext_vector_type(PFA)));
       if (vecC) {
 #pragma unroll
         for (int i = 0; i < NBN; ++i) {
 #pragma unroll
           for (int r = 0; r < Tr::NACC; ++r) {
-            const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
-            cvec_t* const cp = reinterpret_cast<cvec_t*>(C + (long)(n0 + n) * ldc + m0 + wm + NBM * idx);
-            cvec_t v;
+            const int n = row_b(i, Tr::drow(r, kk));
 #pragma unroll
-            for (int j = 0; j < NBM; ++j) v[j] = alpha * acc[i][j][r];
-            if (beta != T(0)) {
-              const cvec_t c = *cp;
+            for (int q = 0; q < NBM / PFA; ++q) {
+              cvec_t* const cp = reinterpret_cast<cvec_t*>(C + (long)(n0 + n) * ldc + m0 + row_a(q * PFA));
+              cvec_t v;
 #pragma unroll
-              for (int j = 0; j < NBM; ++j) v[j] += beta * c[j];
+              for (int e = 0; e < PFA; ++e) v[e] = alpha * acc[i][q * PFA + e][r];
+              if (beta != T(0)) {
+                const cvec_t c = *cp;
+#pragma unroll
+                for (int e = 0; e < PFA; ++e) v[e] += beta * c[e];
+              }
+              *cp = v;
             }
-            *cp = v;
           }
         }
         return;
@@ -616,33 +634,31 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     for (int i = 0; i < NBN; ++i) {
 #pragma unroll
       for (int r = 0; r < Tr::NACC; ++r) {
-        const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
+        const int n = row_b(i, Tr::drow(r, kk));
         T* const ccol = C + (long)(n0 + n) * ldc + m0;
         T v[NBM];
 #pragma unroll
         for (int j = 0; j < NBM; ++j) v[j] = alpha * acc[i][j][r];
         if (beta != T(0)) {
 #pragma unroll
-          for (int j = 0; j < NBM; ++j) v[j] += beta * ccol[A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx];
+          for (int j = 0; j < NBM; ++j) v[j] += beta * ccol[row_a(j)];
         }
 #pragma unroll
-        for (int j = 0; j < NBM; ++j) ccol[A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx] = v[j];
+        for (int j = 0; j < NBM; ++j) ccol[row_a(j)] = v[j];
       }
     }
     return;
   }
-  // epilogue: acc[i][j][r] is C(m0 + wm + j*BLK + idx, n0 + wn + i*BLK + drow(r, kk)), or with the paired row rule
-  // C(m0 + wm + NBM*idx + j, n0 + wn + NBN*drow(r, kk) + i)
 #pragma unroll
   for (int i = 0; i < NBN; ++i) {
 #pragma unroll
     for (int r = 0; r < Tr::NACC; ++r) {
-      const int n = B_PAIR ? wn + NBN * Tr::drow(r, kk) + i : wn + i * BLK + Tr::drow(r, kk);
+      const int n = row_b(i, Tr::drow(r, kk));
       if (n < nrem) {
         T* ccol = C + (long)(n0 + n) * ldc + m0;
 #pragma unroll
         for (int j = 0; j < NBM; ++j) {
-          const int m = A_PAIR ? wm + NBM * idx + j : wm + j * BLK + idx;
+          const int m = row_a(j);
           if (m < mrem) {
             T v = alpha * acc[i][j][r];
             if (beta != T(0)) v += beta * ccol[m];
