@@ -8,11 +8,12 @@
 //     workgroups per CU); fp32 also has 256 x 128 (two workgroups per CU) and 256 x 256 (each wave owns 128 x 128
 //     with 256 accumulator registers, one workgroup per CU) for problems with enough such tiles to fill the CUs;
 //   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2 or 4 x 4);
-//   * A and B k-panels (16 elements deep, 32 for the large tile) are staged global -> registers -> LDS,
-//     double-buffered, one barrier per k-panel; the next panel's global loads are in flight while the current one is
-//     multiplied; when both operands are MN-major (NT) and a panel row is exactly 1 KiB (fp64 128 x 128, fp32
-//     256 x 256) the rows go global -> LDS directly instead (fp64 NT 72.8 -> 73.7, fp32 NT 148.7 -> 149.9 TFLOP/s at
-//     8192^3);
+//   * A and B k-panels (16 elements deep, 32 for the large tile) sit in LDS, double-buffered, one barrier per k-panel.
+//     They get there through registers (global loads two panels ahead, LDS stores one ahead, both spread between the
+//     MFMAs) or, where every panel of the tile can, straight from global memory (global_load_lds_dwordx4, one panel
+//     ahead): MN-major panels whose rows are exactly 1 KiB (fp64 128 x 128, fp32 256 x 256), K-major panels of those
+//     tiles in a swizzled unpadded layout.  Direct: fp32 256 x 256 (every transpose), fp64 NT, TN, TT; staged: the
+//     fp64 NN tile (no difference measured), the smaller fp32 tiles, every workgroup with a short k;
 //   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
 //     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
@@ -24,7 +25,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
-// Row index (MFMA i) of accumulator element r for lane group g = lane / 16 in the 16x16 fp64 result block.
+// Build-time switches (timing experiments; the defaults are what ships).
 #ifndef PLK_F64_BK
 #define PLK_F64_BK 16
 #endif
@@ -51,6 +52,7 @@
 #ifndef PLK_DMA_MASK
 #define PLK_DMA_MASK 0x080
 #endif
+// Row index (MFMA i) of accumulator element r for lane group g = lane / 16 in the 16x16 fp64 result block.
 #ifndef PLK_F64_DROW
 #define PLK_F64_DROW(r, g) (4 * (r) + (g))
 #endif
