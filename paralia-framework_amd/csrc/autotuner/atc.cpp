@@ -259,12 +259,15 @@ paralia::StageTimes nominal_stage_times(const ProblemDesc& d, long T) {
 // kernel's larger macro tiles leave no room for a second workgroup on a compute unit, so nothing overlaps a
 // workgroup's prologue (first panels) and epilogue (the read-modify-write of its part of C): measured on sgemm
 // 32768^3 N/T at T = 4096, 336 launches fewer took 13.5 ms less = 40 us each, for one round of 256 tiles of 256 x 256
-// per launch.  The fp64 kernel runs two workgroups per compute unit that cover each other's ends: joining its launches
-// changed nothing (124.0 against 124.3 ms on dgemm 16384^3), so there the planner is not offered the choice.
+// per launch.  The fp64 kernel runs two workgroups per compute unit that cover each other's ends; there a launch saved
+// is worth the gap between two launches of a stream: dgemm 16384^3 at T = 2048 with 128 launches fewer (448 instead of
+// 576) took 0.55 ms less (123.3 / 123.7 against 123.9 / 124.2 ms), 4 us each.
 static double paralia_merge_saving(const ProblemDesc& d, long T) {
-  const char* env = getenv("PARALIA_MERGE_CHAINS");  // "0": never merge, "1": offer it for every type
+  const char* env = getenv("PARALIA_MERGE_CHAINS");  // "0": never merge
   if (env && *env && atoi(env) == 0) return 0.0;
-  if (d.dtype_sz != 4 && !(env && atoi(env) == 1)) return 0.0;
+  // measured for tiles that fill the device by themselves; smaller ones run split-K kernels whose time a joined k range
+  // changes in ways this term does not describe
+  if (d.dtype_sz != 4) return T >= 1792 ? 4e-6 : 0.0;
   // a launch with fewer workgroups than compute units wastes that much less of the device: scale by the rounds of 256
   // workgroups it amounts to, as a fraction
   const double rounds = (double)((T + 255) / 256) * (double)((T + 255) / 256) / 256.0;
