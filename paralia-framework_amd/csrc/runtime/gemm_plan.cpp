@@ -161,6 +161,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   if (p_in.T <= 0 || p_in.M <= 0 || p_in.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
   GemmPlan plan;
   plan.p = p_in;
+  if (order_id < 0 || order_id / ORDER_K_SPLIT > 2) throw std::runtime_error("gemm plan: unknown order id");
   plan.p.k_split = 1 << (order_id / ORDER_K_SPLIT);
   const GemmProblem& p = plan.p;
   if (order_id >= ORDER_K_SPLIT && p.slabs() == 1) throw std::runtime_error("gemm plan: this problem has no thin start");

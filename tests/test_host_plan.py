@@ -444,3 +444,9 @@ def test_thin_start_plans(pkg, order, locs, beta_zero):
     check_async_safety(flat)
     with pytest.raises(pkg.ParaliaError, match="thin start"):
         pkg.plan_rows(M, N, 20, 32, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)     # K < T: nothing to cut
+
+
+def test_unknown_order_ids_are_refused(pkg):
+    for order in (480000, 640001, -5):
+        with pytest.raises(pkg.ParaliaError, match="unknown order id"):
+            pkg.plan_rows(256, 256, 256, 64, 1, 1, 1, 0, 8, 2, 0, order)
