@@ -291,6 +291,8 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.h2d_sl = std::max(1.0, h2d->sl); st.d2h_sl = std::max(1.0, d2h->sl);
   st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
   st.merge_saving = paralia_merge_saving(d, T);
+  const char* thin = getenv("PARALIA_THIN_START");  // "0": never cut the first k tile into slabs
+  st.thin_start = !(thin && *thin && atoi(thin) == 0);
   return st;
 }
 

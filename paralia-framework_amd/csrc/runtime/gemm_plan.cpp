@@ -557,7 +557,7 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   // the best order also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link
   GemmProblem unsplit = p;
   unsplit.k_split = 1;
-  if ((p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit)) {
+  if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit)) {
     const int base_id = best_id;
     for (int s = 1; s <= 2; ++s) {
       try {

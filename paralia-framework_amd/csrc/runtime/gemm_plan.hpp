@@ -125,6 +125,7 @@ struct StageTimes {
   // seconds a launch over kn k tiles of a full T x T C tile takes less than kn separate launches, per launch saved
   // (0: merging K chains is not worth considering for this kernel)
   double merge_saving = 0;
+  bool thin_start = true;            // offer the thin start (order ids of 160000 and above) to the order search
   // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch
   double slab_fixed = 2e-6;  // measured: 2048 x 2048 x 1024 119.9 us, x 512 61.2 us against 236.7 us for the whole tile
 };
