@@ -475,6 +475,30 @@ def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs
             assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("order,T", [(160001, 100), (320002, 100), (240000, 100), (160000, 72)])
+def test_gemm_thin_start_with_odd_slabs(pkg, L, orc, ta, tb, order, T, monkeypatch):
+    """Thin-start slabs whose depth is not a multiple of the 16-byte vector (T = 100: slabs of 50 and of 25 elements; T =
+    72: 36): the tiles that follow a slab start at an odd k, so operands contiguous along k lose their alignment and the
+    tile kernel takes its element-load path.  Integer data, pinned and pageable operands, both types: exact."""
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+    M, N, K = 230, 310, 275 + (order % 7)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    rng = np.random.default_rng(order + T)
+    for dtype, brute in ((np.float64, orc.orc_dgemm_bruteforce), (np.float32, orc.orc_sgemm_bruteforce)):
+        A = rng.integers(-4, 5, ra * ca).astype(dtype)
+        B = rng.integers(-4, 5, rb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, M * N).astype(dtype)
+        for locs in ((-1, -1, -1), (-2, -2, -2)):
+            ref = C0.copy()
+            brute(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A), ra, ptr(B), rb, -1.0, ptr(ref), M)
+            bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, C0, locs[2])
+            info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 2.0, -1.0, bA, ra, bB, rb, bC, M, T=T)
+            assert info.order_id == order and k_tiles(info, K) == -(-K // T) + (1 << (order // 160000)) - 1
+            assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, locs)
+
+
 def test_sgemm_autotuned_call_merges_k_chains(pkg, L, orc, openblas):
     """No pin: for fp32 with A and B on the host the planner is offered the merged variants and its simulator takes
     one when the product is bound by compute and the chains are long (12288 x 12288 x 16384 here); parity against
