@@ -69,6 +69,10 @@ struct GPUexecModel {
   std::vector<long> T;
   std::vector<double> av_time;
   std::vector<char> TransA, TransB;  // empty for BLAS-1
+  // BLAS-3 only, optional (<func>_lone-launch_dev-<id>.log, rows TransA,TransB,T,seconds): time of a tile launch that has
+  // the device to itself; av_time is the time per launch when the compute streams keep it filled.  -1 where not measured.
+  std::vector<double> lone_time;
+  double lone_ratio(long T, char TransA, char TransB) const;  // lone / filled time of that row, 1 when unknown
   long lines() const { return (long)T.size(); }
   long MinT() const;
   long MaxT() const;

@@ -1,6 +1,7 @@
 // Link models and exec-time lookup tables: file parsing and prediction.
 // Formats and arithmetic follow the reference's Autotuner/src/CoModel.cpp:14-66,107-162 and
 // GPUexec_lookup.cpp:15-129,250-359 so that database files are interchangeable.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -207,5 +208,28 @@ GPUexecModel* GPUexecModel_init(const std::string& db_dir, int dev_id, const cha
     delete m;
     error("GPUexecModel_init: empty lookup table %s\n", filename);
   }
+  m->lone_time.assign(m->T.size(), -1.0);
+  if (problem == BLAS3) {
+    snprintf(filename, sizeof filename, "%s/Processed/%s_lone-launch_dev-%d.log", db_dir.c_str(), func, dev_id);
+    fp = fopen(filename, "r");  // optional: databases without it price every launch at its filled-device time
+    if (fp) {
+      while (fgets(line, sizeof line, fp)) {
+        char ta, tb;
+        long Tv;
+        double t;
+        if (sscanf(line, "%c,%c,%ld,%lf", &ta, &tb, &Tv, &t) != 4) continue;
+        for (size_t i = 0; i < m->T.size(); ++i)
+          if (m->T[i] == Tv && m->TransA[i] == ta && m->TransB[i] == tb) m->lone_time[i] = t;
+      }
+      fclose(fp);
+    }
+  }
   return m;
+}
+
+double GPUexecModel::lone_ratio(long Tin, char ta, char tb) const {
+  for (size_t i = 0; i < T.size(); ++i)
+    if (T[i] == Tin && (TransA.empty() || (TransA[i] == ta && TransB[i] == tb)))
+      return (i < lone_time.size() && lone_time[i] > 0 && av_time[i] > 0) ? std::max(1.0, lone_time[i] / av_time[i]) : 1.0;
+  return 1.0;
 }

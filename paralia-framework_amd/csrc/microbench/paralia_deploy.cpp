@@ -89,7 +89,7 @@ static std::vector<long> sweep(long start, long step, long limit, int double_at)
   return out;
 }
 
-struct Row { char ta, tb; long T; Sample s; };
+struct Row { char ta, tb; long T; Sample s; Sample lone; };
 
 static void mkdirs(const std::string& d) {
   mkdir(d.c_str(), 0755);
@@ -149,7 +149,17 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
           return (csecond() - t0) / batch;
         };
         run();  // warm-up
-        Row r{ta, tb, Tt, sample_until_stable(run)};
+        Row r{ta, tb, Tt, sample_until_stable(run), Sample()};
+        // the same launches on one stream only: what a subkernel takes when nothing runs beside it
+        auto run_lone = [&]() {
+          const int n = std::max(2, batch / queues);
+          const double t0 = csecond();
+          for (int i = 0; i < n; ++i) launch(0);
+          must(pl_stream_sync(st[0]), "sync");
+          return (csecond() - t0) / n;
+        };
+        run_lone();
+        r.lone = sample_until_stable(run_lone);
         rows.push_back(r);
         fprintf(fp, "%ld,%ld,%ld, %e,%e,%e,%e,%ld,%e\n", Tt, Tt, Tt, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
         fprintf(stderr, "%s %c%c T=%ld: %.3f ms (%.1f GFLOP/s), margin %.2f%%, %ld samples\n", func, ta, tb, Tt, r.s.mean * 1e3,
@@ -165,6 +175,12 @@ static void bench_gemm(const std::string& db, const char* func, bool quick, int 
   if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
   for (const Row& r : rows)
     fprintf(fp, "%c,%c,%ld,%ld,%ld,%e,%e,%e,%e,%ld,%e\n", r.ta, r.tb, r.T, r.T, r.T, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
+  fclose(fp);
+  // not a table of the reference: the lone-launch times, TransA,TransB,T,seconds
+  snprintf(out, sizeof out, "%s/Processed/%s_lone-launch_dev-0.log", db.c_str(), func);
+  fp = fopen(out, "w");
+  if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  for (const Row& r : rows) fprintf(fp, "%c,%c,%ld,%e\n", r.ta, r.tb, r.T, r.lone.mean);
   fclose(fp);
   for (auto s : st) pl_stream_destroy(s);
   CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
@@ -206,7 +222,7 @@ static void bench_gemv(const std::string& db, bool quick) {
         return (csecond() - t0) / batch;
       };
       run();
-      Row r{ta, 'N', Tt, sample_until_stable(run)};
+      Row r{ta, 'N', Tt, sample_until_stable(run), Sample()};
       rows.push_back(r);
       fprintf(fp, "%ld,%ld, %e,%e,%e,%e,%ld,%e\n", Tt, Tt, r.s.mean, -1.0, -1.0, r.s.margin, r.s.n, r.s.bench_t);
       fprintf(stderr, "Dgemv %c T=%ld: %.4f ms (%.1f GB/s), margin %.2f%%, %ld samples\n", ta, Tt, r.s.mean * 1e3,

@@ -22,28 +22,23 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   std::vector<int> order;
   order.reserve((size_t)Mg * Ng * Kg);
   auto id = [&](int mi, int ni, int ki) { return (mi * Ng + ni) * Kg + ki; };
-  // One panel of C tiles, rows [m0, m1) x columns [n0, n1), in k-outer order.  Its first k-step walks the tiles in
-  // growing squares (shell d = max(row, column) inside the panel), so that every newly fetched A or B tile at once
-  // enables a whole row or column of subkernels; column by column the first fetches would enable one subkernel each
-  // while the compute streams starve.
+  // One panel of C tiles, rows [m0, m1) x columns [n0, n1), in k-outer order.  Every k-step walks the tiles in
+  // growing squares (shell d = max(row, column) inside the panel).  In the first steps, while the link is still behind,
+  // every newly fetched A or B tile then at once enables a whole row or column of subkernels (column by column the
+  // first fetches would enable one subkernel each while the compute streams starve).  Later the walk keeps the streams
+  // level: the K chains are dealt to the exec queues in first-fire order, which is this walk, so its consecutive
+  // subkernels sit on different queues in every step (column by column, a column whose tiles all drew the same queue
+  // runs on one stream while the other waits for the next column's B tile).
   auto panel = [&](int m0, int m1, int n0, int n1) {
     const int rows = m1 - m0, cols = n1 - n0;
     if (rows <= 0 || cols <= 0 || Kg <= 0) return;
-    for (int d = 0; d < std::max(rows, cols); ++d) {
-      if (d < cols)
-        for (int mi = 0; mi < std::min(d, rows); ++mi) order.push_back(id(m0 + mi, n0 + d, 0));
-      if (d < rows)
-        for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(m0 + d, n0 + ni, 0));
-    }
-    for (int ki = 1; ki < Kg; ++ki) {
-      if (orient == 0) {
-        for (int ni = n0; ni < n1; ++ni)
-          for (int mi = m0; mi < m1; ++mi) order.push_back(id(mi, ni, ki));
-      } else {
-        for (int mi = m0; mi < m1; ++mi)
-          for (int ni = n0; ni < n1; ++ni) order.push_back(id(mi, ni, ki));
+    for (int ki = 0; ki < Kg; ++ki)
+      for (int d = 0; d < std::max(rows, cols); ++d) {
+        if (d < cols)
+          for (int mi = 0; mi < std::min(d, rows); ++mi) order.push_back(id(m0 + mi, n0 + d, ki));
+        if (d < rows)
+          for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(m0 + d, n0 + ni, ki));
       }
-    }
   };
   if (orient == 0) {
     w = std::min(w, Ng);
@@ -96,8 +91,17 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
     for (int orient = 0; orient < 2; ++orient) {
       const int g = orient == 0 ? p.Ng() : p.Mg();
       if (probe) {
-        for (int w : probe_widths)
-          if (w < g) ids.push_back(20000 + order_id_of(orient, w));
+        // besides the two standard widths, the widest panel whose accumulators plus one k-step of A and B tiles fit the
+        // pool, and the next wider one: the best width of a limited pool sits there, and a probe without it can misjudge
+        // the tile size by 15 %
+        const int other = orient == 0 ? p.Mg() : p.Ng();
+        const int fit = (int)std::max<long>(1, (p.pool_blocks - other) / (other + 1));
+        int ws[4] = {probe_widths[0], probe_widths[1], fit, fit + 1};
+        for (int i = 0; i < 4; ++i) {
+          bool seen = false;
+          for (int j = 0; j < i; ++j) seen |= ws[j] == ws[i];
+          if (!seen && ws[i] < g) ids.push_back(20000 + order_id_of(orient, ws[i]));
+        }
       } else {
         for (int w : widths)
           if (w < g) ids.push_back(20000 + order_id_of(orient, w));
@@ -541,10 +545,12 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   int best_id = -1;
   PipelineResult best;
   std::string last_err;
+  std::vector<std::pair<double, int>> ranked;  // (makespan, id) of every feasible order, in candidate order
   for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0)) {
     try {
       GemmPlan plan = build_gemm_plan(p, id);
       PipelineResult r = simulate_plan(plan, st);
+      ranked.emplace_back(r.t_total, id);
       if (best_id < 0 || r.t_total < best.t_total * (1.0 - 1e-9)) {
         best = r;
         best_id = id;
@@ -554,22 +560,29 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
     }
   }
   if (best_id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
-  // the best order also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link
+  // the best orders also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link; the
+  // three best, because the order that wins with a thin start is often the runner-up without one (a wider panel,
+  // whose longer wait for its first tiles the slabs take away)
   GemmProblem unsplit = p;
   unsplit.k_split = 1;
   if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit)) {
-    const int base_id = best_id;
-    for (int s = 1; s <= 2; ++s) {
-      try {
-        GemmPlan plan = build_gemm_plan(p, base_id + s * ORDER_K_SPLIT);
-        PipelineResult r = simulate_plan(plan, st);
-        if (plan.n_evictions == 0 && r.t_total < best.t_total * (1.0 - 1e-3)) {
-          best = r;
-          best_id = base_id + s * ORDER_K_SPLIT;
+    // makespans that differ only in the last bits are ties (compared in single precision), and ties keep the candidate
+    // order, as the choice above does
+    std::stable_sort(ranked.begin(), ranked.end(),
+                     [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return (float)a.first < (float)b.first; });
+    const PipelineResult unsplit_best = best;
+    for (size_t b = 0; b < std::min<size_t>(3, ranked.size()); ++b)
+      for (int s = 1; s <= 2; ++s) {
+        try {
+          GemmPlan plan = build_gemm_plan(p, ranked[b].second + s * ORDER_K_SPLIT);
+          PipelineResult r = simulate_plan(plan, st);
+          if (plan.n_evictions == 0 && r.t_total < unsplit_best.t_total * (1.0 - 1e-3) && r.t_total < best.t_total) {
+            best = r;
+            best_id = ranked[b].second + s * ORDER_K_SPLIT;
+          }
+        } catch (const std::runtime_error&) {
         }
-      } catch (const std::runtime_error&) {
       }
-    }
   }
   if (best_out) *best_out = best;
   return best_id;

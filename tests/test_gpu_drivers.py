@@ -194,6 +194,19 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
         a, b = _table(os.path.join(fresh, n), 5), _table(os.path.join(shipped, n), 5)
         for k in keys:
             close(a[k], b[k], band, n + str(k))
+    # lone-launch times (a tile launch with the device to itself): never shorter than the filled-device time per launch
+    # beyond noise, and for 2048^3 fp64 (one workgroup per compute unit) longer by the 5 - 20 % the shipped table shows
+    for func in ("Dgemm", "Sgemm"):
+        lone = _table(os.path.join(fresh, func + "_lone-launch_dev-0.log"), 3)
+        filled = _table(os.path.join(fresh, func + "_lookup-table_dev-0.log"), 5)
+        assert len(lone) == len(filled)
+        for k, t in lone.items():
+            assert t > 0.9 * filled[k + (k[2], k[2])], (func, k, t)
+    lone = _table(os.path.join(fresh, "Dgemm_lone-launch_dev-0.log"), 3)
+    lone_shipped = _table(os.path.join(shipped, "Dgemm_lone-launch_dev-0.log"), 3)
+    close(lone[("N", "N", "2048")], lone_shipped[("N", "N", "2048")], 0.10, "lone 2048^3 fp64 launch")
+    ratio = lone[("N", "N", "2048")] / _table(os.path.join(fresh, names[0]), 5)[("N", "N", "2048", "2048", "2048")]
+    assert 1.03 < ratio < 1.25, ratio
     # matrix-vector and vector kernels take 40 - 80 us at the largest sizes of the quick sweep: launch and
     # synchronisation are a visible part of that, and working sets of 128 - 384 MiB sit partly inside the memory-side
     # cache, so these differ more between machines than the millisecond-scale GEMM tiles: a wider band

@@ -241,3 +241,67 @@ def test_gemm_order_can_be_pinned_and_pool_limits_change_the_pick(L, pkg, monkey
     monkeypatch.setenv("PARALIA_GEMM_ORDER", "8")  # 8 column tiles as one k-outer panel: 64 accumulators at least
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 1024, 5 * 1024 * 1024 * 8, C.byref(info)) == 0
     assert info.order_id != 8
+
+
+def _shipped_db(pkg):
+    return os.path.normpath(os.path.join(os.path.dirname(pkg.LIB_PATH), "..", "db", "mi355x"))
+
+
+def test_lone_launch_table_is_optional_and_raises_the_tile_price(L, pkg, tmp_path, monkeypatch):
+    """<func>_lone-launch_dev-0.log (TransA,TransB,T,seconds: a tile launch with the device to itself) is not a table of
+    the reference: a database without it loads and prices every launch at its filled-device time.  With it, a tile's
+    price grows by 7 % of (lone / filled - 1), so the prediction of a compute-bound call rises by at most that much and
+    tiles whose launches run alone at nearly the filled rate (4096) are hardly touched."""
+    import shutil
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    shipped = _shipped_db(pkg)
+    lone = {}
+    for line in open(os.path.join(shipped, "Processed", "Dgemm_lone-launch_dev-0.log")):
+        ta, tb, T, t = line.strip().split(",")
+        lone[(ta, tb, int(T))] = float(t)
+    filled = {}
+    for line in open(os.path.join(shipped, "Processed", "Dgemm_lookup-table_dev-0.log")):
+        f = line.strip().split(",")
+        filled[(f[0], f[1], int(f[2]))] = float(f[5])
+    assert set(lone) == set(filled)
+    r2048 = lone[("N", "N", 2048)] / filled[("N", "N", 2048)]
+    r3072 = lone[("N", "N", 3072)] / filled[("N", "N", 3072)]
+    r4096 = lone[("N", "N", 4096)] / filled[("N", "N", 4096)]
+    assert 1.03 < r2048 < 1.25 and r3072 > 1.25 and r4096 < 1.05     # whole rounds of workgroups or not
+    bare = tmp_path / "db"
+    shutil.copytree(shipped, bare)
+    for f in ("Dgemm_lone-launch_dev-0.log", "Sgemm_lone-launch_dev-0.log"):
+        os.remove(bare / "Processed" / f)
+    info = pkg.atc_info()
+    pred = {}
+    for name, d in (("with", shipped), ("without", str(bare))):
+        for T in (2048, 3072, 4096):
+            assert L.PARALiA_autotune(d.encode(), b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, T, 0, C.byref(info)) == 0
+            assert info.has_db == 1 and info.T == T
+            pred[(name, T)] = info.pred_t
+    L.PARALiA_set_db_dir(None)
+    for T, r in ((2048, r2048), (3072, r3072), (4096, r4096)):
+        rise = pred[("with", T)] / pred[("without", T)] - 1
+        assert -1e-9 <= rise <= 0.07 * (r - 1) + 1e-3, (T, rise, r)
+    assert pred[("with", 3072)] / pred[("without", 3072)] > pred[("with", 4096)] / pred[("without", 4096)] + 0.01
+
+
+def test_limited_pool_probe_keeps_the_tile_whose_best_panel_width_just_fits(L, pkg, monkeypatch):
+    """With a 1 GiB pool the 16384^3 fp64 problem runs best with 2048-tiles in repeated panels three tiles wide (the
+    widest panel whose accumulators and one k-step of operand tiles nearly fit 32 blocks).  The first pass of the tile
+    search prices every tile size with a few widths only; it must include that width, or the tile is dropped there and a
+    slower one is chosen (measured: 173 ms against 185 ms for the 2816-tile the coarser probe used to pick)."""
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    info = pkg.atc_info()
+    d = _shipped_db(pkg).encode()
+    assert L.PARALiA_autotune(d, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 1 << 30, C.byref(info)) == 0
+    picked_T, picked_t = info.T, info.pred_t
+    best = None
+    for T in (1536, 2048, 2816, 4096):
+        assert L.PARALiA_autotune(d, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, T, 1 << 30, C.byref(info)) == 0
+        if best is None or info.pred_t < best[1]:
+            best = (T, info.pred_t)
+    L.PARALiA_set_db_dir(None)
+    assert picked_T == best[0] == 2048 and abs(picked_t - best[1]) <= 1e-9 * best[1]

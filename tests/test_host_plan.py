@@ -233,6 +233,13 @@ def test_panel_starts_in_growing_squares(pkg):
             fetches_before.append(n_fetch)
     # 2 tiles -> 1 subkernel, 4 -> 4, 6 -> 9, 8 -> 16, 10 -> 25 (5 x 5), then one fetched A tile per 5 subkernels
     assert [fetches_before[i] for i in (0, 3, 8, 15, 24, 29, 39)] == [2, 4, 6, 8, 10, 11, 13]
+    # every later k-step walks the panel the same way, and since the K chains were dealt to the two exec queues in that
+    # order, consecutive subkernels of a step sit on different queues (column by column, column 0 of this panel would be
+    # eight subkernels on one queue while the other waits for the next column's B tile)
+    for ki in range(1, 8):
+        step = [r for r in rows if r["kind"] == GEMM and r["ki"] == ki and r["ni"] < 5]
+        assert [(r["mi"], r["ni"]) for r in step] == first
+        assert all(a["stream"] != b["stream"] for a, b in zip(step, step[1:]))
 
 
 def test_pipeline_simulation(pkg, L):
