@@ -77,8 +77,12 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
     const int g = orient == 0 ? p.Ng() : p.Mg();
     if (orient == 0 && !probe) ids.push_back(order_id_of(0, 0));
     if (probe) {
+      // two narrow panels and one three quarters of the grid wide: compute-bound shapes want the wide one (16384^3: five
+      // or six of eight), and a probe without it misjudged 2048-tiles by 8 % (16384 x 8192 x 16384)
+      const int wide = (3 * g + 2) / 4;
       for (int w : probe_widths)
         if (w < g) ids.push_back(order_id_of(orient, w));
+      if (wide < g && wide != probe_widths[0] && wide != probe_widths[1]) ids.push_back(order_id_of(orient, wide));
     } else {
       for (int w : widths)
         if (w < g) ids.push_back(order_id_of(orient, w));
