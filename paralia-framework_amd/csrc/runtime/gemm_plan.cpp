@@ -40,6 +40,34 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
           for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(m0 + d, n0 + ni, ki));
       }
   };
+  if (w >= ORDER_BLOCK_ROWS) {
+    // Block orders (w = rows * 100 + columns): a block of rows x columns C tiles at the top left as one k-outer panel.
+    // orient 0: then the other rows of the block's columns, then the other columns, tile by tile; orient 1: the other
+    // columns of the block's rows first, then the other rows.  Against a panel over all rows the block needs fewer
+    // tiles before its C tiles are complete, so the write-backs start earlier: the order for shapes the link bounds.
+    const int wm = std::min(w / ORDER_BLOCK_ROWS, Mg), wn = std::min(w % ORDER_BLOCK_ROWS, Ng);
+    if (repeat || wn < 1) throw std::runtime_error("gemm plan: unknown order id");
+    panel(0, wm, 0, wn);
+    auto chains = [&](int m0, int m1, int n0, int n1, bool rows_outer) {
+      if (rows_outer) {
+        for (int mi = m0; mi < m1; ++mi)
+          for (int ni = n0; ni < n1; ++ni)
+            for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+      } else {
+        for (int ni = n0; ni < n1; ++ni)
+          for (int mi = m0; mi < m1; ++mi)
+            for (int ki = 0; ki < Kg; ++ki) order.push_back(id(mi, ni, ki));
+      }
+    };
+    if (orient == 0) {
+      chains(wm, Mg, 0, wn, true);    // a fetched row of A serves the block's columns
+      chains(0, Mg, wn, Ng, false);   // a fetched column of B serves every row
+    } else {
+      chains(0, wm, wn, Ng, false);
+      chains(wm, Mg, 0, Ng, true);
+    }
+    return order;
+  }
   if (orient == 0) {
     w = std::min(w, Ng);
     if (repeat) {
@@ -89,6 +117,16 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
     }
     ids.push_back(order_id_of(orient, g));
   }
+  // blocks one or two tiles short of the grid in each direction (full pool only: a block order re-reads nothing)
+  if (!limited && p.Mg() > 1 && p.Ng() > 1)
+    for (int orient = 0; orient < 2; ++orient)
+      for (int dm = 1; dm <= (probe ? 1 : 2); ++dm)
+        for (int dn = 1; dn <= (probe ? 1 : 2); ++dn) {
+          const int wm = p.Mg() - dm, wn = p.Ng() - dn;
+          if (wm < 1 || wn < 1 || wm >= ORDER_BLOCK_ROWS || wn >= ORDER_BLOCK_ROWS) continue;
+          if (probe && orient == 1) continue;
+          ids.push_back(order_id_of(orient, wm * ORDER_BLOCK_ROWS + wn));
+        }
   // every panel k-outer: what a block pool smaller than the working set needs (each fetched tile is used by a whole
   // row or column of the panel before it is evicted); a panel as wide as the grid is already listed above
   if (!probe || limited)
@@ -546,50 +584,60 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
 }
 
 int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best_out, bool probe) {
-  int best_id = -1;
-  PipelineResult best;
+  // Two groups of orders, each with its own best: the panel orders, and the block orders (w >= ORDER_BLOCK_ROWS), which
+  // end in two tile-by-tile phases and are taken only when they win by more than a percent (12288^3: simulated 0.6 %
+  // faster than the best panel order, measured 1 % slower; 8192^3: simulated 3.9 %, measured 5.6 % faster).
+  struct Group {
+    int id = -1;
+    PipelineResult r;
+    std::vector<std::pair<double, int>> ranked;  // (makespan, id) of every feasible order, in candidate order
+  } grp[2];
+  auto is_block = [](int id) { return id % 10000 >= ORDER_BLOCK_ROWS; };
   std::string last_err;
-  std::vector<std::pair<double, int>> ranked;  // (makespan, id) of every feasible order, in candidate order
   for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0)) {
     try {
       GemmPlan plan = build_gemm_plan(p, id);
       PipelineResult r = simulate_plan(plan, st);
-      ranked.emplace_back(r.t_total, id);
-      if (best_id < 0 || r.t_total < best.t_total * (1.0 - 1e-9)) {
-        best = r;
-        best_id = id;
+      Group& g = grp[is_block(id) ? 1 : 0];
+      g.ranked.emplace_back(r.t_total, id);
+      if (g.id < 0 || r.t_total < g.r.t_total * (1.0 - 1e-9)) {
+        g.r = r;
+        g.id = id;
       }
     } catch (const std::runtime_error& e) {
       last_err = e.what();  // this order does not fit the pool; others may
     }
   }
-  if (best_id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
+  if (grp[0].id < 0 && grp[1].id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
   // the best orders also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link; the
-  // three best, because the order that wins with a thin start is often the runner-up without one (a wider panel,
-  // whose longer wait for its first tiles the slabs take away)
+  // three best of a group, because the order that wins with a thin start is often the runner-up without one (a wider
+  // panel, whose longer wait for its first tiles the slabs take away)
   GemmProblem unsplit = p;
   unsplit.k_split = 1;
-  if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit)) {
-    // makespans that differ only in the last bits are ties (compared in single precision), and ties keep the candidate
-    // order, as the choice above does
-    std::stable_sort(ranked.begin(), ranked.end(),
-                     [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return (float)a.first < (float)b.first; });
-    const PipelineResult unsplit_best = best;
-    for (size_t b = 0; b < std::min<size_t>(3, ranked.size()); ++b)
-      for (int s = 1; s <= 2; ++s) {
-        try {
-          GemmPlan plan = build_gemm_plan(p, ranked[b].second + s * ORDER_K_SPLIT);
-          PipelineResult r = simulate_plan(plan, st);
-          if (plan.n_evictions == 0 && r.t_total < unsplit_best.t_total * (1.0 - 1e-3) && r.t_total < best.t_total) {
-            best = r;
-            best_id = ranked[b].second + s * ORDER_K_SPLIT;
+  if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit))
+    for (Group& g : grp) {
+      if (g.id < 0) continue;
+      // makespans that differ only in the last bits are ties (compared in single precision), and ties keep the
+      // candidate order, as the choice above does
+      std::stable_sort(g.ranked.begin(), g.ranked.end(),
+                       [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return (float)a.first < (float)b.first; });
+      const double unsplit_best = g.r.t_total;
+      for (size_t b = 0; b < std::min<size_t>(3, g.ranked.size()); ++b)
+        for (int s = 1; s <= 2; ++s) {
+          try {
+            GemmPlan plan = build_gemm_plan(p, g.ranked[b].second + s * ORDER_K_SPLIT);
+            PipelineResult r = simulate_plan(plan, st);
+            if (plan.n_evictions == 0 && r.t_total < unsplit_best * (1.0 - 1e-3) && r.t_total < g.r.t_total) {
+              g.r = r;
+              g.id = g.ranked[b].second + s * ORDER_K_SPLIT;
+            }
+          } catch (const std::runtime_error&) {
           }
-        } catch (const std::runtime_error&) {
         }
-      }
-  }
-  if (best_out) *best_out = best;
-  return best_id;
+    }
+  const Group& pick = (grp[0].id < 0 || (grp[1].id >= 0 && grp[1].r.t_total < 0.99 * grp[0].r.t_total)) ? grp[1] : grp[0];
+  if (best_out) *best_out = pick.r;
+  return pick.id;
 }
 
 }  // namespace paralia

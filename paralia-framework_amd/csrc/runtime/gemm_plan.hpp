@@ -94,6 +94,11 @@ struct GemmPlan {
 // large fp32 tiles, whose workgroups hold a compute unit alone, the prologue and epilogue nothing else overlaps -- at
 // the price of starting only when all its tiles have arrived.  Needs a pool that holds the whole working set.
 constexpr int ORDER_MERGE_CHAINS = 80000;
+// w = rows * 100 + columns (rows >= 1): block orders.  That block of C tiles at the top left is the k-outer panel; the
+// other rows of its columns and then the other columns follow tile by tile (orient 1: the other columns of its rows,
+// then the other rows).  Its C tiles are complete after (rows + columns) * Kg fetched tiles instead of (Mg + w) * Kg,
+// so write-backs start earlier: for shapes bounded by the link (dgemm 8192^3 from the host: 24.7 -> 23.3 ms).
+constexpr int ORDER_BLOCK_ROWS = 100;
 // + 160000 * s: thin start (GemmProblem::k_split) with 2^s slabs, s = 1 or 2.
 constexpr int ORDER_K_SPLIT = 160000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }

@@ -85,6 +85,13 @@ struct Resources {
   int rotation = 0;
   int trials = 0;            // rotations tried so far; 4 = settled
   double trial_rate[4] = {0, 0, 0, 0};
+  // The four trial calls are calls of ONE problem (rates of different shapes do not compare), and the more of a call's
+  // time the tile kernels take, the better its time tells the alignments apart: a call bounded by the link runs nearly
+  // the same under all four, and a choice made on such a call is a draw.  So the trial is run again when a problem
+  // comes along whose predicted compute share is clearly higher than that of the problem the last trial ran on.
+  bool rotation_pinned = false;       // PARALIA_STREAM_ROTATION: never tried, never changed
+  const void* trial_problem = nullptr;
+  double trial_weight = -1;           // predicted compute share of trial_problem
   void set_rotation(int r) {
     rotation = r;
     h2d = ring[r];
@@ -100,6 +107,7 @@ struct Resources {
       if (env && atoi(env) >= 0 && atoi(env) < 4) {
         set_rotation(atoi(env));
         trials = 4;
+        rotation_pinned = true;
       } else {
         set_rotation(trials >= 4 ? rotation : 0);  // a choice made before a teardown holds for the new ring
       }
@@ -194,9 +202,11 @@ struct Resources {
     stager_.reset();
     const int keep_rotation = rotation, keep_trials = trials;
     const bool keep_trace = trace_on;
+    const double keep_weight = trial_weight;
     *this = Resources();
     rotation = keep_rotation;
-    trials = keep_trials;
+    trials = keep_trials >= 4 ? 4 : 0;   // a trial in progress starts over on the new ring
+    trial_weight = keep_trials >= 4 ? keep_weight : -1;
     trace_on = keep_trace;
   }
 };
@@ -227,6 +237,7 @@ struct PMDEntry {
   PMDKey key;
   std::unique_ptr<ATC> atc;
   GemmPlan plan;
+  long calls = 0;  // calls served from this entry
 };
 
 struct Runtime {
@@ -465,7 +476,6 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   PMDEntry* entry = nullptr;
   for (auto& e : R.pmd)
     if (e->key == key) { entry = e.get(); break; }
-  const bool cold = entry == nullptr;
   if (entry) ++R.pmd_hits;
   else {
     ++R.pmd_misses;
@@ -532,14 +542,24 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     const GemmPlan& plan = entry->plan;
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T), atc->cache_limit);
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
-    // a first call of a problem also pays for fresh pool memory and cold caches: it would misjudge its rotation
-    const bool trial = R.res.trials < 4 && plan.cmds.size() >= 64 && !no_ab && !cold;
+    // the first two calls of a problem also pay for fresh pool memory and cold caches (the second still runs a few
+    // percent slow): a trial that started there would misjudge its first rotation
+    const bool eligible = !R.res.rotation_pinned && plan.cmds.size() >= 64 && !no_ab && entry->calls >= 2;
+    const double weight = atc->pred_t > 0 ? atc->pipeline.t_exec_busy / atc->pred_t : 0;
+    if (eligible && entry != R.res.trial_problem &&
+        (R.res.trials >= 4 ? weight > R.res.trial_weight + 0.15 : weight >= R.res.trial_weight)) {
+      R.res.trials = 0;               // settled on a less compute-bound problem, or that problem's calls stopped coming
+      R.res.trial_problem = entry;
+      R.res.trial_weight = weight;
+    }
+    const bool trial = eligible && R.res.trials < 4 && entry == R.res.trial_problem;
     if (trial) R.res.begin_trial();
     const double t0 = csecond();
     const bool pageable[3] = {locA == -2, locB == -2, locC == -2};
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC, pageable);
     if (trial) R.res.end_trial((csecond() - t0) / (2.0 * M * N * (double)K));
   }
+  ++entry->calls;
   return atc_copy(atc);
 }
 

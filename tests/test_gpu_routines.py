@@ -443,7 +443,7 @@ def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg,
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
-@pytest.mark.parametrize("order", [80000, 80002, 90003, 160002, 320003, 240002, 330000])
+@pytest.mark.parametrize("order", [80000, 80002, 90003, 160002, 320003, 240002, 330000, 304, 10403, 80405, 250302])
 @pytest.mark.parametrize("locs", [(-1, -1, -1), (-1, -1, 0), (-2, -2, -1), (0, -1, -1)])
 def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs, monkeypatch):
     """Order ids of 80000 and above: the k tiles of every A row panel and B column panel lie side by side on the device
@@ -453,9 +453,10 @@ def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs
     pageable or already on the device, beta = 0 over NaN and beta != 0 (fetched C, lazy reduce): bit for bit the
     untiled result, in fp64 and fp32.  Order ids of 160000 and above add the thin start: the first k tile is cut into 2
     (160000 +) or 4 (320000 +) slabs that are fetched and multiplied as k tiles of their own (7 or 9 k tiles here), alone
-    or together with merged chains (240002)."""
+    or together with merged chains (240002).  Orders whose width is rows * 100 + columns (304, 10403, with merged chains
+    80405, with all three 250302) start with that block of C tiles as the k-outer panel and finish tile by tile."""
     monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
-    orders = [80000, 80002, 90003, 160002, 320003, 240002, 330000]
+    orders = [80000, 80002, 90003, 160002, 320003, 240002, 330000, 304, 10403, 80405, 250302]
     M, N, K, T = 289, 353, 307 + orders.index(order), 64   # a new problem for the metadata cache per order
     ra, ca = (M, K) if ta == "N" else (K, M)
     rb, cb = (K, N) if tb == "N" else (N, K)

@@ -159,7 +159,7 @@ def check_async_safety(rows):
             users[blk] = []
 
 
-ORDERS = [10000, 0, 1, 3, 10002, 10004, 20002, 30001, 50000, 60002]
+ORDERS = [10000, 0, 1, 3, 10002, 10004, 20002, 30001, 50000, 60002, 102, 201, 202, 10201, 10999]
 
 
 @pytest.mark.parametrize("order", ORDERS)
@@ -333,6 +333,8 @@ def test_random_plans_are_safe_and_correct(pkg, seed):
     pool = int(rng.choice([0, 3, 4, 5, max(3, full // 3), max(3, full // 2), full]))
     orient, w = int(rng.integers(0, 2)), int(rng.integers(0, max(Mg, Ng) + 2))
     order = orient * 10000 + w + (20000 if w > 0 and rng.integers(0, 2) else 0) + (40000 if rng.integers(0, 2) else 0)
+    if seed % 5 == 4:   # a block order: rows * 100 + columns, plain or with the other eviction policy
+        order = orient * 10000 + int(rng.integers(1, Mg + 2)) * 100 + int(rng.integers(1, Ng + 2)) + (40000 if rng.integers(0, 2) else 0)
     A = rng.integers(-4, 5, (M, K)).astype(np.float64)
     B = rng.integers(-4, 5, (K, N)).astype(np.float64)
     C = rng.integers(-4, 5, (M, N)).astype(np.float64)
@@ -451,6 +453,45 @@ def test_thin_start_plans(pkg, order, locs, beta_zero):
     check_async_safety(flat)
     with pytest.raises(pkg.ParaliaError, match="thin start"):
         pkg.plan_rows(M, N, 20, 32, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)     # K < T: nothing to cut
+
+
+def test_block_orders(pkg):
+    """w = rows * 100 + columns: that block of C tiles is the k-outer panel (walked in growing squares in every k-step),
+    the rest follows tile by tile with the K chain innermost -- for orient 0 the other rows of the block's columns, then
+    the other columns."""
+    M = N = K = 4 * 64
+    rows, _ = pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, 302)
+    g = [(r["mi"], r["ni"], r["ki"]) for r in rows if r["kind"] == GEMM]
+    block = [(0, 0), (0, 1), (1, 0), (1, 1), (2, 0), (2, 1)]
+    assert g[:24] == [(mi, ni, ki) for ki in range(4) for (mi, ni) in block]
+    assert g[24:32] == [(3, ni, ki) for ni in range(2) for ki in range(4)]
+    assert g[32:] == [(mi, ni, ki) for ni in (2, 3) for mi in range(4) for ki in range(4)]
+    rows, _ = pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, 10302)
+    g = [(r["mi"], r["ni"], r["ki"]) for r in rows if r["kind"] == GEMM]
+    assert g[24:48] == [(mi, ni, ki) for ni in (2, 3) for mi in range(3) for ki in range(4)]
+    assert g[48:] == [(3, ni, ki) for ni in range(4) for ki in range(4)]
+    # the first C tile goes back after three k-steps of the block (3 + 2 tiles each) and two tiles of the last one; a
+    # panel over all rows needs 4 + 2 tiles per k-step
+    def fetched_before_first_writeback(plan_rows):
+        n_fetch = 0
+        for r in plan_rows:
+            if r["kind"] in (FETCH_A, FETCH_B):
+                n_fetch += 1
+            if r["kind"] == WRITEBACK:
+                break
+        return n_fetch
+    assert fetched_before_first_writeback(rows) == 3 * 5 + 2
+    assert fetched_before_first_writeback(pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, 2)[0]) == 3 * 6 + 2
+    # a block larger than the grid is the grid; repeated panels have no block form; zero columns is no order
+    rows, stats = pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, 9999)
+    check_plan(rows, stats, M, N, K, 64, 1, 1, 1, 1, 1 << 20, 2)
+    for order in (20302, 300):
+        with pytest.raises(pkg.ParaliaError, match="unknown order id"):
+            pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, order)
+    # merged chains and thin start combine with it
+    for order in (80302, 160302, 240302):
+        rows, stats = pkg.plan_rows(M, N, K, 64, 1, 1, 1, 1, 8, 2, 0, order)
+        assert stats[5] == 4 * 4 * (4 if order < 160000 else 5)
 
 
 def test_unknown_order_ids_are_refused(pkg):
