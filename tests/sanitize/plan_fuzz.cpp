@@ -29,7 +29,9 @@ int main(int argc, char** argv) {
       if (rng() % 4 == 0) {
         PipelineResult r; pick_gemm_order(p, st, &r, rng() % 2);
       } else {
-        const int orient = rng() % 2, w = rng() % 40;
+        const int orient = rng() % 2;
+        // panel widths, and now and then a block order (rows * 100 + columns; zero columns and repeated panels are refused)
+        const int w = (rng() % 4 == 0) ? (int)((1 + rng() % 30) * ORDER_BLOCK_ROWS + rng() % 30) : (int)(rng() % 40);
         int id = orient * 10000 + w + ((w > 0 && rng() % 2) ? 20000 : 0) + ((rng() % 2) ? 40000 : 0);
         if (rng() % 3 == 0) id = ORDER_MERGE_CHAINS + orient * 10000 + w;  // merged K chains (refused unless the pool holds everything)
         if (rng() % 3 == 0) id += ORDER_K_SPLIT * (1 + rng() % 2);  // thin start: first k tile in 2 or 4 slabs (refused when it does not apply)
