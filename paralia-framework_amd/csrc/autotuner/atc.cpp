@@ -301,6 +301,8 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.merge_saving = paralia_merge_saving(d, T);
   const char* thin = getenv("PARALIA_THIN_START");  // "0": never cut the first k tile into slabs
   st.thin_start = !(thin && *thin && atoi(thin) == 0);
+  const char* blk = getenv("PARALIA_BLOCK_ORDERS");  // "0": never start with a block of C tiles smaller than a full panel
+  st.block_orders = !(blk && *blk && atoi(blk) == 0);
   return st;
 }
 

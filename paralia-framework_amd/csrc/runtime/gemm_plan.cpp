@@ -595,6 +595,7 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   auto is_block = [](int id) { return id % 10000 >= ORDER_BLOCK_ROWS; };
   std::string last_err;
   for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0)) {
+    if (is_block(id) && !st.block_orders) continue;
     try {
       GemmPlan plan = build_gemm_plan(p, id);
       PipelineResult r = simulate_plan(plan, st);

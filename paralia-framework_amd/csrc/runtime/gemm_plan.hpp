@@ -131,6 +131,7 @@ struct StageTimes {
   // (0: merging K chains is not worth considering for this kernel)
   double merge_saving = 0;
   bool thin_start = true;            // offer the thin start (order ids of 160000 and above) to the order search
+  bool block_orders = true;          // offer the block orders (w >= ORDER_BLOCK_ROWS) to the order search
   // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch
   double slab_fixed = 2e-6;  // measured: 2048 x 2048 x 1024 119.9 us, x 512 61.2 us against 236.7 us for the whole tile
 };

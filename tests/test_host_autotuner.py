@@ -305,3 +305,23 @@ def test_limited_pool_probe_keeps_the_tile_whose_best_panel_width_just_fits(L, p
             best = (T, info.pred_t)
     L.PARALiA_set_db_dir(None)
     assert picked_T == best[0] == 2048 and abs(picked_t - best[1]) <= 1e-9 * best[1]
+
+
+def test_block_orders_are_taken_for_link_bound_shapes_and_can_be_switched_off(L, pkg, monkeypatch):
+    """dgemm 8192^3 from the host (H2D 19.3 ms against 15 ms of tile kernels): the planner starts with a 3 x 3 block of the
+    4 x 4 C tiles (order 303) and predicts more than 1 % less than without block orders; 16384^3, bound by compute, keeps
+    its panel order; PARALIA_BLOCK_ORDERS=0 takes the family out of the search."""
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    d = _shipped_db(pkg).encode()
+    info = pkg.atc_info()
+    monkeypatch.setenv("PARALIA_BLOCK_ORDERS", "0")
+    assert L.PARALiA_autotune(d, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 2048, 0, C.byref(info)) == 0
+    assert info.order_id % 10000 < 100
+    t_panel = info.pred_t
+    monkeypatch.delenv("PARALIA_BLOCK_ORDERS")
+    assert L.PARALiA_autotune(d, b"Dgemm", 8192, 8192, 8192, b"N", b"N", HOST3, 1, 2048, 0, C.byref(info)) == 0
+    assert info.order_id % 10000 == 303 and info.pred_t < 0.99 * t_panel
+    assert L.PARALiA_autotune(d, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, 2048, 0, C.byref(info)) == 0
+    assert info.order_id % 10000 < 100
+    L.PARALiA_set_db_dir(None)
