@@ -103,6 +103,10 @@ typedef class Modeler {
   comm_data* revlink[LOC_NUM];  // transfers from this unit to location idx     (Modeler.cpp:27)
   GPUexecModel* exec = nullptr;
   int unit_id = 0;
+  // Power-state transient of the unit (Processed/Power-transient_dev-<id>.log, optional, not a table of the reference):
+  // after its compute units sat idle a tile kernel takes up to (1 + amplitude) times its steady time; the deficit grows
+  // with time constant idle_s while nothing runs and decays with recover_s while kernels do.  amplitude 0: not measured.
+  double transient_amplitude = 0, transient_idle_s = 0, transient_recover_s = 0;
   Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc);
   ~Modeler();
   long getMinT() const;

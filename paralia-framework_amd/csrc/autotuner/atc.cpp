@@ -301,6 +301,11 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.merge_saving = paralia_merge_saving(d, T);
   const char* thin = getenv("PARALIA_THIN_START");  // "0": never cut the first k tile into slabs
   st.thin_start = !(thin && *thin && atoi(thin) == 0);
+  if (d.problem == BLAS3 && m->transient_amplitude > 0) {
+    st.tr_amp = m->transient_amplitude;
+    st.tr_idle = m->transient_idle_s;
+    st.tr_recover = m->transient_recover_s;
+  }
   const char* blk = getenv("PARALIA_BLOCK_ORDERS");  // "0": never start with a block of C tiles smaller than a full panel
   st.block_orders = !(blk && *blk && atoi(blk) == 0);
   return st;

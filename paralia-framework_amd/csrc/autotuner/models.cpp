@@ -3,6 +3,7 @@
 // :287-346 (baseline), :348-408 (data location), :410-474 (bidirectional), :476-551 (reuse) and
 // ModelLvl1.cpp:262-326 (BLAS-1 bidirectional), ModelLvl2.cpp:89-259 (BLAS-2: full / zero overlap and bidirectional),
 // reduced to one GPU plus the host.
+#include <cstdio>
 #include <cmath>
 #include <cstring>
 
@@ -20,6 +21,17 @@ Modeler::Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc)
     }
   }
   exec = GPUexecModel_init(db_dir, dev_id, desc.func);
+  char filename[1024];
+  snprintf(filename, sizeof filename, "%s/Processed/Power-transient_dev-%d.log", db_dir.c_str(), dev_id);
+  if (FILE* fp = fopen(filename, "r")) {
+    double a = 0, rec = 0, idle = 0;
+    if (fscanf(fp, "Amplitude: %lf\nRecovery: %lf\nIdle: %lf", &a, &rec, &idle) == 3 && a > 0 && a < 1 && rec > 0 && idle > 0) {
+      transient_amplitude = a;
+      transient_recover_s = rec;
+      transient_idle_s = idle;
+    }
+    fclose(fp);
+  }
 }
 
 Modeler::~Modeler() {

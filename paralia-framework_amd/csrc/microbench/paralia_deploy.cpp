@@ -4,7 +4,8 @@
 //
 // Measures (1) the tile GEMM kernels over square T for the four transpose combinations, fp64 and fp32,
 // (2) daxpy / ddot over vector lengths and dgemv over square T for both transposes, (3) pinned-host <-> device 2-D tile copies in both directions and the
-// slowdown of each direction while the other is busy; writes the raw logs to <db_dir>/Benchmark-Results and the
+// slowdown of each direction while the other is busy, (4) the power-state transient of the tile kernels after idle time;
+// writes the raw logs to <db_dir>/Benchmark-Results and the
 // tables the autotuner reads to <db_dir>/Processed.
 //
 // What it re-does from the reference: Database_builder/CuCuBLAS/src/dgemm_microbench.cu:26-230 (T sweep from
@@ -287,6 +288,84 @@ static void bench_blas1(const std::string& db, const char* func, bool quick) {
   CoCoFree(x, 0); CoCoFree(y, 0); CoCoFree(ws, 0);
 }
 
+// The device's power-state transient, as the tile kernels see it: pairs of 2048^3 fp64 launches on two streams, 100 pairs
+// back to back (the first burst brings the device to its steady state), then after a host-side gap of 5 and of 20 ms
+// without kernels another 100, every pair timed with events.  Against the steady pair time of a burst's last 40 pairs a
+// burst after a gap loses L(gap) seconds in its first 60 pairs, the slowest pair being (1 + amplitude) x steady.  With
+// the deficit decaying exponentially while kernels run, L(20 ms) = amplitude x recovery constant; with it growing as
+// 1 - exp(-gap / idle constant) while none run, L(5 ms) / L(20 ms) gives the idle constant.  Three repetitions, medians.
+// Written to Processed/Power-transient_dev-0.log (seconds); not a file of the reference.
+static void bench_transient(const std::string& db) {
+  const long Tt = 2048;
+  const int pairs = 100;
+  double *A, *B, *C;
+  A = (double*)CoCoMalloc(Tt * Tt * sizeof(double), 0, 0);
+  B = (double*)CoCoMalloc(Tt * Tt * sizeof(double), 0, 0);
+  C = (double*)CoCoMalloc(2 * Tt * Tt * sizeof(double), 0, 1);
+  CoCoVecInit(A, Tt * Tt, 42, 0);
+  CoCoVecInit(B, Tt * Tt, 43, 0);
+  CoCoVecInit(C, 2 * Tt * Tt, 44, 0);
+  void* st[2];
+  for (auto& s : st) must(pl_stream_create(&s), "stream");
+  std::vector<void*> ev(pairs + 1);
+  for (auto& e : ev) must(pl_event_create(&e, 1), "event");
+  auto burst = [&](std::vector<double>& t) {
+    must(pl_event_record(ev[0], st[0]), "record");
+    for (int i = 0; i < pairs; ++i) {
+      for (int q = 0; q < 2; ++q)
+        must(pl_dgemm_tile_ws('N', 'N', Tt, Tt, Tt, 1e-9, A, Tt, B, Tt, 1.0, C + (long)q * Tt * Tt, Tt, nullptr, 0, st[q]), "gemm");
+      must(pl_event_record(ev[i + 1], st[0]), "record");
+    }
+    for (auto s : st) must(pl_stream_sync(s), "sync");
+    t.resize(pairs);
+    for (int i = 0; i < pairs; ++i) {
+      float ms = 0;
+      must(pl_event_elapsed_ms(ev[i], ev[i + 1], &ms), "elapsed");
+      t[i] = ms * 1e-3;
+    }
+  };
+  auto median3 = [](double a, double b, double c) { return std::max(std::min(a, b), std::min(std::max(a, b), c)); };
+  const double gaps[2] = {5e-3, 20e-3};
+  double loss[2][3], peak[3], steady_t = 0;
+  std::vector<double> t;
+  for (int rep = 0; rep < 3; ++rep)
+    for (int g = 0; g < 2; ++g) {
+      burst(t);  // warm: whatever came before, the device is in its steady state afterwards
+      const double t0 = csecond();
+      while (csecond() - t0 < gaps[g]) {
+      }
+      burst(t);
+      double steady = 0;
+      for (int i = 60; i < pairs; ++i) steady += t[i] / (pairs - 60);
+      double l = 0, p = 0;
+      for (int i = 0; i < 60; ++i) l += t[i] - steady;
+      for (int i = 0; i < 20; ++i) p = std::max(p, t[i] / steady - 1.0);
+      loss[g][rep] = std::max(l, 0.0);
+      if (g == 1) { peak[rep] = p; steady_t = steady; }
+    }
+  const double l5 = median3(loss[0][0], loss[0][1], loss[0][2]), l20 = median3(loss[1][0], loss[1][1], loss[1][2]);
+  double amp = median3(peak[0], peak[1], peak[2]);
+  double recover = 0, idle = 0;
+  if (amp < 0.02 || l20 <= 0) {
+    amp = 0;  // nothing to model on this device
+  } else {
+    recover = l20 / amp;
+    const double frac = std::min(0.95, std::max(0.05, l5 / l20));
+    idle = -gaps[0] / log(1.0 - frac);
+  }
+  char out[1024];
+  snprintf(out, sizeof out, "%s/Processed/Power-transient_dev-0.log", db.c_str());
+  FILE* fp = fopen(out, "w");
+  if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  fprintf(fp, "Amplitude: %e\nRecovery: %e\nIdle: %e\n", amp, recover, idle);
+  fclose(fp);
+  fprintf(stderr, "power transient: steady pair %.3f ms, after 5 / 20 ms idle %.2f / %.2f ms lost, slowest pair +%.1f %% -> recovery %.1f ms, idle %.1f ms\n",
+          steady_t * 1e3, l5 * 1e3, l20 * 1e3, amp * 100, recover * 1e3, idle * 1e3);
+  for (auto e : ev) pl_event_destroy(e);
+  for (auto s : st) pl_stream_destroy(s);
+  CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
+}
+
 static void bench_link(const std::string& db, bool quick) {
   const long maxDim = quick ? 4352 : 10000;
   std::vector<long> dims = sweep(256, 256, maxDim, 8);
@@ -406,6 +485,7 @@ int main(int argc, char** argv) {
     if (only.empty() || only == "gemm") {
       bench_gemm<double>(db, "Dgemm", quick, queues);
       bench_gemm<float>(db, "Sgemm", quick, queues);
+      bench_transient(db);
     }
     if (only.empty() || only == "gemv") bench_gemv(db, quick);
     if (only.empty() || only == "blas1") {

@@ -538,6 +538,7 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
     size_t cur_h2d = 0, cur_d2h = 0;
     double h2d = 0, d2h = 0, exec = 0;
     double qclock[MAX_EXEC_QUEUES] = {0};
+    double deficit = st.tr_amp > 0 ? 1.0 - std::exp(-st.tr_gap0 / st.tr_idle) : 0.0;
     r = PipelineResult();
     for (size_t i = 0; i < plan.cmds.size(); ++i) {
       const Cmd& c = plan.cmds[i];
@@ -572,6 +573,11 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
         // exec queues are in-order each and share the one compute resource
         const int q = c.stream - STREAM_EXEC0;
         const double s = std::max(std::max(ready, qclock[q]), exec);
+        if (st.tr_amp > 0) {
+          if (s > exec) deficit = 1.0 - (1.0 - deficit) * std::exp(-(s - exec) / st.tr_idle);
+          if (c.kind == CMD_GEMM) dur *= 1.0 + st.tr_amp * deficit;
+          deficit *= std::exp(-dur / st.tr_recover);
+        }
         finish[i] = qclock[q] = exec = s + dur;
         r.t_exec += dur;
       }

@@ -131,6 +131,11 @@ struct StageTimes {
   // (0: merging K chains is not worth considering for this kernel)
   double merge_saving = 0;
   bool thin_start = true;            // offer the thin start (order ids of 160000 and above) to the order search
+  // Power-state transient of the device: after the compute units sat idle, tile kernels start slower and recover while
+  // they run.  deficit in [0, 1] grows towards 1 with time constant tr_idle while no kernel runs and decays with
+  // tr_recover while one does; a tile kernel takes (1 + tr_amp * deficit) times its steady time.  tr_amp = 0: not modelled.
+  double tr_amp = 0, tr_idle = 6e-3, tr_recover = 8e-3;
+  double tr_gap0 = 1e-3;             // idle time assumed in front of the call (calls made back to back)
   bool block_orders = true;          // offer the block orders (w >= ORDER_BLOCK_ROWS) to the order search
   // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch
   double slab_fixed = 2e-6;  // measured: 2048 x 2048 x 1024 119.9 us, x 512 61.2 us against 236.7 us for the whole tile

@@ -109,12 +109,13 @@ struct Resources {
         trials = 4;
         rotation_pinned = true;
       } else {
-        set_rotation(trials >= 4 ? rotation : 0);  // a choice made before a teardown holds for the new ring
+        set_rotation(rotation);  // 0 in a new process; after a teardown what was in use (or chosen) before it
       }
     }
     for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
   }
   // Called around a large streamed GEMM: picks the rotation to try, then records seconds per flop.
+  int settled_rotation = 0;  // what the last finished trial chose (0 before any)
   void begin_trial() {
     if (trials < 4) set_rotation(trials);
   }
@@ -122,9 +123,12 @@ struct Resources {
     if (trials >= 4) return;
     trial_rate[trials++] = seconds_per_flop;
     if (trials == 4) {
-      int best = 0;
-      for (int r = 1; r < 4; ++r)
-        if (trial_rate[r] < trial_rate[best]) best = r;
+      // the alignment in use so far stays unless another one is faster by more than the noise of a single call (2 %):
+      // on a call the link bounds all four measure alike, and the winner of such a draw can cost the next problem 7 %
+      int best = settled_rotation;
+      for (int r = 0; r < 4; ++r)
+        if (trial_rate[r] < 0.98 * trial_rate[settled_rotation] && trial_rate[r] < trial_rate[best]) best = r;
+      settled_rotation = best;
       set_rotation(best);
     }
   }
@@ -200,11 +204,12 @@ struct Resources {
     gemv_x.release(); gemv_y.release(); gemv_ws.release();
     for (Scratch& w : gemm_ws) w.release();
     stager_.reset();
-    const int keep_rotation = rotation, keep_trials = trials;
+    const int keep_rotation = rotation, keep_trials = trials, keep_settled = settled_rotation;
     const bool keep_trace = trace_on;
     const double keep_weight = trial_weight;
     *this = Resources();
-    rotation = keep_rotation;
+    rotation = keep_trials >= 4 ? keep_rotation : keep_settled;
+    settled_rotation = keep_settled;
     trials = keep_trials >= 4 ? 4 : 0;   // a trial in progress starts over on the new ring
     trial_weight = keep_trials >= 4 ? keep_weight : -1;
     trace_on = keep_trace;

@@ -207,6 +207,13 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
     close(lone[("N", "N", "2048")], lone_shipped[("N", "N", "2048")], 0.10, "lone 2048^3 fp64 launch")
     ratio = lone[("N", "N", "2048")] / _table(os.path.join(fresh, names[0]), 5)[("N", "N", "2048", "2048", "2048")]
     assert 1.03 < ratio < 1.25, ratio
+    # the power-state transient of the tile kernels: present on this device, its constants of the shipped file's order
+    def transient(path):
+        return {k.strip(): float(v) for k, v in (line.split(":") for line in open(path))}
+    tr, tr_shipped = transient(os.path.join(fresh, "Power-transient_dev-0.log")), transient(os.path.join(shipped, "Power-transient_dev-0.log"))
+    assert 0.1 < tr["Amplitude"] < 0.5, tr
+    for k in ("Amplitude", "Recovery", "Idle"):
+        assert 0.4 * tr_shipped[k] < tr[k] < 2.5 * tr_shipped[k], (k, tr, tr_shipped)
     # matrix-vector and vector kernels take 40 - 80 us at the largest sizes of the quick sweep: launch and
     # synchronisation are a visible part of that, and working sets of 128 - 384 MiB sit partly inside the memory-side
     # cache, so these differ more between machines than the millisecond-scale GEMM tiles: a wider band

@@ -325,3 +325,37 @@ def test_block_orders_are_taken_for_link_bound_shapes_and_can_be_switched_off(L,
     assert L.PARALiA_autotune(d, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, 2048, 0, C.byref(info)) == 0
     assert info.order_id % 10000 < 100
     L.PARALiA_set_db_dir(None)
+
+
+def test_power_transient_file_is_optional_and_prices_sparse_starts(L, pkg, tmp_path, monkeypatch):
+    """Processed/Power-transient_dev-0.log (Amplitude / Recovery / Idle, measured by the deploy tool; not a file of the
+    reference): without it the simulator prices every tile kernel at its steady time.  With it a kernel that starts after
+    idle time takes up to (1 + amplitude) times as long, so (1) the compute-bound 16384^3 call, which keeps the device
+    busy from its first millisecond, gets longer by a fraction of amplitude x recovery at most; (2) for 12288 x 6144 x
+    6144, where the one-row panels the plain model picks leave the kernels idle for the first 8 ms (all of B is
+    fetched for the first row of C), another order wins; (3) a file with nonsense in it is ignored."""
+    import shutil
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    monkeypatch.delenv("PARALIA_T_SELECT", raising=False)
+    shipped = _shipped_db(pkg)
+    vals = {}
+    for line in open(os.path.join(shipped, "Processed", "Power-transient_dev-0.log")):
+        k, v = line.split(":")
+        vals[k.strip()] = float(v)
+    assert 0.05 < vals["Amplitude"] < 0.6 and 1e-3 < vals["Recovery"] < 5e-2 and 1e-3 < vals["Idle"] < 5e-2
+    bare, junk = tmp_path / "bare", tmp_path / "junk"
+    shutil.copytree(shipped, bare)
+    os.remove(bare / "Processed" / "Power-transient_dev-0.log")
+    shutil.copytree(shipped, junk)
+    (junk / "Processed" / "Power-transient_dev-0.log").write_text("Amplitude: 5.0\nRecovery: -1\nIdle: 0\n")
+    info = pkg.atc_info()
+    res = {}
+    for name, d in (("with", shipped), ("bare", str(bare)), ("junk", str(junk))):
+        for shape in ((16384, 16384, 16384), (12288, 6144, 6144)):
+            assert L.PARALiA_autotune(d.encode(), b"Dgemm", *shape, b"N", b"N", HOST3, 1, 2048, 0, C.byref(info)) == 0
+            res[(name, shape[1])] = (info.order_id, info.pred_t)
+    L.PARALiA_set_db_dir(None)
+    assert res[("junk", 16384)] == res[("bare", 16384)] and res[("junk", 6144)] == res[("bare", 6144)]
+    rise = res[("with", 16384)][1] - res[("bare", 16384)][1]
+    assert 0 < rise < 0.25 * vals["Amplitude"] * vals["Recovery"]
+    assert res[("with", 6144)][0] != res[("bare", 6144)][0] and res[("with", 6144)][1] > res[("bare", 6144)][1]
