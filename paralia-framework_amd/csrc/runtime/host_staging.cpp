@@ -15,6 +15,19 @@ namespace {
 void chk(int rc, const char* what) {
   if (rc != 0) throw paralia_error(rc, std::string(what) + " failed: " + (rc == PL_ERR_HIP ? pl_last_error() : "invalid argument"));
 }
+// A dense block of `cols` columns of `rows` elements between a pinned slot and the device, through the 2-D copy call (on
+// a stream of the 1-D call a copy was seen to start only when the copy running on the opposite-direction stream had
+// finished).  One long column (a vector span) goes as columns of 64 KiB plus a short tail.
+void dense_copy_async(void* dst, const void* src, long rows, long cols, int elem, void* stream) {
+  if (cols > 1) {
+    chk(pl_copy2d_async(dst, rows, src, rows, rows, cols, elem, stream), "staged tile copy");
+    return;
+  }
+  const long long bytes = (long long)rows * elem, col = 65536, n = bytes / col, done = n * col;
+  if (n > 0) chk(pl_copy2d_async(dst, col, src, col, col, n, 1, stream), "staged tile copy");
+  if (bytes > done)
+    chk(pl_copy2d_async((char*)dst + done, bytes - done, (const char*)src + done, bytes - done, bytes - done, 1, 1, stream), "staged tile copy");
+}
 }  // namespace
 
 CopyThreads::CopyThreads(int nthreads) {
@@ -93,6 +106,15 @@ void CopyThreads::copy2d(void* dst, size_t dst_pitch, const void* src, size_t sr
 
 HostStager::~HostStager() {
   try { release(); } catch (...) {}
+  if (deferred_.joinable()) {
+    {
+      std::lock_guard<std::mutex> lk(dmu_);
+      stop_ = true;
+    }
+    dcv_.notify_all();
+    deferred_.join();
+  }
+  delete deferred_pool_;
   delete pool_;
 }
 
@@ -106,6 +128,7 @@ CopyThreads* HostStager::threads() {
 }
 
 void HostStager::release() {
+  abandon();  // deferred write-backs still open belong to a call that is over
   for (int s = 0; s < SLOTS; ++s) {
     if (in_[s]) pl_free_pinned(in_[s]);
     if (out_[s]) pl_free_pinned(out_[s]);
@@ -144,7 +167,7 @@ void HostStager::fetch(void* dst, const void* src, long ld_src, long rows, long 
   const int s = (int)(in_next_++ % SLOTS);
   if (in_used_[s]) chk(pl_event_sync(in_ev_[s]), "event sync");  // the slot's previous tile has left for the device
   threads()->copy2d(in_[s], (size_t)rows * elem, src, (size_t)ld_src * elem, (size_t)rows * elem, cols);
-  if (ld_dst <= 0 || ld_dst == rows) chk(pl_copy_async(dst, in_[s], bytes, stream), "staged tile copy");
+  if (ld_dst <= 0 || ld_dst == rows) dense_copy_async(dst, in_[s], rows, cols, elem, stream);
   else chk(pl_copy2d_async(dst, ld_dst, in_[s], rows, rows, cols, elem, stream), "staged tile copy");
   chk(pl_event_record(in_ev_[s], stream), "event record");
   in_used_[s] = true;
@@ -164,17 +187,101 @@ void HostStager::write_back(void* dst, long ld_dst, const void* src, long rows, 
   reserve(bytes);
   const int s = (int)(out_next_++ % SLOTS);
   flush(s);
-  chk(pl_copy_async(out_[s], src, bytes, stream), "staged tile copy");
+  dense_copy_async(out_[s], src, rows, cols, elem, stream);
   chk(pl_event_record(out_ev_[s], stream), "event record");
   Pending& p = pending_[s];
   p.dst = dst; p.ld = ld_dst; p.rows = rows; p.cols = cols; p.elem = elem; p.active = true;
 }
 
+void HostStager::write_back_deferred(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream,
+                                     void* const* after, int n_after) {
+  if (rows <= 0 || cols <= 0) return;
+  reserve((long long)rows * cols * elem);
+  Request r{dst, ld_dst, src, rows, cols, elem, stream, {nullptr}, std::min(n_after, 12)};
+  for (int i = 0; i < r.n_after; ++i) r.after[i] = after[i];
+  {
+    std::lock_guard<std::mutex> lk(dmu_);
+    if (!deferred_.joinable()) {
+      // two threads scatter a 32 MiB tile in 0.85 ms against 0.6 ms on the link; the cores stay with the gathers
+      deferred_pool_ = new CopyThreads(2);
+      deferred_ = std::thread([this] { deferred_loop(); });
+    }
+    requests_.push_back(r);
+    ++open_;
+  }
+  dcv_.notify_all();
+}
+
+// The background thread: keeps up to SLOTS copies on the stream, scatters the oldest when it has arrived.
+void HostStager::deferred_loop() {
+  struct Flight { int slot; Request r; };
+  std::deque<Flight> flying;
+  int next_slot = 0;
+  std::unique_lock<std::mutex> lk(dmu_);
+  for (;;) {
+    dcv_.wait(lk, [&] { return stop_ || !requests_.empty() || !flying.empty(); });
+    if (stop_ && requests_.empty() && flying.empty()) return;
+    const bool drop = dropping_ || error_ != nullptr;
+    std::exception_ptr err;
+    // enqueue copies while slots are free
+    while (!requests_.empty() && (int)flying.size() < SLOTS) {
+      Flight f{next_slot, requests_.front()};
+      requests_.pop_front();
+      next_slot = (next_slot + 1) % SLOTS;
+      if (!drop && !err) {
+        lk.unlock();
+        try {
+          for (int i = 0; i < f.r.n_after; ++i) chk(pl_stream_wait_event(f.r.stream, f.r.after[i]), "stream wait event");
+          dense_copy_async(out_[f.slot], f.r.src, f.r.rows, f.r.cols, f.r.elem, f.r.stream);
+          chk(pl_event_record(out_ev_[f.slot], f.r.stream), "event record");
+        } catch (...) {
+          err = std::current_exception();
+        }
+        lk.lock();
+      }
+      if (drop || err) { --open_; continue; }  // never enqueued: nothing to wait for
+      flying.push_back(f);
+    }
+    // the oldest copy: wait for it, scatter it
+    if (!flying.empty()) {
+      const Flight f = flying.front();
+      flying.pop_front();
+      lk.unlock();
+      try {
+        chk(pl_event_sync(out_ev_[f.slot]), "event sync");
+        if (!drop && !err)
+          deferred_pool_->copy2d(f.r.dst, (size_t)f.r.ld * f.r.elem, out_[f.slot], (size_t)f.r.rows * f.r.elem, (size_t)f.r.rows * f.r.elem, f.r.cols);
+      } catch (...) {
+        if (!err) err = std::current_exception();
+      }
+      lk.lock();
+      --open_;
+    }
+    if (err && !error_) error_ = err;
+    dcv_.notify_all();
+  }
+}
+
 void HostStager::abandon() {
   for (int s = 0; s < SLOTS; ++s) pending_[s].active = false;
+  std::unique_lock<std::mutex> lk(dmu_);
+  dropping_ = true;
+  dcv_.notify_all();
+  dcv_.wait(lk, [&] { return open_ == 0; });
+  dropping_ = false;
+  error_ = nullptr;
 }
 
 void HostStager::finish() {
+  {
+    std::unique_lock<std::mutex> lk(dmu_);
+    dcv_.wait(lk, [&] { return open_ == 0; });
+    if (error_) {
+      std::exception_ptr e = error_;
+      error_ = nullptr;
+      std::rethrow_exception(e);
+    }
+  }
   for (int i = 0; i < SLOTS; ++i) flush((int)((out_next_ + i) % SLOTS));  // oldest first
 }
 

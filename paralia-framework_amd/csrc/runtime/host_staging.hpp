@@ -12,6 +12,8 @@
 #include <atomic>
 #include <condition_variable>
 #include <cstddef>
+#include <deque>
+#include <exception>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -61,7 +63,16 @@ class HostStager {
   // dst (pageable host, leading dimension ld_dst)  <-  src (device, dense) on `stream`; the host-side scatter happens
   // when the slot is needed again or in finish().
   void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream);
-  // Completes every pending scatter.  Call after the streams were synchronised.
+  // The same, handed to a background thread: it makes `stream` wait for the n_after events (the tile's last kernels),
+  // copies the tile into a pinned slot as slots come free, waits for the copy and scatters it.  The caller does not
+  // wait for a slot, so the thread that enqueues a plan keeps going when many C tiles complete close together (with
+  // the blocking call it fell back to the pace of the write-backs there, the kernels behind them were launched late and
+  // a call with a pageable C took 148 ms instead of 125 ms at 16384^3).  Nothing else may use `stream` or the slots
+  // until finish(); the device memory at src must stay untouched until then.
+  void write_back_deferred(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream,
+                           void* const* after, int n_after);
+  // Completes every pending scatter, deferred ones included (those need not have been waited for: their copies are
+  // synchronised here); rethrows what the background thread ran into.  The blocking ones need the streams synchronised.
   void finish();
   // Forgets pending scatters without performing them: after a failed call their destinations may no longer be valid.
   void abandon();
@@ -83,6 +94,20 @@ class HostStager {
   long long slot_bytes_ = 0;
   long in_next_ = 0, out_next_ = 0;
   CopyThreads* pool_ = nullptr;
+  // deferred write-backs: requests in call order; the background thread owns the out_ slots while any are open
+  struct Request {
+    void* dst; long ld; const void* src; long rows, cols; int elem; void* stream;
+    void* after[12]; int n_after;
+  };
+  void deferred_loop();
+  std::thread deferred_;
+  CopyThreads* deferred_pool_ = nullptr;
+  std::mutex dmu_;
+  std::condition_variable dcv_;
+  std::deque<Request> requests_;
+  long open_ = 0;              // requests accepted and not yet scattered (or dropped)
+  bool stop_ = false, dropping_ = false;
+  std::exception_ptr error_;
 };
 
 // Completes the staged write-backs on the normal path, drops them when the call unwinds with an error.

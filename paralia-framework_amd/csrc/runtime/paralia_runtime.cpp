@@ -354,11 +354,18 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
     return base + p.k0(ki) * p.tn(ni);
   };
 
+  // Write-backs into a pageable C are handed to the stager's background thread (it waits for the tile's kernels, copies
+  // and scatters at the pace of the link while this thread goes on enqueuing), unless a later command waits for a
+  // write-back (a pool smaller than the working set recycles accumulator blocks) or the call is being traced.
+  bool defer_wb = pageable[2] && !trace;
+  for (const Cmd& c : plan.cmds) defer_wb = defer_wb && !(c.kind == CMD_WRITEBACK && c.signals);
+
   DrainOnError guard(R.res);
   for (size_t i = 0; i < plan.cmds.size(); ++i) {
     const Cmd& c = plan.cmds[i];
     void* s = R.res.stream(c.stream);
-    for (int w = 0; w < c.nwait; ++w) chk(pl_stream_wait_event(s, ev[c.wait[w]]), "stream wait event");
+    const bool deferred = defer_wb && c.kind == CMD_WRITEBACK;  // its waits are enqueued with its copy, by the other thread
+    for (int w = 0; w < c.nwait && !deferred; ++w) chk(pl_stream_wait_event(s, ev[c.wait[w]]), "stream wait event");
     if (trace) chk(pl_event_record(R.res.timing_events[1 + 2 * i], s), "event record");
     switch (c.kind) {
       case CMD_FETCH_A: {
@@ -412,7 +419,11 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       case CMD_WRITEBACK: {
         const long m = p.tm(c.mi), n = p.tn(c.ni);
         T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
-        if (pageable[2]) stager.write_back(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s);
+        if (deferred) {
+          void* after[MAX_WAITS];
+          for (int w = 0; w < c.nwait; ++w) after[w] = ev[c.wait[w]];
+          stager.write_back_deferred(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s, after, c.nwait);
+        } else if (pageable[2]) stager.write_back(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s);
         else chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
       } break;
     }
@@ -422,6 +433,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       chk(pl_event_record(ev[i], s), "event record");
     }
   }
+  if (defer_wb) stager.finish();  // the background thread is done with the write-back stream and the pinned slots
   R.res.sync_all();
   guard.armed = false;
   staged.finish();
