@@ -78,8 +78,7 @@ struct Resources {
   // one runs the streamed 16384^3 fp64 GEMM in 130 ms, the others in 148-169 ms.  The alignment depends on how
   // many streams the application created before this library did, which cannot be queried.  So seven streams
   // are created back to back, "rotation" r uses streams r .. r+3 as (H2D, D2H, compute 0, compute 1), and
-  // the first four large streamed GEMM calls that repeat an already tuned problem each run under a different
-  // rotation; the fastest is kept
+  // calls three to six of a large streamed GEMM problem each run under a different rotation; the fastest is kept
   // (PARALIA_STREAM_ROTATION=r skips the trial).  With 8 or more hardware queues all rotations are equal.
   void* ring[7] = {nullptr};
   int rotation = 0;
