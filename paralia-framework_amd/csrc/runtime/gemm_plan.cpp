@@ -551,7 +551,8 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
         case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
         case CMD_GEMM:
           for (int k = c.ki; k < c.ki + c.kn; ++k) {
-            if (k < p.slabs() && p.slabs() > 1) dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.T) / p.slabs() + st.slab_fixed;
+            if (k < p.slabs() && p.slabs() > 1)
+              dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.T) / p.slabs() + st.slab_fixed * std::max(1.0, 1024.0 / (double)p.tk(k));
             else dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
           }
           if (c.kn > 1) dur = std::max(0.5 * dur, dur - (c.kn - 1) * st.merge_saving * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2);

@@ -137,8 +137,10 @@ struct StageTimes {
   double tr_amp = 0, tr_idle = 6e-3, tr_recover = 8e-3;
   double tr_gap0 = 1e-3;             // idle time assumed in front of the call (calls made back to back)
   bool block_orders = true;          // offer the block orders (w >= ORDER_BLOCK_ROWS) to the order search
-  // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch
-  double slab_fixed = 2e-6;  // measured: 2048 x 2048 x 1024 119.9 us, x 512 61.2 us against 236.7 us for the whole tile
+  // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch for slabs 1024 deep
+  // or deeper, in inverse proportion to the depth below that (measured inside streamed calls, two launches sharing the
+  // device: 2048 x 2048 x 1024 slabs +2 us, x 512 slabs +4.5 us against a quarter of the whole tile's 231.5 us)
+  double slab_fixed = 2e-6;
 };
 struct PipelineResult {
   double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource
