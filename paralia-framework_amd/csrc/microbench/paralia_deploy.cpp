@@ -289,11 +289,12 @@ static void bench_blas1(const std::string& db, const char* func, bool quick) {
 }
 
 // The device's power-state transient, as the tile kernels see it: pairs of 2048^3 fp64 launches on two streams, 100 pairs
-// back to back (the first burst brings the device to its steady state), then after a host-side gap of 5 and of 20 ms
-// without kernels another 100, every pair timed with events.  Against the steady pair time of a burst's last 40 pairs a
-// burst after a gap loses L(gap) seconds in its first 60 pairs, the slowest pair being (1 + amplitude) x steady.  With
-// the deficit decaying exponentially while kernels run, L(20 ms) = amplitude x recovery constant; with it growing as
-// 1 - exp(-gap / idle constant) while none run, L(5 ms) / L(20 ms) gives the idle constant.  Three repetitions, medians.
+// back to back (the first burst brings the device to its steady state), then after a host-side gap of 2, 5, 10, 20 and
+// 50 ms without kernels another 100, every pair timed with events.  Against the steady pair time of a burst's last 40
+// pairs a burst after a gap loses L(gap) seconds in its first 60 pairs, the slowest pair being (1 + amplitude) x steady.
+// With the deficit decaying exponentially while kernels run, L(50 ms) = amplitude x recovery constant; with it growing
+// as 1 - exp(-gap / idle constant) while none run, the idle constant is the one that fits L(gap) / L(50 ms) over the
+// five gaps best (least squares over a grid of constants).  Three repetitions, medians.
 // Written to Processed/Power-transient_dev-0.log (seconds); not a file of the reference.
 static void bench_transient(const std::string& db) {
   const long Tt = 2048;
@@ -325,11 +326,12 @@ static void bench_transient(const std::string& db) {
     }
   };
   auto median3 = [](double a, double b, double c) { return std::max(std::min(a, b), std::min(std::max(a, b), c)); };
-  const double gaps[2] = {5e-3, 20e-3};
-  double loss[2][3], peak[3], steady_t = 0;
+  constexpr int NG = 5;
+  const double gaps[NG] = {2e-3, 5e-3, 10e-3, 20e-3, 50e-3};
+  double loss[NG][3], peak[3], steady_t = 0;
   std::vector<double> t;
   for (int rep = 0; rep < 3; ++rep)
-    for (int g = 0; g < 2; ++g) {
+    for (int g = 0; g < NG; ++g) {
       burst(t);  // warm: whatever came before, the device is in its steady state afterwards
       const double t0 = csecond();
       while (csecond() - t0 < gaps[g]) {
@@ -341,17 +343,27 @@ static void bench_transient(const std::string& db) {
       for (int i = 0; i < 60; ++i) l += t[i] - steady;
       for (int i = 0; i < 20; ++i) p = std::max(p, t[i] / steady - 1.0);
       loss[g][rep] = std::max(l, 0.0);
-      if (g == 1) { peak[rep] = p; steady_t = steady; }
+      if (g == NG - 1) { peak[rep] = p; steady_t = steady; }
     }
-  const double l5 = median3(loss[0][0], loss[0][1], loss[0][2]), l20 = median3(loss[1][0], loss[1][1], loss[1][2]);
+  double L[NG];
+  for (int g = 0; g < NG; ++g) L[g] = median3(loss[g][0], loss[g][1], loss[g][2]);
   double amp = median3(peak[0], peak[1], peak[2]);
   double recover = 0, idle = 0;
-  if (amp < 0.02 || l20 <= 0) {
+  if (amp < 0.02 || L[NG - 1] <= 0) {
     amp = 0;  // nothing to model on this device
   } else {
-    recover = l20 / amp;
-    const double frac = std::min(0.95, std::max(0.05, l5 / l20));
-    idle = -gaps[0] / log(1.0 - frac);
+    recover = L[NG - 1] / amp;
+    double best = 1e300;
+    for (double tau = 1e-3; tau <= 60e-3; tau += 0.25e-3) {
+      // the longest gap is not quite infinite: compare with the curve normalised at that gap
+      const double full = 1.0 - exp(-gaps[NG - 1] / tau);
+      double sq = 0;
+      for (int g = 0; g < NG - 1; ++g) {
+        const double d = L[g] / L[NG - 1] - (1.0 - exp(-gaps[g] / tau)) / full;
+        sq += d * d;
+      }
+      if (sq < best) { best = sq; idle = tau; }
+    }
   }
   char out[1024];
   snprintf(out, sizeof out, "%s/Processed/Power-transient_dev-0.log", db.c_str());
@@ -359,8 +371,8 @@ static void bench_transient(const std::string& db) {
   if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
   fprintf(fp, "Amplitude: %e\nRecovery: %e\nIdle: %e\n", amp, recover, idle);
   fclose(fp);
-  fprintf(stderr, "power transient: steady pair %.3f ms, after 5 / 20 ms idle %.2f / %.2f ms lost, slowest pair +%.1f %% -> recovery %.1f ms, idle %.1f ms\n",
-          steady_t * 1e3, l5 * 1e3, l20 * 1e3, amp * 100, recover * 1e3, idle * 1e3);
+  fprintf(stderr, "power transient: steady pair %.3f ms, after 2 / 5 / 10 / 20 / 50 ms idle %.2f / %.2f / %.2f / %.2f / %.2f ms lost, slowest pair +%.1f %% -> recovery %.1f ms, idle %.1f ms\n",
+          steady_t * 1e3, L[0] * 1e3, L[1] * 1e3, L[2] * 1e3, L[3] * 1e3, L[4] * 1e3, amp * 100, recover * 1e3, idle * 1e3);
   for (auto e : ev) pl_event_destroy(e);
   for (auto s : st) pl_stream_destroy(s);
   CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
