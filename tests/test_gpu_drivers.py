@@ -211,9 +211,11 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
     def transient(path):
         return {k.strip(): float(v) for k, v in (line.split(":") for line in open(path))}
     tr, tr_shipped = transient(os.path.join(fresh, "Power-transient_dev-0.log")), transient(os.path.join(shipped, "Power-transient_dev-0.log"))
-    assert 0.1 < tr["Amplitude"] < 0.5, tr
-    for k in ("Amplitude", "Recovery", "Idle"):
-        assert 0.4 * tr_shipped[k] < tr[k] < 2.5 * tr_shipped[k], (k, tr, tr_shipped)
+    # (the two time constants come out of a fit to a curve that is only roughly exponential: wide bands)
+    assert 0.05 < tr["Amplitude"] < 0.6, tr
+    assert 0.5 * tr_shipped["Amplitude"] < tr["Amplitude"] < 2.0 * tr_shipped["Amplitude"], (tr, tr_shipped)
+    for k in ("Recovery", "Idle"):
+        assert 0.25 * tr_shipped[k] < tr[k] < 4.0 * tr_shipped[k], (k, tr, tr_shipped)
     # matrix-vector and vector kernels take 40 - 80 us at the largest sizes of the quick sweep: launch and
     # synchronisation are a visible part of that, and working sets of 128 - 384 MiB sit partly inside the memory-side
     # cache, so these differ more between machines than the millisecond-scale GEMM tiles: a wider band
