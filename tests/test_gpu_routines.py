@@ -442,6 +442,47 @@ def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg,
     pkg.check(L.PARALiA_runtime_shutdown(), "shutdown twice is harmless")
 
 
+def test_stream_alignment_trial_runs_on_calls_three_to_six_and_can_be_pinned(pkg, L, monkeypatch):
+    """The stream-to-hardware-queue alignment is tried on calls three to six of a streamed GEMM problem with at least 64
+    commands (each under one of the four rotations of the stream ring; the results stay exact), reported as settled after
+    that, kept over a teardown, and never tried when PARALIA_STREAM_ROTATION pins it.  A problem with fewer commands does
+    not start a trial."""
+    def state():
+        rot, settled = C.c_int(-1), C.c_int(-1)
+        pkg.check(L.PARALiA_stream_rotation(C.byref(rot), C.byref(settled)), "rotation")
+        return rot.value, settled.value
+    M = N = K = 768
+    rng = np.random.default_rng(5)
+    A, B = rng.integers(-3, 4, M * K).astype(np.float64), rng.integers(-3, 4, K * N).astype(np.float64)
+    ref = (A.reshape(K, M).T @ B.reshape(N, K).T).T.ravel()
+    bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, np.zeros(M * N), -1)
+    monkeypatch.delenv("PARALIA_STREAM_ROTATION", raising=False)
+    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")        # a new stream ring, nothing settled
+    seen = []
+    for call in range(8):
+        # T = 384: 2 x 2 x 2 tiles, under 64 commands -> no trial; T = 128: 6 x 6 x 6 tiles -> trial
+        before = state()
+        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=384)
+        assert state() == before
+        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
+        assert np.array_equal(bC.get(), ref)
+        seen.append(state())
+    assert [s[1] for s in seen] == [0, 0, 0, 0, 0, 1, 1, 1]      # settled by the sixth call of the problem
+    assert [s[0] for s in seen[2:5]] == [0, 1, 2]                # calls three to five ran under rotations 0, 1, 2
+    chosen = seen[-1][0]
+    assert 0 <= chosen < 4
+    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
+    call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
+    assert state() == (chosen, 1)                                 # the choice outlives the teardown
+    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
+    monkeypatch.setenv("PARALIA_STREAM_ROTATION", "2")
+    for call in range(4):
+        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
+        assert state() == (2, 1) and np.array_equal(bC.get(), ref)
+    monkeypatch.delenv("PARALIA_STREAM_ROTATION")
+    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")        # the next test builds an unpinned ring again
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 @pytest.mark.parametrize("order", [80000, 80002, 90003, 160002, 320003, 240002, 330000, 304, 10403, 80405, 250302])
 @pytest.mark.parametrize("locs", [(-1, -1, -1), (-1, -1, 0), (-2, -2, -1), (0, -1, -1)])
