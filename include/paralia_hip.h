@@ -63,6 +63,13 @@ int pl_stream_wait_event(void* stream, void* event);
 int pl_event_sync(void* event);
 int pl_event_query(void* event, int* done);
 int pl_event_elapsed_ms(void* start, void* stop, float* ms);
+/* *shares <- 1 when `candidate` executes in order with at least one of others[0 .. n-1] (n <= PL_MAX_PROBE_STREAMS),
+ * i.e. HIP placed it on the same hardware queue; 0 when its work can overlap theirs.  Launches two tiny kernels per
+ * stream and waits for them (about half a millisecond).  The reference creates its queues per link and per backend
+ * worker (Subkernel.cpp:249-306) and relies on CUDA streams being independent; HIP streams are only independent when
+ * they sit on different hardware queues. */
+#define PL_MAX_PROBE_STREAMS 8
+int pl_stream_shares_queue(void* candidate, void* const* others, int n, int* shares);
 
 /* ---- copies (CoCoMemcpy2DAsync: Subkernel_backup.cpp:526-529,1229-1232; CoCoMemcpyAsync: :468-470;
  *      CoCoMemcpy: dgemm_runner.cpp:77; CoCoSyncCheckErr: dgemm.cpp:597) ---- */
@@ -186,9 +193,11 @@ int PARALiA_runtime_shutdown(void);
 #define PL_TRACE_ROW 7
 int PARALiA_trace_enable(int on);
 long PARALiA_trace_read(double* rows, long max_rows);
-/* which of the four stream-to-hardware-queue alignments the scheduler uses, and whether its start-up trial of
- * them (first four large streamed GEMM calls) is over; no counterpart in the reference */
-int PARALiA_stream_rotation(int* rotation, int* settled);
+/* the scheduler's stream inventory: *independent <- how many of its four busy streams (H2D, D2H, two compute) were
+ * found to sit on hardware queues of their own (4 unless the process has fewer than four hardware queues), *created <-
+ * how many streams it created to find them; both 0 before the first call that needs streams.  No counterpart in the
+ * reference. */
+int PARALiA_stream_queues(int* independent, int* created);
 /* directory holding Processed/ lookup tables and link models (DEPLOYDB, CMakeLists.txt:376) */
 int PARALiA_set_db_dir(const char* dir);
 

@@ -57,6 +57,7 @@ _SIGS = {
     "pl_copy2d_async": (_i, [_vp, _l, _vp, _l, _l, _l, _i, _vp]),
     "pl_copy_async": (_i, [_vp, _vp, _ll, _vp]),
     "pl_copy": (_i, [_vp, _vp, _ll]),
+    "pl_stream_shares_queue": (_i, [_vp, C.POINTER(_vp), _i, _pi]),
     "pl_memset_async": (_i, [_vp, _i, _ll, _vp]),
     "pl_sync_check": (_i, []),
     "pl_dgemm_tile": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp]),
@@ -83,7 +84,7 @@ _SIGS = {
     "PARALiA_dev_cache_free": (_i, [_i]),
     "PARALiA_runtime_stats": (_i, [C.POINTER(_l), C.POINTER(_l), C.POINTER(_ll), C.POINTER(_l)]),
     "PARALiA_runtime_reset": (_i, []),
-    "PARALiA_stream_rotation": (_i, [_pi, _pi]),
+    "PARALiA_stream_queues": (_i, [_pi, _pi]),
     "PARALiA_runtime_shutdown": (_i, []),
     "PARALiA_trace_enable": (_i, [_i]),
     "PARALiA_trace_read": (_l, [C.POINTER(_d), _l]),

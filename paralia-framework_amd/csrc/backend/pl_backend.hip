@@ -25,6 +25,17 @@ int fail(hipError_t e, const char* what) {
     hipError_t e_ = (call);               \
     if (e_ != hipSuccess) return fail(e_, #call); \
   } while (0)
+
+// One wave that stays on the device for `ticks` of the constant-rate wall clock; the loop count bounds it whatever
+// the clock reads.
+__global__ void hold_kernel(long long ticks) {
+  const long long t0 = (long long)wall_clock64();
+  for (int i = 0; i < 4096; ++i) {
+    if ((long long)wall_clock64() - t0 >= ticks) break;
+    __builtin_amdgcn_s_sleep(64);
+  }
+}
+__global__ void noop_kernel() {}
 }  // namespace
 
 int pl_fail_hip(int hip_error, const char* what) { return fail((hipError_t)hip_error, what); }
@@ -142,6 +153,57 @@ int pl_event_query(void* event, int* done) {
 }
 int pl_event_elapsed_ms(void* start, void* stop, float* ms) {
   PL_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return 0;
+}
+
+// Does `candidate` run in order with one of others[0 .. n-1]?  HIP places the streams of a process on a few hardware
+// queues (GPU_MAX_HW_QUEUES, 4 by default): a new stream goes to the queue with the fewest streams, ties broken in an
+// order that is not creation order, so which streams end up together cannot be told from how many were created.
+// Streams on one queue execute strictly one after the other, as if they were one stream.  The test is functional: a
+// one-wave kernel that stays resident for half a millisecond goes to each of the others, an empty kernel to the
+// candidate; if the empty kernel has completed while all the holders are still running, the candidate's queue is its
+// own.  A candidate that shares a queue cannot pass (its kernel is behind a holder); one that does not share can only
+// fail when the calling thread loses the processor for the rest of the half millisecond, and the caller then simply
+// tries another stream.
+int pl_stream_shares_queue(void* candidate, void* const* others, int n, int* shares) {
+  *shares = 0;
+  if (n <= 0) return 0;
+  if (n > PL_MAX_PROBE_STREAMS || !candidate) return pl_fail_msg(PL_ERR_ARG, "pl_stream_shares_queue: 1 to 8 streams to compare with");
+  int dev = 0, khz = 0;
+  PL_TRY(hipGetDevice(&dev));
+  PL_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+  if (khz <= 0) khz = 100000;
+  const long long hold_ticks = (long long)khz / 2;  // 0.5 ms of the constant-rate clock
+  static bool warmed = false;  // the first launch of a kernel loads its code: not inside the measured window
+  if (!warmed) {
+    hipLaunchKernelGGL(hold_kernel, dim3(1), dim3(64), 0, (hipStream_t)candidate, 0LL);
+    hipLaunchKernelGGL(noop_kernel, dim3(1), dim3(64), 0, (hipStream_t)candidate);
+    PL_TRY(hipGetLastError());
+    PL_TRY(hipStreamSynchronize((hipStream_t)candidate));
+    warmed = true;
+  }
+  hipEvent_t held[PL_MAX_PROBE_STREAMS], done;
+  for (int i = 0; i < n; ++i) PL_TRY(hipEventCreateWithFlags(&held[i], hipEventDisableTiming));
+  PL_TRY(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+  for (int i = 0; i < n; ++i) {
+    hipLaunchKernelGGL(hold_kernel, dim3(1), dim3(64), 0, (hipStream_t)others[i], hold_ticks);
+    PL_TRY(hipEventRecord(held[i], (hipStream_t)others[i]));
+  }
+  hipLaunchKernelGGL(noop_kernel, dim3(1), dim3(64), 0, (hipStream_t)candidate);
+  PL_TRY(hipGetLastError());
+  PL_TRY(hipEventRecord(done, (hipStream_t)candidate));
+  PL_TRY(hipEventSynchronize(done));
+  for (int i = 0; i < n; ++i) {
+    hipError_t e = hipEventQuery(held[i]);
+    if (e == hipSuccess) *shares = 1;                       // a holder had finished before the candidate's kernel ran
+    else if (e == hipErrorNotReady) (void)hipGetLastError();
+    else return fail(e, "hipEventQuery");
+  }
+  for (int i = 0; i < n; ++i) {
+    PL_TRY(hipEventSynchronize(held[i]));
+    PL_TRY(hipEventDestroy(held[i]));
+  }
+  PL_TRY(hipEventDestroy(done));
   return 0;
 }
 

@@ -20,7 +20,7 @@ ATC_p ddot_impl(long, double*, long, double*, long, double*, ATC_p);
 void cache_free_impl(short);
 void runtime_stats(long*, long*, long long*, long*);
 void runtime_reset();
-void stream_rotation(int*, int*);
+void stream_queues(int*, int*);
 void runtime_shutdown();
 void trace_enable(int);
 long trace_read(double*, long);
@@ -140,8 +140,8 @@ long PARALiA_trace_read(double* rows, long max_rows) {
   guarded([&] { n = paralia::trace_read(rows, max_rows); });
   return n;
 }
-int PARALiA_stream_rotation(int* rotation, int* settled) {
-  return guarded([&] { paralia::stream_rotation(rotation, settled); });
+int PARALiA_stream_queues(int* independent, int* created) {
+  return guarded([&] { paralia::stream_queues(independent, created); });
 }
 int PARALiA_set_db_dir(const char* dir) {
   paralia_set_db_dir(dir);

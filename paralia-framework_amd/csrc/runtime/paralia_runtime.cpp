@@ -72,63 +72,77 @@ struct Resources {
   double* dot_ws = nullptr;      // ddot partials
   double* dot_result = nullptr;  // device scalar
   double* dot_host = nullptr;    // pinned scalar
-  // HIP deals the streams of a process round-robin onto GPU_MAX_HW_QUEUES hardware queues (4 by default), in
-  // creation order and counting the default stream.  With 4 queues the four streams this scheduler keeps busy
-  // always sit on four different queues, yet which stream sits on which queue matters: of the four alignments
-  // one runs the streamed 16384^3 fp64 GEMM in 130 ms, the others in 148-169 ms.  The alignment depends on how
-  // many streams the application created before this library did, which cannot be queried.  So seven streams
-  // are created back to back, "rotation" r uses streams r .. r+3 as (H2D, D2H, compute 0, compute 1), and
-  // calls three to six of a large streamed GEMM problem each run under a different rotation; the fastest is kept
-  // (PARALIA_STREAM_ROTATION=r skips the trial).  With 8 or more hardware queues all rotations are equal.
-  void* ring[7] = {nullptr};
-  int rotation = 0;
-  int trials = 0;            // rotations tried so far; 4 = settled
-  double trial_rate[4] = {0, 0, 0, 0};
-  // The four trial calls are calls of ONE problem (rates of different shapes do not compare), and the more of a call's
-  // time the tile kernels take, the better its time tells the alignments apart: a call bounded by the link runs nearly
-  // the same under all four, and a choice made on such a call is a draw.  So the trial is run again when a problem
-  // comes along whose predicted compute share is clearly higher than that of the problem the last trial ran on.
-  bool rotation_pinned = false;       // PARALIA_STREAM_ROTATION: never tried, never changed
-  const void* trial_problem = nullptr;
-  double trial_weight = -1;           // predicted compute share of trial_problem
-  void set_rotation(int r) {
-    rotation = r;
-    h2d = ring[r];
-    d2h = ring[r + 1];
-    exec[0] = ring[r + 2];
-    exec[1] = ring[r + 3];
+  // HIP places the streams of a process on GPU_MAX_HW_QUEUES hardware queues (4 by default), and streams that share
+  // a queue run strictly one after the other.  A new stream goes to the queue with the fewest streams, ties broken in
+  // a fixed order that is not creation order (seven streams created back to back land on queues 1 2 3 4 4 3 2), and
+  // streams the application created earlier shift everything.  What sharing costs the streamed 16384^3 fp64 GEMM:
+  // both compute streams on one queue 138 ms (no two tile kernels ever overlap), each copy stream sharing with a
+  // compute stream 150 ms (a tile kernel waits for every fetch enqueued before it), both copy streams on one queue
+  // 160 ms, four queues of their own 122 ms.  So the four busy streams are not taken as they come: streams are
+  // created one at a time and each is kept only if a functional test (pl_stream_shares_queue) shows that it does not
+  // run in order with the ones already kept; the others are destroyed again.  A few milliseconds, once.
+  std::vector<void*> owned;   // every stream this inventory created and still holds
+  int independent = 0;        // how many of (h2d, d2h, exec0, exec1) sit on a hardware queue of their own
+  int created = 0;            // streams created while looking for them
+  void* new_stream() {
+    void* s = nullptr;
+    chk(pl_stream_create(&s), "stream create");
+    ++created;
+    return s;
+  }
+  bool shares_queue(void* cand, const std::vector<void*>& with) {
+    if (with.empty()) return false;
+    int shares = 0;
+    chk(pl_stream_shares_queue(cand, with.data(), (int)with.size(), &shares), "stream placement test");
+    if (shares) chk(pl_stream_shares_queue(cand, with.data(), (int)with.size(), &shares), "stream placement test");  // confirm
+    return shares != 0;
   }
   void ensure_streams(int nq) {
-    if (!ring[0]) {
-      for (void*& s : ring) chk(pl_stream_create(&s), "stream create");
-      nexec = 2;
-      const char* env = getenv("PARALIA_STREAM_ROTATION");
-      if (env && atoi(env) >= 0 && atoi(env) < 4) {
-        set_rotation(atoi(env));
-        trials = 4;
-        rotation_pinned = true;
-      } else {
-        set_rotation(rotation);  // 0 in a new process; after a teardown what was in use (or chosen) before it
+    if (!h2d) {
+      std::vector<void*> kept, sharing;
+      // at most 4 hardware queues are expected to matter; 16 candidates cover an application that already holds a
+      // dozen streams on them
+      for (int tries = 0; kept.size() < 4 && tries < 16; ++tries) {
+        void* s = new_stream();
+        (shares_queue(s, kept) ? sharing : kept).push_back(s);
       }
+      independent = (int)kept.size();
+      // Fewer than four queues to be had (GPU_MAX_HW_QUEUES below 4): the copy streams keep queues of their own first,
+      // and a compute stream rather shares with the other compute stream than with a copy stream.
+      while (kept.size() < 4) {
+        const std::vector<void*> copies(kept.begin(), kept.begin() + std::min<size_t>(2, kept.size()));
+        size_t pick = sharing.size();
+        for (size_t i = 0; i < sharing.size() && pick == sharing.size(); ++i)
+          if (kept.size() >= 2 && !shares_queue(sharing[i], copies)) pick = i;
+        if (pick == sharing.size()) {
+          if (sharing.empty()) sharing.push_back(new_stream());
+          pick = 0;
+        }
+        kept.push_back(sharing[pick]);
+        sharing.erase(sharing.begin() + pick);
+      }
+      for (void* s : sharing) chk(pl_stream_destroy(s), "stream destroy");
+      owned = kept;
+      h2d = kept[0];
+      d2h = kept[1];
+      exec[0] = kept[2];
+      exec[1] = kept[3];
+      nexec = 2;
     }
-    for (; nexec < nq; ++nexec) chk(pl_stream_create(&exec[nexec]), "stream create");
-  }
-  // Called around a large streamed GEMM: picks the rotation to try, then records seconds per flop.
-  int settled_rotation = 0;  // what the last finished trial chose (0 before any)
-  void begin_trial() {
-    if (trials < 4) set_rotation(trials);
-  }
-  void end_trial(double seconds_per_flop) {
-    if (trials >= 4) return;
-    trial_rate[trials++] = seconds_per_flop;
-    if (trials == 4) {
-      // the alignment in use so far stays unless another one is faster by more than the noise of a single call (2 %):
-      // on a call the link bounds all four measure alike, and the winner of such a draw can cost the next problem 7 %
-      int best = settled_rotation;
-      for (int r = 0; r < 4; ++r)
-        if (trial_rate[r] < 0.98 * trial_rate[settled_rotation] && trial_rate[r] < trial_rate[best]) best = r;
-      settled_rotation = best;
-      set_rotation(best);
+    // further compute streams (PARALIA_EXEC_QUEUES above 2) have to share a queue with somebody: not with a copy stream
+    for (; nexec < nq; ++nexec) {
+      const std::vector<void*> copies = {h2d, d2h};
+      std::vector<void*> sharing;
+      void* pick = nullptr;
+      for (int tries = 0; !pick && tries < 8; ++tries) {
+        void* s = new_stream();
+        if (shares_queue(s, copies)) sharing.push_back(s);
+        else pick = s;
+      }
+      if (!pick) { pick = sharing.back(); sharing.pop_back(); }
+      for (void* s : sharing) chk(pl_stream_destroy(s), "stream destroy");
+      owned.push_back(pick);
+      exec[nexec] = pick;
     }
   }
   void ensure_events(size_t n) {
@@ -191,11 +205,10 @@ struct Resources {
     }
   }
   // The counterpart of CoCoPeLiaFreeResources (Subkernel.cpp:330): streams, events, workspaces and bounce buffers
-  // go; the next call creates them again.  The stream-alignment choice already made is kept.
+  // go; the next call creates them again (and places its streams anew).
   void destroy() {
     drain();
-    for (void* s : ring) if (s) pl_stream_destroy(s);
-    for (int q = 2; q < nexec; ++q) if (exec[q]) pl_stream_destroy(exec[q]);
+    for (void* s : owned) pl_stream_destroy(s);
     for (void* e : events) pl_event_destroy(e);
     for (void* e : timing_events) pl_event_destroy(e);
     if (dot_ws) pl_free_device(dot_ws);
@@ -203,14 +216,8 @@ struct Resources {
     gemv_x.release(); gemv_y.release(); gemv_ws.release();
     for (Scratch& w : gemm_ws) w.release();
     stager_.reset();
-    const int keep_rotation = rotation, keep_trials = trials, keep_settled = settled_rotation;
     const bool keep_trace = trace_on;
-    const double keep_weight = trial_weight;
     *this = Resources();
-    rotation = keep_trials >= 4 ? keep_rotation : keep_settled;
-    settled_rotation = keep_settled;
-    trials = keep_trials >= 4 ? 4 : 0;   // a trial in progress starts over on the new ring
-    trial_weight = keep_trials >= 4 ? keep_weight : -1;
     trace_on = keep_trace;
   }
 };
@@ -558,22 +565,8 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     const GemmPlan& plan = entry->plan;
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T), atc->cache_limit);
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
-    // the first two calls of a problem also pay for fresh pool memory and cold caches (the second still runs a few
-    // percent slow): a trial that started there would misjudge its first rotation
-    const bool eligible = !R.res.rotation_pinned && plan.cmds.size() >= 64 && !no_ab && entry->calls >= 2;
-    const double weight = atc->pred_t > 0 ? atc->pipeline.t_exec_busy / atc->pred_t : 0;
-    if (eligible && entry != R.res.trial_problem &&
-        (R.res.trials >= 4 ? weight > R.res.trial_weight + 0.15 : weight >= R.res.trial_weight)) {
-      R.res.trials = 0;               // settled on a less compute-bound problem, or that problem's calls stopped coming
-      R.res.trial_problem = entry;
-      R.res.trial_weight = weight;
-    }
-    const bool trial = eligible && R.res.trials < 4 && entry == R.res.trial_problem;
-    if (trial) R.res.begin_trial();
-    const double t0 = csecond();
     const bool pageable[3] = {locA == -2, locB == -2, locC == -2};
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC, pageable);
-    if (trial) R.res.end_trial((csecond() - t0) / (2.0 * M * N * (double)K));
   }
   ++entry->calls;
   return atc_copy(atc);
@@ -932,11 +925,11 @@ void runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long
   if (pmd_entries) *pmd_entries = (long)R.pmd.size();
 }
 
-void stream_rotation(int* rotation, int* settled) {
+void stream_queues(int* independent, int* created) {
   Runtime& R = rt();
   std::lock_guard<std::mutex> lk(R.mu);
-  if (rotation) *rotation = R.res.rotation;
-  if (settled) *settled = R.res.trials >= 4 ? 1 : 0;
+  if (independent) *independent = R.res.independent;
+  if (created) *created = R.res.created;
 }
 
 void runtime_reset() {

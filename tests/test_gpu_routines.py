@@ -1,6 +1,7 @@
 """Parity of the PARALiA routines (tiling, streaming, block pool, lazy write-back, metadata reuse) called through
 the C ABI, against OpenBLAS / the oracle on the same seeded inputs, for every operand placement."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -442,45 +443,49 @@ def test_runtime_shutdown_releases_everything_and_the_next_call_starts_cold(pkg,
     pkg.check(L.PARALiA_runtime_shutdown(), "shutdown twice is harmless")
 
 
-def test_stream_alignment_trial_runs_on_calls_three_to_six_and_can_be_pinned(pkg, L, monkeypatch):
-    """The stream-to-hardware-queue alignment is tried on calls three to six of a streamed GEMM problem with at least 64
-    commands (each under one of the four rotations of the stream ring; the results stay exact), reported as settled after
-    that, kept over a teardown, and never tried when PARALIA_STREAM_ROTATION pins it.  A problem with fewer commands does
-    not start a trial."""
-    def state():
-        rot, settled = C.c_int(-1), C.c_int(-1)
-        pkg.check(L.PARALiA_stream_rotation(C.byref(rot), C.byref(settled)), "rotation")
-        return rot.value, settled.value
+def test_stream_placement_probe_and_the_schedulers_own_streams(pkg, L):
+    """pl_stream_shares_queue is a functional test of "runs in order with": a stream compared with itself must be found
+    to share, nine streams cannot all be independent on the hardware queues of one process (HIP's default is four), and
+    the first of them must find at least one other that overlaps with it.  The scheduler builds its inventory from that
+    test: after a teardown, with one to three more application streams alive than before, its four busy streams are
+    again on hardware queues of their own, and the results stay exact."""
+    def new_stream():
+        s = C.c_void_p()
+        pkg.check(L.pl_stream_create(C.byref(s)), "stream")
+        return s
+
+    def shares(cand, others):
+        arr = (C.c_void_p * len(others))(*[o.value for o in others])
+        out = C.c_int(-1)
+        pkg.check(L.pl_stream_shares_queue(cand, arr, len(others), C.byref(out)), "placement test")
+        return out.value
+    streams = [new_stream() for _ in range(9)]
+    assert shares(streams[0], [streams[0]]) == 1
+    verdicts = [shares(streams[0], [s]) for s in streams[1:]]
+    print("  stream 0 against streams 1..8: shares =", verdicts, flush=True)
+    assert 0 in verdicts and 1 in verdicts
+    assert shares(streams[0], streams[1:]) == 1                 # one of the eight holds its queue
     M = N = K = 768
     rng = np.random.default_rng(5)
     A, B = rng.integers(-3, 4, M * K).astype(np.float64), rng.integers(-3, 4, K * N).astype(np.float64)
     ref = (A.reshape(K, M).T @ B.reshape(N, K).T).T.ravel()
     bA, bB, bC = place(pkg, A, -1), place(pkg, B, -1), place(pkg, np.zeros(M * N), -1)
-    monkeypatch.delenv("PARALIA_STREAM_ROTATION", raising=False)
-    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")        # a new stream ring, nothing settled
-    seen = []
-    for call in range(8):
-        # T = 384: 2 x 2 x 2 tiles, under 64 commands -> no trial; T = 128: 6 x 6 x 6 tiles -> trial
-        before = state()
-        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=384)
-        assert state() == before
+    queues = int(os.environ.get("GPU_MAX_HW_QUEUES", "4") or 4)
+    extra = []
+    for more in range(4):
+        pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
+        ind, made = C.c_int(-1), C.c_int(-1)
+        pkg.check(L.PARALiA_stream_queues(C.byref(ind), C.byref(made)), "stream queues")
+        assert (ind.value, made.value) == (0, 0)                  # nothing held after a teardown
         call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
         assert np.array_equal(bC.get(), ref)
-        seen.append(state())
-    assert [s[1] for s in seen] == [0, 0, 0, 0, 0, 1, 1, 1]      # settled by the sixth call of the problem
-    assert [s[0] for s in seen[2:5]] == [0, 1, 2]                # calls three to five ran under rotations 0, 1, 2
-    chosen = seen[-1][0]
-    assert 0 <= chosen < 4
+        pkg.check(L.PARALiA_stream_queues(C.byref(ind), C.byref(made)), "stream queues")
+        print("  %d application streams alive: %d independent scheduler streams, %d created to find them" % (9 + more, ind.value, made.value), flush=True)
+        assert ind.value == min(4, queues) and 4 <= made.value <= 16
+        extra.append(new_stream())
+    for s in streams + extra:
+        pkg.check(L.pl_stream_destroy(s), "stream destroy")
     pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
-    call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
-    assert state() == (chosen, 1)                                 # the choice outlives the teardown
-    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")
-    monkeypatch.setenv("PARALIA_STREAM_ROTATION", "2")
-    for call in range(4):
-        call_gemm(pkg, L, np.float64, "N", "N", M, N, K, 1.0, 0.0, bA, M, bB, K, bC, M, T=128)
-        assert state() == (2, 1) and np.array_equal(bC.get(), ref)
-    monkeypatch.delenv("PARALIA_STREAM_ROTATION")
-    pkg.check(L.PARALiA_runtime_shutdown(), "shutdown")        # the next test builds an unpinned ring again
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
