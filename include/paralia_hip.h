@@ -135,8 +135,12 @@ int pl_dgemv(char trans, long M, long N, double alpha, const double* A, long lda
  * reference.  The partial sums go to a fixed array of PL_DGEMV_NOALLOC_MAX_DOUBLES doubles (4 MiB) that every GPU
  * the library runs on holds until the process ends; kernels, chunking and summation order are those of pl_dgemv,
  * so the results are bitwise the same.  A shape with pl_dgemv_workspace_doubles(trans, M, N) above that size is
- * refused with PL_ERR_DIM (pl_last_error() says why).  All calls on one GPU share the array: calls that may
- * overlap there (different streams, different threads) race; calls on one stream are safe. */
+ * refused with PL_ERR_DIM (pl_last_error() says why).  All calls on one GPU share the array and nothing in the call
+ * checks for a call still in flight (a check would need an event query, which graph capture forbids): the caller must
+ * serialise them -- calls on one stream are safe, calls that may overlap on different streams or threads race.  The
+ * array's address on a device is resolved by pl_set_device and pl_stream_create on that device (the look-up may make
+ * the HIP runtime load the code object, which is not something to do under capture); only a caller who has used
+ * neither pays for it in its first pl_dgemv_noalloc call there. */
 #define PL_DGEMV_NOALLOC_MAX_DOUBLES 524288
 long long pl_dgemv_noalloc_max_doubles(void);
 int pl_dgemv_noalloc(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx,

@@ -55,7 +55,10 @@ int pl_device_count(int* count) {
   *count = c;
   return 0;
 }
-int pl_set_device(int dev) { PL_TRY(hipSetDevice(dev)); return 0; }
+int pl_set_device(int dev) {
+  PL_TRY(hipSetDevice(dev));
+  return pl_noalloc_setup_current_device();
+}
 int pl_get_device(int* dev) { PL_TRY(hipGetDevice(dev)); return 0; }
 int pl_device_sync(void) { PL_TRY(hipDeviceSynchronize()); return 0; }
 
@@ -121,7 +124,7 @@ int pl_stream_create(void** stream) {
   hipStream_t s;
   PL_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   *stream = (void*)s;
-  return 0;
+  return pl_noalloc_setup_current_device();   // so that pl_dgemv_noalloc on this stream finds its scratch resolved
 }
 int pl_stream_destroy(void* stream) { PL_TRY(hipStreamDestroy((hipStream_t)stream)); return 0; }
 int pl_stream_sync(void* stream) { PL_TRY(hipStreamSynchronize((hipStream_t)stream)); return 0; }

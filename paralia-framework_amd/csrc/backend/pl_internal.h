@@ -6,4 +6,7 @@
 int pl_fail_hip(int hip_error, const char* what);   // "<what>: <HIP error string>", returns PL_ERR_HIP
 int pl_fail_msg(int code, const char* message);     // returns code
 
+// Resolves, once per device, the address of the fixed scratch array behind pl_dgemv_noalloc on the current device.
+int pl_noalloc_setup_current_device(void);
+
 #endif

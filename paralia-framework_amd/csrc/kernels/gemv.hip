@@ -233,6 +233,14 @@ static int noalloc_scratch(double** out) {
 
 }  // namespace plk
 
+// Set-up half of pl_dgemv_noalloc: looks the scratch address of the current device up, which may make the runtime load
+// the code object there.  pl_set_device and pl_stream_create call it, so that a caller who holds a stream from this
+// library never pays for it inside pl_dgemv_noalloc (under graph capture, say).
+int pl_noalloc_setup_current_device(void) {
+  double* unused = nullptr;
+  return plk::noalloc_scratch(&unused);
+}
+
 extern "C" {
 
 long long pl_dgemv_workspace_doubles(char trans, long M, long N) {

@@ -19,6 +19,8 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   const bool repeat = order_id >= 20000;  // every panel k-outer, not only the first
   const int orient = (order_id % 20000) / 10000;
   int w = order_id % 10000;
+  if (w == ORDER_FULL_PANEL) w = orient == 0 ? Ng : Mg;   // may now exceed 99: the block test below is on the id's own w
+  const bool block = order_id % 10000 >= ORDER_BLOCK_ROWS;
   std::vector<int> order;
   order.reserve((size_t)Mg * Ng * Kg);
   auto id = [&](int mi, int ni, int ki) { return (mi * Ng + ni) * Kg + ki; };
@@ -40,7 +42,7 @@ std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
           for (int ni = 0; ni <= std::min(d, cols - 1); ++ni) order.push_back(id(m0 + d, n0 + ni, ki));
       }
   };
-  if (w >= ORDER_BLOCK_ROWS) {
+  if (block) {
     // Block orders (w = rows * 100 + columns): a block of rows x columns C tiles at the top left as one k-outer panel.
     // orient 0: then the other rows of the block's columns, then the other columns, tile by tile; orient 1: the other
     // columns of the block's rows first, then the other rows.  Against a panel over all rows the block needs fewer
@@ -107,7 +109,7 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
     if (probe) {
       // two narrow panels and one three quarters of the grid wide: compute-bound shapes want the wide one (16384^3: five
       // or six of eight), and a probe without it misjudged 2048-tiles by 8 % (16384 x 8192 x 16384)
-      const int wide = (3 * g + 2) / 4;
+      const int wide = std::min((3 * g + 2) / 4, ORDER_FULL_PANEL - 1);
       for (int w : probe_widths)
         if (w < g) ids.push_back(order_id_of(orient, w));
       if (wide < g && wide != probe_widths[0] && wide != probe_widths[1]) ids.push_back(order_id_of(orient, wide));
@@ -115,7 +117,7 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
       for (int w : widths)
         if (w < g) ids.push_back(order_id_of(orient, w));
     }
-    ids.push_back(order_id_of(orient, g));
+    ids.push_back(order_id_of(orient, std::min(g, ORDER_FULL_PANEL)));   // the whole grid as one k-outer panel
   }
   // blocks one or two tiles short of the grid in each direction (full pool only: a block order re-reads nothing)
   if (!limited && p.Mg() > 1 && p.Ng() > 1)
@@ -137,7 +139,7 @@ std::vector<int> gemm_candidate_orders(const GemmProblem& p, bool probe, bool me
         // pool, and the next wider one: the best width of a limited pool sits there, and a probe without it can misjudge
         // the tile size by 15 %
         const int other = orient == 0 ? p.Mg() : p.Ng();
-        const int fit = (int)std::max<long>(1, (p.pool_blocks - other) / (other + 1));
+        const int fit = (int)std::min<long>(ORDER_FULL_PANEL - 2, std::max<long>(1, (p.pool_blocks - other) / (other + 1)));
         int ws[4] = {probe_widths[0], probe_widths[1], fit, fit + 1};
         for (int i = 0; i < 4; ++i) {
           bool seen = false;

@@ -99,6 +99,9 @@ constexpr int ORDER_MERGE_CHAINS = 80000;
 // then the other rows).  Its C tiles are complete after (rows + columns) * Kg fetched tiles instead of (Mg + w) * Kg,
 // so write-backs start earlier: for shapes bounded by the link (dgemm 8192^3 from the host: 24.7 -> 23.3 ms).
 constexpr int ORDER_BLOCK_ROWS = 100;
+// Panel widths therefore stay below 100, and w = 99 stands for "the whole grid", however many tiles that is (a grid of
+// 128 column tiles would otherwise read as the block 1 x 28).
+constexpr int ORDER_FULL_PANEL = 99;
 // + 160000 * s: thin start (GemmProblem::k_split) with 2^s slabs, s = 1 or 2.
 constexpr int ORDER_K_SPLIT = 160000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }

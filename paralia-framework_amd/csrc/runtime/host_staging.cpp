@@ -197,13 +197,16 @@ void HostStager::write_back_deferred(void* dst, long ld_dst, const void* src, lo
                                      void* const* after, int n_after) {
   if (rows <= 0 || cols <= 0) return;
   reserve((long long)rows * cols * elem);
-  Request r{dst, ld_dst, src, rows, cols, elem, stream, {nullptr}, std::min(n_after, 12)};
+  // a dropped wait would let the copy start before the tile's kernels have finished
+  if (n_after < 0 || n_after > MAX_DEFERRED_WAITS) throw paralia_error(PL_ERR_ARG, "deferred write-back: too many events to wait for");
+  Request r{dst, ld_dst, src, rows, cols, elem, stream, {nullptr}, n_after};
   for (int i = 0; i < r.n_after; ++i) r.after[i] = after[i];
   {
     std::lock_guard<std::mutex> lk(dmu_);
     if (!deferred_.joinable()) {
       // two threads scatter a 32 MiB tile in 0.85 ms against 0.6 ms on the link; the cores stay with the gathers
       deferred_pool_ = new CopyThreads(2);
+      chk(pl_get_device(&device_), "get device");
       deferred_ = std::thread([this] { deferred_loop(); });
     }
     requests_.push_back(r);
@@ -217,6 +220,7 @@ void HostStager::deferred_loop() {
   struct Flight { int slot; Request r; };
   std::deque<Flight> flying;
   int next_slot = 0;
+  pl_set_device(device_);   // a new thread starts on device 0: the streams and events it is handed belong to device_
   std::unique_lock<std::mutex> lk(dmu_);
   for (;;) {
     dcv_.wait(lk, [&] { return stop_ || !requests_.empty() || !flying.empty(); });

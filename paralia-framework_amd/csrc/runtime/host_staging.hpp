@@ -53,6 +53,7 @@ class CopyThreads {
 // Ring of pinned slots for tiles on their way to the device, and a second ring for tiles coming back.
 class HostStager {
  public:
+  static constexpr int MAX_DEFERRED_WAITS = 12;   // events a deferred write-back may wait for (the plan's MAX_WAITS)
   HostStager() = default;
   ~HostStager();
   HostStager(const HostStager&) = delete;
@@ -97,8 +98,9 @@ class HostStager {
   // deferred write-backs: requests in call order; the background thread owns the out_ slots while any are open
   struct Request {
     void* dst; long ld; const void* src; long rows, cols; int elem; void* stream;
-    void* after[12]; int n_after;
+    void* after[MAX_DEFERRED_WAITS]; int n_after;
   };
+  int device_ = 0;             // device that was current when the background thread was started; the thread makes it its own
   void deferred_loop();
   std::thread deferred_;
   CopyThreads* deferred_pool_ = nullptr;

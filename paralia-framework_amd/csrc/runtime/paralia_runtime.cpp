@@ -6,6 +6,7 @@
 // sgemm.cpp:296, daxpy.cpp:200, ddot.cpp:201, Subkernel.cpp:249-306 (queue inventory), :488 (cache free).
 // All device work goes through the C ABI in paralia_hip.h; this file includes no HIP header.
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -323,13 +324,20 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   if (pageable[0] || pageable[1] || pageable[2]) stager.reserve((long long)Tt * Tt * (long long)sizeof(T));
   StagerScope staged(stager);
   // what the tile kernel can use to split K when a tile product has too few workgroups (small T): the largest need
-  // over the full and the ragged tile extents
+  // over the launches of the plan -- full and ragged tile extents, slabs of a thin start, and merged chains, whose one
+  // launch covers the summed k of their tiles
   long ws_bytes = 0;
-  for (int e = 0; e < 12; ++e) {
-    const long m = (e & 1) ? p.tm(p.Mg() - 1) : std::min<long>(Tt, p.M), n = (e & 2) ? p.tn(p.Ng() - 1) : std::min<long>(Tt, p.N);
-    // a full k tile, the last one, or a slab of the thin start
-    const long k = p.Kg() > 0 ? (e / 4 == 1 ? p.tk(p.Kg() - 1) : e / 4 == 2 ? p.tk(0) : std::min<long>(Tt, p.K)) : 0;
-    ws_bytes = std::max(ws_bytes, pl_gemm_tile_workspace_bytes(m, n, k, (int)sizeof(T)));
+  {
+    std::vector<std::array<long, 3>> seen;
+    for (const Cmd& c : plan.cmds) {
+      if (c.kind != CMD_GEMM) continue;
+      long k = 0;
+      for (int kt = c.ki; kt < c.ki + c.kn; ++kt) k += p.tk(kt);
+      const std::array<long, 3> shape = {p.tm(c.mi), p.tn(c.ni), k};
+      if (std::find(seen.begin(), seen.end(), shape) != seen.end()) continue;
+      seen.push_back(shape);
+      ws_bytes = std::max(ws_bytes, pl_gemm_tile_workspace_bytes(shape[0], shape[1], shape[2], (int)sizeof(T)));
+    }
   }
   void* ws[MAX_EXEC_QUEUES] = {nullptr};
   if (ws_bytes > 0)
@@ -426,6 +434,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         const long m = p.tm(c.mi), n = p.tn(c.ni);
         T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
         if (deferred) {
+          static_assert(MAX_WAITS <= HostStager::MAX_DEFERRED_WAITS, "a deferred write-back must be able to carry every wait of a command");
           void* after[MAX_WAITS];
           for (int w = 0; w < c.nwait; ++w) after[w] = ev[c.wait[w]];
           stager.write_back_deferred(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s, after, c.nwait);

@@ -494,6 +494,30 @@ def test_block_orders(pkg):
         assert stats[5] == 4 * 4 * (4 if order < 160000 else 5)
 
 
+def test_whole_grid_panel_on_grids_of_a_hundred_tiles_and_more(pkg, L):
+    """Panel widths live below 100 in the order id (100 and above encode blocks), and 99 stands for the whole grid.  On a
+    128 x 128 grid of C tiles (M = N = 32768 at T = 256) the whole-grid panel is still a candidate and is planned as one:
+    the first k-step fires all 128 x 128 subkernels before the second starts."""
+    import ctypes as C
+    T, g = 256, 128
+    M = N = g * T
+    rows, stats = pkg.plan_rows(M, N, 2 * T, T, 1, 1, 0, 0, 8, 2, 0, 99)
+    gem = [(r["mi"], r["ni"], r["ki"]) for r in rows if r["kind"] == GEMM]
+    assert len(gem) == g * g * 2 and all(ki == 0 for (_, _, ki) in gem[:g * g]) and all(ki == 1 for (_, _, ki) in gem[g * g:])
+    assert sorted((mi, ni) for (mi, ni, _) in gem[:g * g]) == [(mi, ni) for mi in range(g) for ni in range(g)]
+    rows10, _ = pkg.plan_rows(M, N, 2 * T, T, 1, 1, 0, 0, 8, 2, 0, 10099)
+    assert [(r["mi"], r["ni"], r["ki"]) for r in rows10 if r["kind"] == GEMM][:g * g] == gem[:g * g]
+    # width 98 is a panel of 98 columns, not the grid
+    rows98, _ = pkg.plan_rows(M, N, 2 * T, T, 1, 1, 0, 0, 8, 2, 0, 98)
+    gem98 = [(r["mi"], r["ni"], r["ki"]) for r in rows98 if r["kind"] == GEMM]
+    assert all(ni < 98 for (_, ni, _) in gem98[:2 * g * 98]) and gem98[2 * g * 98][1] == 98
+    # the order search still simulates the whole-grid panel on such a grid: pinned to it, the simulator accepts the id
+    picked = C.c_int(-1)
+    busy = (C.c_double * 3)()
+    t = L.PARALiA_gemm_plan_simulate(M, N, 2 * T, T, 1, 1, 0, 0, 8, 2, 0, 99, 1e-5, 1e-6, 1e-11, 1e-6, 1e-11, 1e-6, 1.0, 1.0, C.byref(picked), busy)
+    assert t > 0 and picked.value == 99
+
+
 def test_unknown_order_ids_are_refused(pkg):
     for order in (480000, 640001, -5):
         with pytest.raises(pkg.ParaliaError, match="unknown order id"):
