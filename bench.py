@@ -49,14 +49,28 @@ def load_package():
 
 
 def traffic_from_profile():
-    """HBM bytes of one headline call as measured with rocprofv3 --pmc (the summary file states how); None when the
-    file has no such line."""
+    """HBM bytes of one headline call as measured with rocprofv3 --pmc (the summary file states how), together with the
+    plan the counters were taken on (order id, tile launches per call): (bytes, order_id, launches), each None when
+    the file has no such line.  Counters cannot be read inside an unprofiled run, so the figure is only reported when
+    the run's own plan is the one that was profiled."""
     try:
         text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
     except OSError:
-        return None
-    m = re.search(r"^hbm_bytes_per_call:\s*([0-9.eE+]+)", text, re.M)
-    return float(m.group(1)) if m else None
+        return None, None, None
+
+    def field(name, conv):
+        m = re.search(r"^%s:\s*([0-9.eE+]+)" % name, text, re.M)
+        return conv(m.group(1)) if m else None
+    return field("hbm_bytes_per_call", float), field("measured_on_order_id", int), field("measured_on_launches_per_call", int)
+
+
+def duplex_bound_ms(b_in, b_out, h_alone, d_alone, h_both, d_both):
+    """Shortest time to move b_in bytes towards the device and b_out bytes back when the two directions run at
+    h_both / d_both B/s while both are busy and at h_alone / d_alone once one of them has finished."""
+    t_in, t_out = b_in / h_both, b_out / d_both
+    if t_in <= t_out:
+        return (t_in + (b_out - d_both * t_in) / d_alone) * 1e3
+    return (t_out + (b_in - h_both * t_out) / h_alone) * 1e3
 
 
 def union_length(intervals):
@@ -185,8 +199,13 @@ def main():
 
     # ------------------------------------------------------------------ headline: host-resident PARALiADgemm
     t0 = time.perf_counter()
-    step_host()                         # cold call: autotune, plan, block pool allocation
+    step_host()                         # cold call: autotune, plan, block pool allocation, stream placement
     t_cold = time.perf_counter() - t0
+    ph = (C.c_double * 6)()
+    pkg.check(L.PARALiA_last_call_phases(ph), "phases")
+    cold_phases = {"autotune_ms": ph[0] * 1e3, "plan_ms": ph[1] * 1e3, "pool_alloc_ms": ph[2] * 1e3, "stream_setup_ms": ph[3] * 1e3,
+                   "execute_ms": ph[4] * 1e3, "call_ms": ph[5] * 1e3,
+                   "note": "host-side phases of the first call; the first kernel launch of the process also loads the code objects (inside execute_ms)"}
     for _ in range(args.warmup):
         step_host()
     sync()
@@ -236,12 +255,63 @@ def main():
     h2d = copy_rate(tile.ptr, T, hA.ptr, n)
     d2h_src = Buf(pkg, T * T, np.float64, -1)     # not into C: the result is still needed
     d2h = copy_rate(d2h_src.ptr, T, tile.ptr, T)
+    # dense tiles (what the BLAS-1 routines and dense operands move), and both directions at once on two streams
+    h2d_dense = copy_rate(tile.ptr, T, hA.ptr, T)
+    s2 = stream()
+    tile2 = Buf(pkg, T * T, np.float64, 0)
+
+    def duplex():
+        for _ in range(2):
+            pkg.check(L.pl_copy2d_async(tile.ptr, T, hA.ptr, n, T, T, 8, s), "copy")
+            pkg.check(L.pl_copy2d_async(d2h_src.ptr, T, tile2.ptr, T, T, T, 8, s2), "copy")
+        pkg.check(L.pl_stream_sync(s), "sync")
+        pkg.check(L.pl_stream_sync(s2), "sync")
+        e = [event() for _ in range(4)]
+        pkg.check(L.pl_event_record(e[0], s), "record")
+        pkg.check(L.pl_event_record(e[2], s2), "record")
+        for _ in range(12):
+            pkg.check(L.pl_copy2d_async(tile.ptr, T, hA.ptr, n, T, T, 8, s), "copy")
+            pkg.check(L.pl_copy2d_async(d2h_src.ptr, T, tile2.ptr, T, T, T, 8, s2), "copy")
+        pkg.check(L.pl_event_record(e[1], s), "record")
+        pkg.check(L.pl_event_record(e[3], s2), "record")
+        pkg.check(L.pl_stream_sync(s), "sync")
+        pkg.check(L.pl_stream_sync(s2), "sync")
+        pkg.check(L.pl_event_elapsed_ms(e[0], e[1], C.byref(ms)), "elapsed")
+        t_in = ms.value * 1e-3
+        pkg.check(L.pl_event_elapsed_ms(e[2], e[3], C.byref(ms)), "elapsed")
+        t_out = ms.value * 1e-3
+        for x in e:
+            L.pl_event_destroy(x)
+        return 12.0 * T * T * 8 / t_in, 12.0 * T * T * 8 / t_out
+    h2d_both, d2h_both = duplex()
+    # 256 MiB spans in 64 KiB columns, the way the BLAS-1 routines move their vector tiles: the per-copy latency all but vanishes
+    big = Buf(pkg, 1 << 25, np.float64, 0)
+
+    def span_rate(dst, src):
+        pkg.check(L.pl_copy2d_async(dst, 8192, src, 8192, 8192, 4096, 8, s), "copy")
+        pkg.check(L.pl_stream_sync(s), "sync")
+        t0 = time.perf_counter()
+        for _ in range(3):
+            pkg.check(L.pl_copy2d_async(dst, 8192, src, 8192, 8192, 4096, 8, s), "copy")
+        pkg.check(L.pl_stream_sync(s), "sync")
+        return 3.0 * (1 << 28) / (time.perf_counter() - t0)
+    h2d_span = span_rate(big.ptr, hA.ptr)
+    span_host = Buf(pkg, 1 << 25, np.float64, -1)
+    d2h_span = span_rate(span_host.ptr, big.ptr)
+    big.free()
+    span_host.free()
+    link = {"h2d": max(h2d, h2d_dense, h2d_span), "d2h": max(d2h, d2h_span), "h2d_strided_tiles": h2d, "h2d_dense_tiles": h2d_dense,
+            "h2d_256MiB_span": h2d_span, "d2h_tiles": d2h, "d2h_256MiB_span": d2h_span,
+            "h2d_while_d2h_runs": min(h2d_both, max(h2d, h2d_dense)), "d2h_while_h2d_runs": min(d2h_both, d2h),
+            "note": "B/s, measured in this run on the library's copy call (32 MiB tiles, and 256 MiB spans); h2d / d2h are the best of them and price the roofs of the link-bound configurations below"}
     tile.free()
+    tile2.free()
     d2h_src.free()
+    pkg.check(L.pl_stream_destroy(s2), "stream destroy")
     b_h2d, b_d2h = 2.0 * n * n * 8, 1.0 * n * n * 8     # beta == 0: C is not fetched
     legs = {"mfma_ms": flops / FP64_MFMA_PEAK * 1e3, "h2d_ms_measured_link": b_h2d / h2d * 1e3, "d2h_ms_measured_link": b_d2h / d2h * 1e3,
             "h2d_ms_at_64GBps": b_h2d / PCIE_THEORETICAL * 1e3, "d2h_ms_at_64GBps": b_d2h / PCIE_THEORETICAL * 1e3}
-    roof_ms = max(legs["mfma_ms"], legs["h2d_ms_measured_link"], legs["d2h_ms_measured_link"])
+    roof_ms = max(legs["mfma_ms"], legs["h2d_ms_measured_link"], legs["d2h_ms_measured_link"])   # legs at the tile-copy rates: what this call's copies can reach
     bound = "mfma" if roof_ms == legs["mfma_ms"] else "pcie"
     kernel = None
     if timeline:
@@ -252,12 +322,17 @@ def main():
                   "tflops_while_a_kernel_runs": timeline["tflops_while_a_kernel_runs"],
                   "frac_of_peak_while_a_kernel_runs": (timeline["tflops_while_a_kernel_runs"] or 0) * 1e12 / FP64_MFMA_PEAK,
                   "profile": "profiles/dgemm_16384_host_operands_kernel_and_copy_trace.txt"}
-    traffic = traffic_from_profile() if n == 16384 else None
+    traffic, traffic_order, traffic_launches = traffic_from_profile() if n == 16384 else (None, None, None)
+    traffic_plan = {"order_id": traffic_order, "launches_per_call": traffic_launches}
+    this_plan = {"order_id": int(info.order_id), "launches_per_call": timeline["launches_per_call"] if timeline else None}
+    if traffic is not None and traffic_plan != this_plan:
+        traffic = None      # the counters were taken on another plan than the one this run executed
     roofline = {"bound": bound, "achieved": flops / t_step / 1e12, "peak": FP64_MFMA_PEAK / 1e12, "unit": "TFLOP/s",
                 "frac": roof_ms / (t_step * 1e3), "roof": "min(FP64 MFMA peak, PCIe-bound rate): roof_ms = max(F / 78.6 TFLOP/s, B_h2d / BW_h2d, B_d2h / BW_d2h)",
                 "roof_ms": roof_ms, "legs": legs, "flop_per_call": flops, "h2d_bytes_per_call": b_h2d, "d2h_bytes_per_call": b_d2h,
                 "h2d_GBps_measured": h2d / 1e9, "d2h_GBps_measured": d2h / 1e9,
-                "traffic": traffic, "traffic_source": TRAFFIC_PROFILE if traffic else None,
+                "traffic": traffic, "traffic_source": TRAFFIC_PROFILE, "traffic_measured_on_plan": traffic_plan, "plan_of_this_run": this_plan,
+                "link_rates_measured": link,
                 "algorithmic_hbm_bytes_per_call": 3.0 * n * n * 8, "dominant_kernel": kernel, "timeline": timeline}
 
     # ------------------------------------------------------------------ the same product, operands already in HBM
@@ -331,20 +406,37 @@ def main():
                    "T_selected_by": info.selected_by.decode(), "subkernels": int(info.subkernel_num), "order_id": int(info.order_id),
                    "predicted_ms": info.pred_t * 1e3, "GPU_MAX_HW_QUEUES": os.environ.get("GPU_MAX_HW_QUEUES"),
                    "independent_scheduler_streams": ind.value, "streams_created_to_find_them": made.value},
-        "min_ms": min(times) * 1e3, "max_ms": max(times) * 1e3, "cold_call_ms": t_cold * 1e3,
+        "min_ms": min(times) * 1e3, "max_ms": max(times) * 1e3, "cold_call_ms": t_cold * 1e3, "cold_call_phases": cold_phases,
         "parity_checksum_err": parity,
         "roofline": roofline, "cpu_baseline": cpu, "device_resident": device_resident,
     }
 
     if args.other_configs and n == 16384:
         try:
-            out["other_configs"] = other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu)
+            out["other_configs"] = other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu, link)
         except Exception as e:  # the headline line must come out whatever happens in the extras
             out["other_configs"] = {"error": str(e)[:300]}
+    out["fractions_above_one"] = sorted(set(fractions_above_one(out)))
     print(json.dumps(out))
 
 
-def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
+def fractions_above_one(node, path=""):
+    """Every reported fraction of a roof that exceeds 1 (none should: a roof is a bound)."""
+    found = []
+    if isinstance(node, dict):
+        for k, v in node.items():
+            here = path + "/" + str(k)
+            if isinstance(v, (dict, list)):
+                found += fractions_above_one(v, here)
+            elif isinstance(v, float) and "frac" in str(k) and v > 1.0:
+                found.append(here)
+    elif isinstance(node, list):
+        for i, v in enumerate(node):
+            found += fractions_above_one(v, path + "/%d" % i)
+    return found
+
+
+def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu, link):
     """The remaining BASELINE.json configurations, each with its own roof.  hA / hB / hC are the 2 GiB pinned buffers of
     the headline (2^28 doubles each), dA / dB / dC their device twins."""
     import oracle_binding as ob
@@ -392,8 +484,9 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
         bytes_in = 3.0 * m1 * m1 * 8        # beta != 0: C is fetched too
         row = {"workload": "dgemm 4096^3 fp64 NN alpha=1.2 beta=1.1, A/B/C pinned host (BASELINE config 1 on the GPU path)",
                "ms_per_call": t * 1e3, "min_ms": tmin * 1e3, "max_ms": tmax * 1e3, "gflops": f1 / t / 1e9, "T": int(inf.T),
-               "predicted_ms": inf.pred_t * 1e3, "roof": "H2D of A, B and C (4.03e8 B) at the measured 56.25 GB/s", "roof_ms": bytes_in / 56.25e9 * 1e3,
-               "frac_of_roof": bytes_in / 56.25e9 / t}
+               "predicted_ms": inf.pred_t * 1e3, "roof": "H2D of A, B and C (4.03e8 B) at the H2D rate measured in this run", "roof_ms": bytes_in / link["h2d"] * 1e3,
+               "frac_of_roof": bytes_in / link["h2d"] / t,
+               "duplex_roof_ms": duplex_bound_ms(bytes_in, m1 * m1 * 8.0, link["h2d"], link["d2h"], link["h2d_while_d2h_runs"], link["d2h_while_h2d_runs"])}
         if have_blas:
             ref = c0.copy()
             orc.orc_openblas_dgemm(b"N", b"N", m1, m1, m1, 1.2, a1.ptr, m1, b1.ptr, m1, 1.1, ob.ptr(ref), m1)   # warm-up, and the parity reference
@@ -416,19 +509,23 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
     # ---- config 2, device-resident: daxpy / ddot N = 2^28 (and dgemv on the same 2 GiB as a 16384^2 matrix)
     nd = 1 << 28
     try:
-        t_ax = timed_events(lambda: pkg.check(L.pl_daxpy(nd, 0.7, dA.ptr, 1, dB.ptr, 1, s), "daxpy"), 20, 5)
-        # where the two vectors lie in HBM changes the daxpy rate by a few percent: repeat on fresh allocations and
-        # report the slowest as well
-        per_alloc = [t_ax]
-        for _ in range(4):
-            fx, fy = Buf(pkg, nd, np.float64, 0), Buf(pkg, nd, np.float64, 0)
-            per_alloc.append(timed_events(lambda: pkg.check(L.pl_daxpy(nd, 0.7, fx.ptr, 1, fy.ptr, 1, s), "daxpy"), 10, 3))
-            fx.free()
-            fy.free()
+        # Nothing is freed between these measurements: for a few seconds after a hipFree of gigabytes the device works on
+        # the released memory, and a streaming kernel measured meanwhile loses about 5 % (ddot 0.636 instead of 0.609 ms).
         ws = Buf(pkg, max(int(L.pl_ddot_workspace_doubles()), int(L.pl_dgemv_workspace_doubles(b"N", 16384, 16384))) + 1, np.float64, 0)
         res, yv = Buf(pkg, 1, np.float64, 0), Buf(pkg, 16384, np.float64, 0)
+        t_ax = timed_events(lambda: pkg.check(L.pl_daxpy(nd, 0.7, dA.ptr, 1, dB.ptr, 1, s), "daxpy"), 20, 5)
         t_dot = timed_events(lambda: pkg.check(L.pl_ddot(nd, dA.ptr, 1, dB.ptr, 1, res.ptr, 0, ws.ptr, s), "ddot"), 20)
         t_mv = timed_events(lambda: pkg.check(L.pl_dgemv(b"N", 16384, 16384, 1.2, dA.ptr, 16384, dB.ptr, 1, 1.1, yv.ptr, 1, ws.ptr, s), "dgemv"), 20)
+        # where the two vectors lie in HBM changes the rates by a few percent: repeat on fresh allocations (all held until
+        # the last one has been measured) and report the slowest as well
+        per_alloc, per_alloc_dot, fresh = [t_ax], [t_dot], []
+        for _ in range(4):
+            fx, fy = Buf(pkg, nd, np.float64, 0), Buf(pkg, nd, np.float64, 0)
+            fresh += [fx, fy]
+            per_alloc.append(timed_events(lambda: pkg.check(L.pl_daxpy(nd, 0.7, fx.ptr, 1, fy.ptr, 1, s), "daxpy"), 10, 3))
+            per_alloc_dot.append(timed_events(lambda: pkg.check(L.pl_ddot(nd, fx.ptr, 1, fy.ptr, 1, res.ptr, 0, ws.ptr, s), "ddot"), 10, 3))
+        for b in fresh:
+            b.free()
         mv_bytes = 8.0 * (16384.0 * 16384 + 3 * 16384)
         other["blas1_2p28_device"] = {
             "workload": "daxpy / ddot N=2^28 fp64 alpha=0.7, x and y in HBM (BASELINE config 2, device-resident), HIP events",
@@ -436,6 +533,8 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
             "daxpy_GBps_per_fresh_allocation": [24.0 * nd / t / 1e9 for t in per_alloc],
             "daxpy_min_frac_of_hbm_peak": 24.0 * nd / max(per_alloc) / HBM_PEAK,
             "ddot_GBps": 16.0 * nd / t_dot / 1e9, "ddot_ms": t_dot * 1e3, "ddot_frac_of_hbm_peak": 16.0 * nd / t_dot / HBM_PEAK,
+            "ddot_GBps_per_fresh_allocation": [16.0 * nd / t / 1e9 for t in per_alloc_dot],
+            "ddot_min_frac_of_hbm_peak": 16.0 * nd / max(per_alloc_dot) / HBM_PEAK,
             "dgemv_16384_GBps": mv_bytes / t_mv / 1e9, "dgemv_16384_frac_of_hbm_peak": mv_bytes / t_mv / HBM_PEAK}
         for b in (ws, res, yv):
             b.free()
@@ -443,6 +542,7 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
         other["blas1_2p28_device"] = {"error": str(e)[:200]}
     for b in (dA, dB, dC):
         b.free()
+    time.sleep(3.0)     # 22 GiB went back to the driver just now: let it finish with them before the link is timed
 
     # ---- config 2, host-resident in pinned memory: PCIe-bound (x = the headline's A, y = its C buffer)
     try:
@@ -451,12 +551,14 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
         T_ax = int(inf.T)
         r = C.c_double(0.0)
         t_dot, dot_min, _ = wall(lambda: pkg.check(L.PARALiA_ddot(nd, hA.ptr, 1, hB.ptr, 1, C.byref(r), -1, C.byref(inf)), "ddot host"), 5, 2)
-        roof = 16.0 * nd / 56.25e9     # both vectors cross the link towards the device; daxpy's y returns in the other direction
+        roof = 16.0 * nd / link["h2d"]     # both vectors cross the link towards the device; daxpy's y returns in the other direction
+        ax_duplex = duplex_bound_ms(16.0 * nd, 8.0 * nd, link["h2d"], link["d2h"], link["h2d_while_d2h_runs"], link["d2h_while_h2d_runs"]) * 1e-3
         row = {"workload": "daxpy / ddot N=2^28 fp64, x and y in pinned host memory (BASELINE config 2, host-resident)",
                "daxpy_ms": t_ax * 1e3, "daxpy_min_ms": ax_min * 1e3, "daxpy_link_GBps": 16.0 * nd / t_ax / 1e9, "daxpy_T": T_ax,
                "ddot_ms": t_dot * 1e3, "ddot_min_ms": dot_min * 1e3, "ddot_link_GBps": 16.0 * nd / t_dot / 1e9, "ddot_T": int(inf.T),
-               "roof": "H2D of x and y (4.295e9 B) at the measured 56.25 GB/s", "roof_ms": roof * 1e3,
-               "daxpy_frac_of_roof": roof / t_ax, "ddot_frac_of_roof": roof / t_dot}
+               "roof": "H2D of x and y (4.295e9 B) at the H2D rate measured in this run", "roof_ms": roof * 1e3,
+               "daxpy_duplex_roof_ms": ax_duplex * 1e3, "daxpy_duplex_roof": "x and y in, y out at the rates measured with both directions busy",
+               "daxpy_frac_of_roof": roof / t_ax, "daxpy_frac_of_duplex_roof": ax_duplex / t_ax, "ddot_frac_of_roof": roof / t_dot}
         if have_blas:
             # OpenBLAS on the same vectors, 1 warm-up + 3 timed
             yb = np.array(hC.host_view()[:nd])
@@ -482,7 +584,7 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
     for b in (hA, hB, hC):
         b.free()
 
-    def streamed(tag, fn, dtype, ta, tb, M, N, K, alpha, beta, locs, roof_ms, roof_note, T_list=(-1,)):
+    def streamed(tag, fn, dtype, ta, tb, M, N, K, alpha, beta, locs, roof_ms, roof_note, T_list=(-1,), duplex_roof_ms=None):
         try:
             ra, ca = (M, K) if ta == b"N" else (K, M)
             rb, cb = (K, N) if tb == b"N" else (N, K)
@@ -505,6 +607,9 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
             pick = rows[list(T_list).index(-1)]
             row = dict(pick)
             row.update({"roof_ms": roof_ms, "roof": roof_note})
+            if duplex_roof_ms is not None:
+                row.update({"duplex_roof_ms": duplex_roof_ms, "frac_of_duplex_roof": duplex_roof_ms / row["ms_per_call"],
+                            "duplex_roof": "all bytes in and all bytes out at the rates measured with both directions busy, the rest at the one-way rate"})
             sweep = [r for r, Tset in zip(rows, T_list) if Tset > 0]
             if sweep:
                 row["T_sweep"] = sorted(sweep, key=lambda r: r["T"])
@@ -521,8 +626,15 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu):
     streamed("sgemm_32768_NT_AB_host_C_device", L.PARALiA_sgemm, np.float32, b"N", b"T", 32768, 32768, 32768, 1.0, 1.0, (-1, -1, 0),
              2.0 * 32768 ** 3 / FP32_MFMA_PEAK * 1e3, "fp32 MFMA peak 157.3 TFLOP/s (H2D of A and B, 8.59e9 B, takes 153 ms)")
     streamed("dgemm_40000x40000x2048_host_beta0.5", L.PARALiA_dgemm, np.float64, b"N", b"N", 40000, 40000, 2048, 1.5, 0.5, (-1, -1, -1),
-             (40000.0 * 2048 * 2 + 40000.0 * 40000) * 8 / 56.25e9 * 1e3, "PCIe: H2D of A, B and C (1.411e10 B) at the measured 56.25 GB/s",
-             T_list=(8192, -1, 4096, 2048, 1024))
+             (40000.0 * 2048 * 2 + 40000.0 * 40000) * 8 / link["h2d"] * 1e3, "PCIe: H2D of A, B and C (1.411e10 B) at the H2D rate measured in this run",
+             T_list=(8192, -1, 4096, 2048, 1024),
+             duplex_roof_ms=duplex_bound_ms((40000.0 * 2048 * 2 + 40000.0 * 40000) * 8, 40000.0 * 40000 * 8, link["h2d"], link["d2h"],
+                                            link["h2d_while_d2h_runs"], link["d2h_while_h2d_runs"]))
+    # dgemm 8192^3 from the host: the mid-size shape the link bounds (H2D of A and B against 14 ms of compute)
+    streamed("dgemm_8192_host_beta0", L.PARALiA_dgemm, np.float64, b"N", b"N", 8192, 8192, 8192, 1.0, 0.0, (-1, -1, -1),
+             2.0 * 8192 * 8192 * 8 / link["h2d"] * 1e3, "PCIe: H2D of A and B (1.07e9 B) at the H2D rate measured in this run",
+             duplex_roof_ms=duplex_bound_ms(2.0 * 8192 * 8192 * 8, 8192.0 * 8192 * 8, link["h2d"], link["d2h"],
+                                            link["h2d_while_d2h_runs"], link["d2h_while_h2d_runs"]))
     return other
 
 

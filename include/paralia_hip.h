@@ -197,6 +197,12 @@ int PARALiA_runtime_shutdown(void);
 #define PL_TRACE_ROW 7
 int PARALiA_trace_enable(int on);
 long PARALiA_trace_read(double* rows, long max_rows);
+/* host-side phases of the most recent PARALiA_dgemm / PARALiA_sgemm call, in seconds: [0] autotune (database lookups,
+ * tile and order search), [1] plan (static plan of the chosen order), [2] device block pool (allocation or growth),
+ * [3] streams (creation and placement test), [4] execution (enqueue, device work, final sync), [5] whole call.  [0] and
+ * [1] are 0 when the problem came from the metadata cache.  What the reference's TEST build prints per call
+ * (dgemm.cpp:330-333,430-445,497-511,598-604). */
+int PARALiA_last_call_phases(double seconds[6]);
 /* the scheduler's stream inventory: *independent <- how many of its four busy streams (H2D, D2H, two compute) were
  * found to sit on hardware queues of their own (4 unless the process has fewer than four hardware queues), *created <-
  * how many streams it created to find them; both 0 before the first call that needs streams.  No counterpart in the

@@ -85,6 +85,7 @@ _SIGS = {
     "PARALiA_runtime_stats": (_i, [C.POINTER(_l), C.POINTER(_l), C.POINTER(_ll), C.POINTER(_l)]),
     "PARALiA_runtime_reset": (_i, []),
     "PARALiA_stream_queues": (_i, [_pi, _pi]),
+    "PARALiA_last_call_phases": (_i, [C.POINTER(_d)]),
     "PARALiA_runtime_shutdown": (_i, []),
     "PARALiA_trace_enable": (_i, [_i]),
     "PARALiA_trace_read": (_l, [C.POINTER(_d), _l]),

@@ -306,6 +306,8 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
     st.tr_idle = m->transient_idle_s;
     st.tr_recover = m->transient_recover_s;
   }
+  const char* search = getenv("PARALIA_PLAN_SEARCH");  // "exhaustive": no candidate is dismissed by a bound
+  st.exhaustive = search && !strcmp(search, "exhaustive");
   const char* blk = getenv("PARALIA_BLOCK_ORDERS");  // "0": never start with a block of C tiles smaller than a full panel
   st.block_orders = !(blk && *blk && atoi(blk) == 0);
   return st;
@@ -349,6 +351,8 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
   pipeline = PipelineEstimate();
 
   if (problem.problem == BLAS3) {
+    int searched_order = -1;            // order search result of the tile size the pipeline model chose, if it ran
+    paralia::PipelineResult searched_r;
     const long min_dim = std::min(problem.D1, std::min(problem.D2, problem.D3));
     const long max_dim = std::max(problem.D1, std::max(problem.D2, problem.D3));
     if (T > 0) {
@@ -369,8 +373,13 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       // Two passes over the benchmarked tile sizes.  The first prices each T with a handful of representative
       // subkernel orders (largest tiles first: they have few subkernels and are cheap to simulate, and once a good
       // makespan is known the small tiles, whose kernels alone already take longer than that, are dismissed without
-      // building a plan).  The second runs the full order search only for the (at most three) T whose penalised probe is within 10 % of the best.
-      struct Cand { long T; double probe_t; };
+      // building a plan).  The second runs the full order search for the (at most three) T whose penalised probe is
+      // within 10 % of the best, best probe first, and skips a T whose floor is above a result already in hand.
+      struct Cand { long T; double probe_t, floor_t; };
+      const char* verbose_env = getenv("PARALIA_VERBOSE");
+      const bool chatty = verbose_env && atoi(verbose_env) > 1;
+      const char* search_env = getenv("PARALIA_PLAN_SEARCH");
+      const bool exhaustive = search_env && !strcmp(search_env, "exhaustive");
       // predictions of neighbouring T differ by less than the model's accuracy: the reference's penalty terms
       // (ragged edges, too few or too many subkernels, Autotuner.cpp:571-603) break such near-ties
       auto penalty = [&](long cand) {
@@ -379,9 +388,41 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         get_T_slowdowns(sl, (int)cand);
         return 1.0 + 0.02 * sl[0];
       };
-      std::vector<Cand> cands;
+      // What no order of a tile size can beat: the tile kernels run one at a time on the simulated device, so a call
+      // takes at least the sum of its subkernels' times, less what merged K chains can save at most (one saving per
+      // k-step after a C tile's first).  A tile size whose floor is above a makespan already found is dismissed without
+      // building a single plan -- for the small tiles, whose plans have thousands of commands, that is most of the
+      // search's time.
+      auto compute_floor = [&](const paralia::GemmProblem& gp, const paralia::StageTimes& st) {
+        double total = 0;
+        const long kfull = problem.D3 / gp.T, krem = problem.D3 % gp.T;
+        for (int mi = 0; mi < gp.Mg(); ++mi)
+          for (int ni = 0; ni < gp.Ng(); ++ni) {
+            const long m = gp.tm(mi), n = gp.tn(ni);
+            total += kfull * st.exec_time(gp.T, m, n, gp.T) + (krem ? st.exec_time(gp.T, m, n, krem) : 0.0);
+          }
+        const double saved = (double)(gp.subkernels() - (long)gp.Mg() * gp.Ng()) * st.merge_saving;
+        return std::max(0.5 * total, total - saved);
+      };
+      // ... and at both ends nothing overlaps: no kernel starts before the first pair of A and B tiles has crossed the
+      // link (a quarter of each, if the thin start cuts them into four slabs), and the C tile of the last kernel goes
+      // back (after its lazy reduce) when every kernel has finished.
+      auto call_floor = [&](const paralia::GemmProblem& gp, const paralia::StageTimes& st) {
+        double t = compute_floor(gp, st);
+        const double quarter = (double)gp.T * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz;
+        if (gp.a_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(quarter, (double)gp.tm(gp.Mg() - 1) * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz);
+        if (gp.b_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(quarter, (double)gp.tn(gp.Ng() - 1) * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz);
+        if (gp.c_remote) {
+          const double smallest = (double)std::min(gp.tm(0), gp.tm(gp.Mg() - 1)) * std::min(gp.tn(0), gp.tn(gp.Ng() - 1));
+          t += st.d2h_ti + st.d2h_tb * smallest * problem.dtype_sz;
+          if (!gp.beta_zero) t += st.t_reduce * smallest / ((double)gp.T * gp.T);
+        }
+        return t;
+      };
+      // the tile sizes in the order of their floors: a good makespan early dismisses the most
+      struct Entry { long T; double floor_t; paralia::GemmProblem gp; };
+      std::vector<Entry> entries;
       long prev = -1;
-      double best_probe = DBL_MAX;
       for (long i = m->exec->lines() - 1; i >= 0; i--) {
         const long cand = m->exec->T[i];
         if (cand == prev) continue;
@@ -392,18 +433,29 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         if (cand < m->getMinT() && std::min(problem.D1, problem.D2) >= m->getMinT()) continue;
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         if (gp.pool_blocks < 3 || gp.subkernels() > 20000) continue;
-        const paralia::StageTimes st = paralia_stage_times(this, cand);
-        if ((double)gp.subkernels() * st.exec_time(cand, std::min(cand, problem.D1), std::min(cand, problem.D2),
-                                                    std::min(cand, problem.D3)) * 0.9 > best_probe) continue;
+        entries.push_back({cand, call_floor(gp, paralia_stage_times(this, cand)) * penalty(cand), gp});
+      }
+      std::stable_sort(entries.begin(), entries.end(), [](const Entry& x, const Entry& y) { return x.floor_t < y.floor_t; });
+      std::vector<Cand> cands;
+      double best_probe = DBL_MAX, best_probe_score = DBL_MAX;
+      for (const Entry& e : entries) {
+        const long cand = e.T;
+        if (e.floor_t > best_probe_score && !exhaustive) break;   // and so is every floor behind it
         paralia::PipelineResult r;
         try {
-          paralia::pick_gemm_order(gp, st, &r, /*probe=*/true);
+          paralia::pick_gemm_order(e.gp, paralia_stage_times(this, cand), &r, /*probe=*/true);
         } catch (const std::runtime_error&) { continue; }
-        cands.push_back({cand, r.t_total * penalty(cand)});
+        cands.push_back({cand, r.t_total * penalty(cand), e.floor_t});
         best_probe = std::min(best_probe, r.t_total);
+        best_probe_score = std::min(best_probe_score, r.t_total * penalty(cand));
+        if (chatty) fprintf(stderr, "  probe T = %ld: %.3lf ms (floor %.3lf), %ld plans simulated so far\n", cand, r.t_total * 1e3, e.floor_t * 1e3, paralia::plan_simulations.load());
       }
+      // back to table order (largest T first): what the selection below was written for
+      std::sort(cands.begin(), cands.end(), [](const Cand& x, const Cand& y) { return x.T > y.T; });
       long best_T = -1;
       double best_t = DBL_MAX;
+      int best_order = -1;
+      paralia::PipelineResult best_r;
       // at most the three best probes go on (kept in table order, largest T first, so that ties still go to the
       // smaller tile below)
       double cut = DBL_MAX;
@@ -413,17 +465,27 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         std::nth_element(ts.begin(), ts.begin() + 2, ts.end());
         cut = ts[2];
       }
-      for (const Cand& c : cands) {
-        if (c.probe_t > 1.1 * best_probe || c.probe_t > cut) continue;
-        const long cand = c.T;
+      // the full search of the best probe first: its result dismisses the others by their floors
+      std::vector<const Cand*> finalists;
+      for (const Cand& c : cands)
+        if (!(c.probe_t > 1.1 * best_probe || c.probe_t > cut)) finalists.push_back(&c);
+      std::stable_sort(finalists.begin(), finalists.end(), [](const Cand* x, const Cand* y) { return x->probe_t < y->probe_t; });
+      for (const Cand* c : finalists) {
+        if (c->floor_t > best_t && !exhaustive) continue;
+        const long cand = c->T;
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         paralia::PipelineResult r;
+        int oid = -1;
         try {
-          paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
+          oid = paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
         } catch (const std::runtime_error&) { continue; }
         const double score = r.t_total * penalty(cand);
-        if (score <= best_t) { best_t = score; best_T = cand; }  // ties go to the smaller tile (largest T comes first)
+        if (chatty) fprintf(stderr, "  full search T = %ld: %.3lf ms, order %d, %ld plans simulated so far\n", cand, r.t_total * 1e3, oid, paralia::plan_simulations.load());
+        if (score < best_t || (score == best_t && cand < best_T)) {  // ties go to the smaller tile
+          best_t = score; best_T = cand; best_order = oid; best_r = r;
+        }
       }
+      if (best_T >= 0) { searched_order = best_order; searched_r = best_r; }
       if (best_T < 0) {
         // C narrower than every benchmarked tile: one tile across the short side, as square as that allows
         T = std::max(std::min(problem.D1, problem.D2), std::min(max_dim, m->exec->MinT()));
@@ -445,7 +507,9 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       error("PARALiA gemm: Problem cannot run with less memory than %lld\n", 3LL * T * T * problem.dtype_sz);
     paralia::PipelineResult r;
     try {
-      order_id = paralia::pick_gemm_order(gp, paralia_stage_times(this, T), &r);
+      // the tile search has already run the order search of the tile it chose
+      if (searched_order >= 0) { order_id = searched_order; r = searched_r; }
+      else order_id = paralia::pick_gemm_order(gp, paralia_stage_times(this, T), &r);
       // PARALIA_GEMM_ORDER pins the subkernel order family (gemm_plan.hpp) when that order fits the block pool
       const char* o_env = getenv("PARALIA_GEMM_ORDER");
       if (o_env && *o_env) {
@@ -551,6 +615,9 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
   }
   pred_J = -1.0;  // no power sampling on this platform
   const char* verbose = getenv("PARALIA_VERBOSE");
+  if (verbose && atoi(verbose) > 1)
+    fprintf(stderr, "ATC::autotune_problem: %ld plans simulated so far in this process, this search took %.2lf ms\n",
+            paralia::plan_simulations.load(), (csecond() - timer) * 1000);
   if (verbose && atoi(verbose) > 0) {
     fprintf(stderr, "====================================\n");
     fprintf(stderr, "ATC::autotune_problem: %s (%ld,%ld,%ld) -> T = %ld [%s], order %d, %ld subkernels, "

@@ -21,6 +21,7 @@ void cache_free_impl(short);
 void runtime_stats(long*, long*, long long*, long*);
 void runtime_reset();
 void stream_queues(int*, int*);
+void last_call_phases(double*);
 void runtime_shutdown();
 void trace_enable(int);
 long trace_read(double*, long);
@@ -139,6 +140,12 @@ long PARALiA_trace_read(double* rows, long max_rows) {
   long n = -1;
   guarded([&] { n = paralia::trace_read(rows, max_rows); });
   return n;
+}
+int PARALiA_last_call_phases(double seconds[6]) {
+  return guarded([&] {
+    if (!seconds) throw paralia_error(PL_ERR_NULL, "PARALiA_last_call_phases: null output\n");
+    paralia::last_call_phases(seconds);
+  });
 }
 int PARALiA_stream_queues(int* independent, int* created) {
   return guarded([&] { paralia::stream_queues(independent, created); });

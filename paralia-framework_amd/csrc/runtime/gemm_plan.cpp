@@ -3,11 +3,18 @@
 #include "gemm_plan.hpp"
 
 #include <algorithm>
+#include <atomic>
+#include <cfloat>
 #include <climits>
 #include <cmath>
+#include <condition_variable>
+#include <cstdlib>
 #include <deque>
+#include <functional>
+#include <mutex>
 #include <stdexcept>
 #include <string>
+#include <thread>
 
 namespace paralia {
 
@@ -183,7 +190,10 @@ struct Block {
   int idx = -1;
   int content_cmd = -1;        // command after which the content is valid (the fetch)
   int last_touch = -1;         // latest command that wrote or read the content
-  std::vector<int> pending;    // commands that must complete before the block may be overwritten
+  // commands that must complete before the block may be overwritten: at most one per stream (streams run their
+  // commands in order, so the latest of a stream covers the earlier ones)
+  int pending[MAX_WAITS];
+  int npending = 0;
   bool ever_used = false;
 };
 
@@ -225,15 +235,23 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
     throw std::runtime_error("PARALiA gemm: Not able to run with < 3 blocks per cache");
 
   // positions at which every A / B tile is used, for farthest-next-use eviction
-  std::vector<std::vector<int>> a_uses((size_t)Mg * Kg), b_uses((size_t)Kg * Ng);
+  // (every A tile is used by Ng subkernels, every B tile by Mg: two dense tables, rows filled in order of use)
+  struct Uses {
+    int per = 0;
+    std::vector<int> pos, fill;
+    Uses(size_t tiles, int per_tile) : per(per_tile), pos(tiles * (size_t)per_tile), fill(tiles, 0) {}
+    void add(size_t tile, int p) { pos[tile * per + fill[tile]++] = p; }
+    int size(size_t tile) const { return fill[tile]; }
+    int at(size_t tile, int i) const { return pos[tile * per + i]; }
+  } a_uses((size_t)Mg * Kg, Ng), b_uses((size_t)Kg * Ng, Mg);
   for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
     const int t = plan.task_order[pos];
     const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
-    a_uses[(size_t)mi * Kg + ki].push_back(pos);
-    b_uses[(size_t)ki * Ng + ni].push_back(pos);
+    a_uses.add((size_t)mi * Kg + ki, pos);
+    b_uses.add((size_t)ki * Ng + ni, pos);
   }
-  std::vector<int> a_ptr(a_uses.size(), 0), b_ptr(b_uses.size(), 0);
-  std::vector<int> a_blk(a_uses.size(), -1), b_blk(b_uses.size(), -1), c_blk((size_t)Mg * Ng, -1);
+  std::vector<int> a_ptr((size_t)Mg * Kg, 0), b_ptr((size_t)Kg * Ng, 0);
+  std::vector<int> a_blk((size_t)Mg * Kg, -1), b_blk((size_t)Kg * Ng, -1), c_blk((size_t)Mg * Ng, -1);
   std::vector<int> fired((size_t)Mg * Ng, 0), queue_of((size_t)Mg * Ng, 0);
   std::vector<Block> blocks((size_t)(any_remote ? p.pool_blocks : 0));
   // FIFO: never-used blocks first, then released blocks oldest first, so a recycled block's previous users
@@ -259,7 +277,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   auto release = [&](int b, int after_cmd) {
     blocks[b].kind = -1;
     blocks[b].idx = -1;
-    blocks[b].pending.assign(1, after_cmd);
+    blocks[b].pending[0] = after_cmd;
+    blocks[b].npending = 1;
     blocks[b].last_touch = after_cmd;
     free_list.push_back(b);
   };
@@ -282,11 +301,11 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
         if (i == pin1 || i == pin2) continue;
         int next;
         if (blocks[i].kind == 0) {
-          const auto& u = a_uses[blocks[i].idx];
-          next = a_ptr[blocks[i].idx] < (int)u.size() ? u[a_ptr[blocks[i].idx]] : INT_MAX;
+          const int t = blocks[i].idx;
+          next = a_ptr[t] < a_uses.size(t) ? a_uses.at(t, a_ptr[t]) : INT_MAX;
         } else if (blocks[i].kind == 1) {
-          const auto& u = b_uses[blocks[i].idx];
-          next = b_ptr[blocks[i].idx] < (int)u.size() ? u[b_ptr[blocks[i].idx]] : INT_MAX;
+          const int t = blocks[i].idx;
+          next = b_ptr[t] < b_uses.size(t) ? b_uses.at(t, b_ptr[t]) : INT_MAX;
         } else {
           continue;  // free blocks; accumulators and source-C blocks are exclusive: never evicted
         }
@@ -310,8 +329,8 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
       else b_blk[blocks[b].idx] = -1;
       ++plan.n_evictions;
     }
-    waits.insert(waits.end(), blocks[b].pending.begin(), blocks[b].pending.end());
-    blocks[b].pending.clear();
+    waits.insert(waits.end(), blocks[b].pending, blocks[b].pending + blocks[b].npending);
+    blocks[b].npending = 0;
     blocks[b].ever_used = true;
     return b;
   };
@@ -319,13 +338,14 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   auto note_reader = [&](int b, int cmd_idx) {
     // one pending reader per stream is enough: streams run their commands in order
     blocks[b].last_touch = cmd_idx;
-    auto& pend = blocks[b].pending;
-    for (int& w : pend)
-      if (cmds[w].stream == cmds[cmd_idx].stream) {
-        w = cmd_idx;
+    Block& blk = blocks[b];
+    for (int i = 0; i < blk.npending; ++i)
+      if (cmds[blk.pending[i]].stream == cmds[cmd_idx].stream) {
+        blk.pending[i] = cmd_idx;
         return;
       }
-    pend.push_back(cmd_idx);
+    if (blk.npending >= MAX_WAITS) throw std::runtime_error("gemm plan: too many streams read one block");
+    blk.pending[blk.npending++] = cmd_idx;
   };
 
   struct OpenChain {
@@ -343,6 +363,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
     return (int)cmds.size() - 1;
   };
 
+  std::vector<int> gemm_waits, w;   // scratch, reused by every subkernel
   for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
     const int t = plan.task_order[pos];
     const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
@@ -351,11 +372,11 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
     ++a_ptr[ai];
     ++b_ptr[bi];
     int ablk = -1, bblk = -1;
-    std::vector<int> gemm_waits;
+    gemm_waits.clear();
 
     if (p.a_remote) {
       if (a_blk[ai] < 0) {
-        std::vector<int> w;
+        w.clear();
         const int b = plan.panels ? plan.a_first + mi * Kg + ki : alloc(p.b_remote ? b_blk[bi] : -1, -1, w);
         blocks[b].ever_used = true;
         Cmd c;
@@ -371,7 +392,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
     }
     if (p.b_remote) {
       if (b_blk[bi] < 0) {
-        std::vector<int> w;
+        w.clear();
         const int b = plan.panels ? plan.b_first + ni * Kg + ki : alloc(ablk, -1, w);
         blocks[b].ever_used = true;
         Cmd c;
@@ -420,12 +441,12 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
       // A tile that no later subkernel reads gives its block back at once (its readers stay pending on the block): the
       // FIFO then hands out the longest-dead block first, so the fetch that reuses it rarely waits and the copy stream
       // can run a whole k-step ahead of the subkernels even when the pool is much smaller than the operands.
-      if (ablk >= 0 && a_ptr[ai] == (int)a_uses[ai].size()) {
+      if (ablk >= 0 && a_ptr[ai] == a_uses.size(ai)) {
         blocks[ablk].kind = -1; blocks[ablk].idx = -1;
         a_blk[ai] = -1;
         free_list.push_back(ablk);
       }
-      if (bblk >= 0 && b_ptr[bi] == (int)b_uses[bi].size()) {
+      if (bblk >= 0 && b_ptr[bi] == b_uses.size(bi)) {
         blocks[bblk].kind = -1; blocks[bblk].idx = -1;
         b_blk[bi] = -1;
         free_list.push_back(bblk);
@@ -438,7 +459,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
       int last = gemm_idx;
       if (!p.beta_zero) {
         // lazy reduce: fetch the caller's tile now, out = beta * src + acc (dgemm.cpp:173-179)
-        std::vector<int> w;
+        w.clear();
         const int sb = alloc(accb, -1, w);
         Cmd f;
         f.kind = CMD_FETCH_C; f.mi = mi; f.ni = ni; f.stream = STREAM_H2D; f.block = sb;
@@ -524,7 +545,10 @@ void add_interval(Intervals& v, double a, double b) {
 
 }  // namespace
 
+std::atomic<long> plan_simulations{0};
+
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
+  ++plan_simulations;
   const GemmProblem& p = plan.p;
   const double T2 = (double)p.T * p.T;
   std::vector<double> finish(plan.cmds.size(), 0.0);
@@ -592,6 +616,105 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
   return r;
 }
 
+namespace {
+
+// Worker threads of the order search.  The candidates of one search are independent (build a plan, simulate it), so
+// they are dealt to a few threads through a shared counter and their results are gathered per candidate; which order
+// wins is then decided by one thread walking the results in candidate order, so the outcome does not depend on timing.
+// The pool lives as long as the process; PARALIA_PLAN_THREADS sets its size (1: everything on the calling thread).
+class SearchThreads {
+ public:
+  static SearchThreads& get() {
+    static SearchThreads* pool = new SearchThreads();   // never destroyed: joining at exit could wait on a thread that is gone
+    return *pool;
+  }
+  // runs fn(i) for i in [0, n), on the calling thread and the workers
+  // (small = true: the items are too cheap to be worth waking anybody)
+  void run(int n, const std::function<void(int)>& fn, bool small = false) {
+    if (n <= 0) return;
+    if (workers_.empty() || n == 1 || small) {
+      for (int i = 0; i < n; ++i) fn(i);
+      return;
+    }
+    std::lock_guard<std::mutex> one_search_at_a_time(run_mu_);
+    std::unique_lock<std::mutex> lk(mu_);
+    fn_ = &fn; n_ = n; next_ = 0; done_ = 0; ++generation_;
+    cv_.notify_all();
+    lk.unlock();
+    work();
+    lk.lock();
+    done_cv_.wait(lk, [&] { return done_ == n_ && active_ == 0; });
+    fn_ = nullptr;
+  }
+
+ private:
+  SearchThreads() {
+    // more than four gain nothing: a search has a few dozen plans of some tens of microseconds each
+    unsigned want = std::min(4u, std::max(1u, std::thread::hardware_concurrency()));
+    if (const char* env = getenv("PARALIA_PLAN_THREADS")) want = (unsigned)std::max(1, std::min(64, atoi(env)));
+    for (unsigned t = 1; t < want; ++t) workers_.emplace_back([this] { loop(); });
+    for (auto& w : workers_) w.detach();
+  }
+  void work() {
+    for (;;) {
+      int i;
+      {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (!fn_ || next_ >= n_) return;
+        i = next_++;
+      }
+      (*fn_)(i);
+      std::lock_guard<std::mutex> lk(mu_);
+      if (++done_ == n_) done_cv_.notify_all();
+    }
+  }
+  void loop() {
+    long seen = 0;
+    std::unique_lock<std::mutex> lk(mu_);
+    for (;;) {
+      cv_.wait(lk, [&] { return generation_ != seen; });
+      seen = generation_;
+      ++active_;
+      lk.unlock();
+      work();
+      lk.lock();
+      if (--active_ == 0) done_cv_.notify_all();
+    }
+  }
+  std::vector<std::thread> workers_;
+  std::mutex mu_, run_mu_;
+  std::condition_variable cv_, done_cv_;
+  const std::function<void(int)>* fn_ = nullptr;
+  int n_ = 0, next_ = 0, done_ = 0, active_ = 0;
+  long generation_ = 0;
+};
+
+struct Evaluated {
+  bool ok = false;
+  PipelineResult r;
+  long evictions = 0;
+  std::string err;
+};
+
+// build + simulate every id of the list, in parallel
+std::vector<Evaluated> evaluate_orders(const GemmProblem& p, const StageTimes& st, const std::vector<int>& ids) {
+  std::vector<Evaluated> out(ids.size());
+  const std::function<void(int)> one = [&](int i) {
+    try {
+      GemmPlan plan = build_gemm_plan(p, ids[i]);
+      out[i].r = simulate_plan(plan, st);
+      out[i].evictions = plan.n_evictions;
+      out[i].ok = true;
+    } catch (const std::runtime_error& e) {
+      out[i].err = e.what();  // this order does not fit the pool; others may
+    }
+  };
+  SearchThreads::get().run((int)ids.size(), one, /*small=*/p.subkernels() * (long)ids.size() < 6000);
+  return out;
+}
+
+}  // namespace
+
 int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best_out, bool probe) {
   // Two groups of orders, each with its own best: the panel orders, and the block orders (w >= ORDER_BLOCK_ROWS), which
   // end in two tile-by-tile phases and are taken only when they win by more than a percent (12288^3: simulated 0.6 %
@@ -603,20 +726,41 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   } grp[2];
   auto is_block = [](int id) { return id % 10000 >= ORDER_BLOCK_ROWS; };
   std::string last_err;
-  for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0)) {
-    if (is_block(id) && !st.block_orders) continue;
-    try {
-      GemmPlan plan = build_gemm_plan(p, id);
-      PipelineResult r = simulate_plan(plan, st);
+  // The variants with merged K chains come second: merging takes at most (launches saved) x (saving per launch) off an
+  // order's makespan -- it removes that much compute and otherwise only delays launches -- so a merged variant is built
+  // only where its plain order, less that bound, gets under the best plain order.
+  std::vector<int> ids, merged_ids;
+  for (int id : gemm_candidate_orders(p, probe, st.merge_saving > 0))
+    if (!is_block(id) || st.block_orders) (id % ORDER_K_SPLIT >= ORDER_MERGE_CHAINS ? merged_ids : ids).push_back(id);
+  auto gather = [&](const std::vector<int>& list, const std::vector<Evaluated>& evals) {
+    for (size_t i = 0; i < list.size(); ++i) {
+      const int id = list[i];
+      if (!evals[i].ok) { last_err = evals[i].err; continue; }
+      const PipelineResult& r = evals[i].r;
       Group& g = grp[is_block(id) ? 1 : 0];
       g.ranked.emplace_back(r.t_total, id);
       if (g.id < 0 || r.t_total < g.r.t_total * (1.0 - 1e-9)) {
         g.r = r;
         g.id = id;
       }
-    } catch (const std::runtime_error& e) {
-      last_err = e.what();  // this order does not fit the pool; others may
     }
+  };
+  const std::vector<Evaluated> evals = evaluate_orders(p, st, ids);
+  gather(ids, evals);
+  if (!merged_ids.empty()) {
+    double best_plain = DBL_MAX;
+    for (const Evaluated& e : evals)
+      if (e.ok) best_plain = std::min(best_plain, e.r.t_total);
+    const double most_saved = (double)(p.subkernels() - (long)p.Mg() * p.Ng()) * st.merge_saving;
+    std::vector<int> worth;
+    for (int id : merged_ids) {
+      const auto plain = std::find(ids.begin(), ids.end(), id - ORDER_MERGE_CHAINS);
+      if (plain == ids.end()) { worth.push_back(id); continue; }
+      const Evaluated& e = evals[plain - ids.begin()];
+      if (st.exhaustive || (e.ok && e.r.t_total - most_saved <= best_plain)) worth.push_back(id);
+    }
+    // the ranking keeps candidate order: merged variants behind the plain ones, as the candidate list has them
+    gather(worth, evaluate_orders(p, st, worth));
   }
   if (grp[0].id < 0 && grp[1].id < 0) throw std::runtime_error(last_err.empty() ? "gemm plan: no feasible order" : last_err);
   // the best orders also with a thin start (first k tile in 2 or 4 slabs), where the operands cross the link; the
@@ -627,22 +771,24 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit))
     for (Group& g : grp) {
       if (g.id < 0) continue;
+      // a thin start takes at most three quarters of the first A and B tiles' fetch off a call: a group that would
+      // still trail the other group's plain best by more than that is not worth the six plans
+      const Group& other = grp[&g == &grp[0] ? 1 : 0];
+      const double thin_gain = ((p.a_remote ? 1 : 0) + (p.b_remote ? 1 : 0)) * 0.75 * st.h2d_tb * (double)p.T * std::min(p.T, p.K) * p.elem;
+      if (!st.exhaustive && other.id >= 0 && g.r.t_total - thin_gain > other.r.t_total) continue;
       // makespans that differ only in the last bits are ties (compared in single precision), and ties keep the
       // candidate order, as the choice above does
       std::stable_sort(g.ranked.begin(), g.ranked.end(),
                        [](const std::pair<double, int>& a, const std::pair<double, int>& b) { return (float)a.first < (float)b.first; });
       const double unsplit_best = g.r.t_total;
+      std::vector<int> thin_ids;
       for (size_t b = 0; b < std::min<size_t>(3, g.ranked.size()); ++b)
-        for (int s = 1; s <= 2; ++s) {
-          try {
-            GemmPlan plan = build_gemm_plan(p, g.ranked[b].second + s * ORDER_K_SPLIT);
-            PipelineResult r = simulate_plan(plan, st);
-            if (plan.n_evictions == 0 && r.t_total < unsplit_best * (1.0 - 1e-3) && r.t_total < g.r.t_total) {
-              g.r = r;
-              g.id = g.ranked[b].second + s * ORDER_K_SPLIT;
-            }
-          } catch (const std::runtime_error&) {
-          }
+        for (int s = 1; s <= 2; ++s) thin_ids.push_back(g.ranked[b].second + s * ORDER_K_SPLIT);
+      const std::vector<Evaluated> thin = evaluate_orders(p, st, thin_ids);
+      for (size_t i = 0; i < thin_ids.size(); ++i)
+        if (thin[i].ok && thin[i].evictions == 0 && thin[i].r.t_total < unsplit_best * (1.0 - 1e-3) && thin[i].r.t_total < g.r.t_total) {
+          g.r = thin[i].r;
+          g.id = thin_ids[i];
         }
     }
   const Group& pick = (grp[0].id < 0 || (grp[1].id >= 0 && grp[1].r.t_total < 0.99 * grp[0].r.t_total)) ? grp[1] : grp[0];

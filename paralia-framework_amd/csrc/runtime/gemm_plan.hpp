@@ -12,6 +12,7 @@
 #ifndef PARALIA_GEMM_PLAN_HPP
 #define PARALIA_GEMM_PLAN_HPP
 
+#include <atomic>
 #include <utility>
 #include <vector>
 
@@ -140,6 +141,9 @@ struct StageTimes {
   double tr_amp = 0, tr_idle = 6e-3, tr_recover = 8e-3;
   double tr_gap0 = 1e-3;             // idle time assumed in front of the call (calls made back to back)
   bool block_orders = true;          // offer the block orders (w >= ORDER_BLOCK_ROWS) to the order search
+  // simulate every candidate, also those a bound shows cannot win (merged variants, thin starts of a trailing group):
+  // the slow search the pruned one is tested against
+  bool exhaustive = false;
   // a slab of the thin start: the full tile's time in proportion to its k, plus this much per launch for slabs 1024 deep
   // or deeper, in inverse proportion to the depth below that (measured inside streamed calls, two launches sharing the
   // device: 2048 x 2048 x 1024 slabs +2 us, x 512 slabs +4.5 us against a quarter of the whole tile's 231.5 us)
@@ -149,6 +153,7 @@ struct PipelineResult {
   double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource
 };
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st);
+extern std::atomic<long> plan_simulations;   // plans simulated by this process so far (the order search's unit of work)
 // Builds every candidate order, simulates it, returns the id with the smallest makespan.
 int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best, bool probe = false);
 

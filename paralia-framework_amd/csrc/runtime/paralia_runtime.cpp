@@ -258,6 +258,10 @@ struct Runtime {
   Resources res;
   std::vector<std::unique_ptr<PMDEntry>> pmd;  // at most PROBLEM_MD_CACHE entries, oldest dropped first
   long pmd_hits = 0, pmd_misses = 0;
+  // Host-side phases of the most recent GEMM call, in seconds (the reference's TEST build prints the same split:
+  // dgemm.cpp:330-333 autotune, :430-445 decomposition and tile maps, :497-511 cache allocation and queues, :598-604
+  // execution).  autotune and plan are 0 on a call served from the metadata cache.
+  struct Phases { double autotune = 0, plan = 0, pool = 0, streams = 0, execute = 0, total = 0; } phases;
 };
 static Runtime& rt() {
   // never destroyed: at process exit the HIP runtime may already be gone, and freeing pinned buffers, events or
@@ -505,6 +509,8 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   key.predef_T = predef ? predef->T : -1;
   key.cache_limit = predef ? predef->cache_limit : 0;
 
+  const double t_call = csecond();
+  R.phases = Runtime::Phases();
   PMDEntry* entry = nullptr;
   for (auto& e : R.pmd)
     if (e->key == key) { entry = e.get(); break; }
@@ -537,7 +543,10 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     // alpha == 0 or K == 0: C <- beta*C only, one "subkernel" per C tile with an empty K; K must not
     // constrain the tile choice then
     if (d.D3 == 0) d.D3 = std::min(M, N);
+    double t_phase = csecond();
     atc->autotune_problem(GemmFns<T>::name, d);
+    R.phases.autotune = csecond() - t_phase;
+    t_phase = csecond();
     if (any_remote) {
       GemmProblem gp;
       gp.M = M; gp.N = N; gp.K = no_ab ? 0 : K; gp.T = atc->T;
@@ -556,6 +565,7 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
       atc->update_sk_num(ne->plan.p.subkernels());  // the plan's own problem: a thin start adds k tiles
       atc->distribute_subkernels(ne->plan.p.Mg(), ne->plan.p.Ng(), ne->plan.p.Kg());
     }
+    R.phases.plan = csecond() - t_phase;
     if ((int)R.pmd.size() >= PROBLEM_MD_CACHE) R.pmd.erase(R.pmd.begin());
     R.pmd.push_back(std::move(ne));
     entry = R.pmd.back().get();
@@ -572,11 +582,18 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;
+    double t_phase = csecond();
     R.pool.ensure(plan.blocks_used, (long long)plan.p.T * plan.p.T * (long long)sizeof(T), atc->cache_limit);
+    R.phases.pool = csecond() - t_phase;
+    t_phase = csecond();
     R.res.ensure_streams(std::max(1, std::min(plan.p.exec_queues, MAX_EXEC_QUEUES)));
+    R.phases.streams = csecond() - t_phase;
+    t_phase = csecond();
     const bool pageable[3] = {locA == -2, locB == -2, locC == -2};
     execute_gemm_plan<T>(R, plan, ta, tb, alpha, A, ldA, B, ldB, beta, C, ldC, pageable);
+    R.phases.execute = csecond() - t_phase;
   }
+  R.phases.total = csecond() - t_call;
   ++entry->calls;
   return atc_copy(atc);
 }
@@ -932,6 +949,13 @@ void runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long
   if (pmd_misses) *pmd_misses = R.pmd_misses;
   if (pool_bytes) *pool_bytes = R.pool.bytes();
   if (pmd_entries) *pmd_entries = (long)R.pmd.size();
+}
+
+void last_call_phases(double seconds[6]) {
+  Runtime& R = rt();
+  std::lock_guard<std::mutex> lk(R.mu);
+  const Runtime::Phases& ph = R.phases;
+  seconds[0] = ph.autotune; seconds[1] = ph.plan; seconds[2] = ph.pool; seconds[3] = ph.streams; seconds[4] = ph.execute; seconds[5] = ph.total;
 }
 
 void stream_queues(int* independent, int* created) {

@@ -15,6 +15,8 @@ extern "C" {
 const char* pl_last_error(void) { return ""; }
 int pl_malloc_pinned(void** p, long long b) { *p = malloc(b); return 0; }
 int pl_free_pinned(void* p) { free(p); return 0; }
+int pl_get_device(int* d) { *d = 0; return 0; }
+int pl_set_device(int) { return 0; }
 int pl_event_create(void** e, int) { *e = malloc(1); return 0; }
 int pl_event_destroy(void* e) { free(e); return 0; }
 int pl_event_record(void*, void*) { return 0; }

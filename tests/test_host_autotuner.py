@@ -359,3 +359,54 @@ def test_power_transient_file_is_optional_and_prices_sparse_starts(L, pkg, tmp_p
     rise = res[("with", 16384)][1] - res[("bare", 16384)][1]
     assert 0 < rise < 0.25 * vals["Amplitude"] * vals["Recovery"]
     assert res[("with", 6144)][0] != res[("bare", 6144)][0] and res[("with", 6144)][1] > res[("bare", 6144)][1]
+
+
+SEARCH_SHAPES = [  # (routine, M, N, K, transposes, locations, beta == 0, pool budget in bytes)
+    (b"Dgemm", 16384, 16384, 16384, b"NN", (-1, -1, -1), 1, 0), (b"Dgemm", 8192, 8192, 8192, b"NN", (-1, -1, -1), 1, 0),
+    (b"Dgemm", 4096, 4096, 4096, b"NN", (-1, -1, -1), 0, 0), (b"Dgemm", 12288, 6144, 6144, b"NN", (-1, -1, -1), 1, 0),
+    (b"Dgemm", 16384, 4096, 8192, b"NN", (-1, -1, -1), 1, 0), (b"Dgemm", 6000, 7000, 5000, b"NN", (-1, -1, -1), 1, 0),
+    (b"Dgemm", 20000, 20000, 4096, b"NN", (-1, -1, -1), 1, 0), (b"Dgemm", 40000, 40000, 2048, b"NN", (-1, -1, -1), 0, 0),
+    (b"Dgemm", 16384, 16384, 16384, b"TN", (-1, -1, -1), 1, 0), (b"Dgemm", 16384, 16384, 16384, b"NN", (-1, -1, -1), 1, 2 * 10 ** 9),
+    (b"Sgemm", 32768, 32768, 32768, b"NT", (-1, -1, 0), 0, 0), (b"Sgemm", 12288, 12288, 12288, b"NN", (-1, -1, -1), 1, 0),
+    (b"Sgemm", 16384, 8192, 8192, b"NN", (-1, -1, -1), 1, 0), (b"Dgemm", 32768, 32768, 32768, b"NN", (-1, -1, -1), 1, 0),
+]
+
+
+def test_pruned_search_picks_what_the_exhaustive_search_picks(L, pkg, monkeypatch):
+    """The tile and order search dismisses candidates by bounds (a tile size whose kernels alone, plus the first fetch
+    and the last write-back, take longer than a makespan already found; a merged-chain variant that cannot make up its
+    plain order's distance; the thin start of a trailing group).  PARALIA_PLAN_SEARCH=exhaustive switches every bound
+    off: on the shipped database both searches must agree on tile, order and predicted time, for compute-bound,
+    link-bound, ragged, limited-pool, transposed and fp32 problems."""
+    db = _shipped_db(pkg).encode()
+    info = pkg.atc_info()
+    for func, M, N, K, tr, locs, bz, budget in SEARCH_SHAPES:
+        picks = []
+        for mode in (None, "exhaustive"):
+            if mode:
+                monkeypatch.setenv("PARALIA_PLAN_SEARCH", mode)
+            else:
+                monkeypatch.delenv("PARALIA_PLAN_SEARCH", raising=False)
+            assert L.PARALiA_autotune(db, func, M, N, K, tr[0:1], tr[1:2], loc3(*locs), bz, -1, budget, C.byref(info)) == 0
+            picks.append((info.T, info.order_id, info.pred_t))
+        assert picks[0][:2] == picks[1][:2] and abs(picks[0][2] - picks[1][2]) <= 1e-12 * picks[1][2], (func, M, N, K, picks)
+    monkeypatch.delenv("PARALIA_PLAN_SEARCH", raising=False)
+
+
+def test_planner_time_of_a_first_call(L, pkg, monkeypatch):
+    """What a new problem's first call spends in the planner (best of five, database already read): the headline shape
+    within 5 ms, the largest benchmark shapes (32768^3, fp64 and fp32) within 20 ms."""
+    import time
+    monkeypatch.delenv("PARALIA_PLAN_SEARCH", raising=False)
+    db = _shipped_db(pkg).encode()
+    info = pkg.atc_info()
+    for func, M, N, K, tr, locs, bz, bound_ms in ((b"Dgemm", 16384, 16384, 16384, b"NN", (-1, -1, -1), 1, 5.0),
+                                                 (b"Dgemm", 32768, 32768, 32768, b"NN", (-1, -1, -1), 1, 20.0),
+                                                 (b"Sgemm", 32768, 32768, 32768, b"NT", (-1, -1, 0), 0, 20.0)):
+        best = 1e9
+        for _ in range(6):
+            t0 = time.perf_counter()
+            assert L.PARALiA_autotune(db, func, M, N, K, tr[0:1], tr[1:2], loc3(*locs), bz, -1, 0, C.byref(info)) == 0
+            best = min(best, (time.perf_counter() - t0) * 1e3)
+        print("  planner %s %d x %d x %d: %.2f ms (T = %d, order %d)" % (func.decode(), M, N, K, best, info.T, info.order_id), flush=True)
+        assert best <= bound_ms, (func, M, N, K, best)

@@ -34,6 +34,18 @@ def test_planner_under_address_and_undefined_behaviour_sanitizers(tmp_path):
     assert "built" in run.stdout and "runtime error" not in run.stderr and "AddressSanitizer" not in run.stderr
 
 
+def test_order_search_threads_under_thread_sanitizer(tmp_path):
+    """The order search deals its candidate plans to a few worker threads; the same fuzzer under TSan, with the pool
+    forced to four threads whatever the machine has, and the small-work shortcut left to chance by the problem sizes."""
+    exe = _build(tmp_path, "plan_fuzz_tsan", [os.path.join(ROOT, "tests", "sanitize", "plan_fuzz.cpp"), os.path.join(CSRC, "runtime", "gemm_plan.cpp")],
+                 ["-fsanitize=thread"])
+    run = subprocess.run([exe, "400"], capture_output=True, text=True, timeout=900, env=dict(os.environ, PARALIA_PLAN_THREADS="4"))
+    if "FATAL: ThreadSanitizer: unexpected memory mapping" in run.stderr:
+        pytest.skip("ThreadSanitizer cannot map its shadow memory in this container")
+    assert run.returncode == 0, (run.stdout[-500:], run.stderr[-3000:])
+    assert "built" in run.stdout and "ThreadSanitizer" not in run.stderr
+
+
 def test_copy_thread_pool_under_thread_sanitizer(tmp_path):
     exe = _build(tmp_path, "copy_threads", [os.path.join(ROOT, "tests", "sanitize", "copy_threads.cpp"), os.path.join(CSRC, "runtime", "host_staging.cpp")],
                  ["-fsanitize=thread"])
