@@ -12,6 +12,8 @@
 #include <string>
 #include <vector>
 
+#include "paralia_hip.h"
+
 #ifndef LOC_NUM
 #define LOC_NUM 2  // one GPU (index 0) + host (last index), as in the reference's idxize(-1) = LOC_NUM - 1
 #endif
@@ -81,6 +83,25 @@ struct GPUexecModel {
 };
 GPUexecModel* GPUexecModel_init(const std::string& db_dir, int dev_id, const char* func);
 
+/// Fitted constants of this device's kernels that are not table rows: the tile-GEMM launcher's cost model (handed to
+/// the launcher with pl_gemm_set_fit when a Modeler is built) and the terms the plan simulator adds to the table times.
+/// Read from Processed/Kernel-fit_dev-<id>.log ("name: value" lines, written by the deploy tool; not a file of the
+/// reference, whose kernels are cuBLAS's); a missing file or a missing line leaves the built-in value (measured on an
+/// MI355X).
+struct KernelFit {
+  pl_gemm_fit launcher;
+  double merge_saving_us_f64 = 4.0;    // a launch saved by merging K chains, fp64: the gap between two launches of a stream
+  // fp32, per round of 256 large tiles and per transpose (NN, NT, TN, TT): the fixed cost of a launch that accumulates,
+  // less the launch gap
+  double merge_saving_us_f32[4] = {40.0, 40.0, 40.0, 40.0};
+  double lone_share = 0.07;            // share of a streamed call's launches that run without a partner on the device
+  double geadd_bytes_per_s = 3e12;     // rate of the lazy-reduce kernel over its 3 T^2 elements
+  double slab_fixed_us = 2.0;          // extra time of a thin-start slab launch 1024 deep (deeper: the same, shallower: in inverse proportion)
+  bool from_file = false;
+  KernelFit() { pl_gemm_fit_defaults(&launcher); }
+};
+KernelFit KernelFit_load(const std::string& db_dir, int dev_id);
+
 /// What the models need to know about one call (the reference's Vdata + Modeler fields, Autotuner.hpp:22-36,70-84).
 struct ProblemDesc {
   const char* func = "Dgemm";
@@ -107,6 +128,7 @@ typedef class Modeler {
   // after its compute units sat idle a tile kernel takes up to (1 + amplitude) times its steady time; the deficit grows
   // with time constant idle_s while nothing runs and decays with recover_s while kernels do.  amplitude 0: not measured.
   double transient_amplitude = 0, transient_idle_s = 0, transient_recover_s = 0;
+  KernelFit fit;                // Processed/Kernel-fit_dev-<id>.log, optional
   Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc);
   ~Modeler();
   long getMinT() const;

@@ -104,6 +104,33 @@ int pl_sgemm_tile_ws(char transA, char transB, long M, long N, long K, float alp
                      const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
                      void* stream);
 
+/* Fitted constants of the tile-GEMM launcher's cost model: how it chooses between its macro tiles (fp32: 128 x 128,
+ * 256 x 128 "wide", 256 x 256 "large") and how many ways it splits K for products with few tiles.  They describe one
+ * device and one build of the kernels; the deploy tool measures them and writes Processed/Kernel-fit_dev-<id>.log, the
+ * autotuner's database loader hands them over with pl_gemm_set_fit (the role of the reference's deploy-time kernel
+ * tables, Deploy.in:14-18, Database_builder/CuCuBLAS/src/dgemm_microbench.cu:125-160, for a library that owns its
+ * kernels).  Without a call the built-in values (measured on an MI355X) apply.  Times in microseconds.
+ * Transpose index: 0 NN, 1 NT, 2 TN, 3 TT. */
+typedef struct pl_gemm_fit {
+  double lone_us_per_k[2];          /* [0] fp64, [1] fp32: one 128 x 128 workgroup per compute unit, per unit of k */
+  double lone_fixed_k;              /* its prologue and epilogue, in units of k */
+  double splitk_launch_us;          /* the second launch of a split product */
+  double pass_bytes_per_us;         /* rate of the pass that adds the split-K slices */
+  double f32_small_us_per_k;        /* a round of 512 small fp32 tiles (two per compute unit), per unit of k */
+  double f32_small_fixed_us;        /* ... and its fixed part */
+  double f32_wide_gain;             /* wide tile: 2 * f32_small_us_per_k * K / gain per round of 512 */
+  double f32_wide_fixed_us[2];      /* beta == 0, beta != 0 */
+  double f32_large_gain[4];         /* large tile: 2 * f32_small_us_per_k * K / (1 + gain) per round of 256, per transpose */
+  double f32_large_fixed_us[4][2];  /* per transpose; beta == 0, beta != 0 */
+} pl_gemm_fit;
+void pl_gemm_fit_defaults(pl_gemm_fit* fit);
+int pl_gemm_set_fit(const pl_gemm_fit* fit);   /* null: back to the built-in values */
+int pl_gemm_get_fit(pl_gemm_fit* fit);
+/* What the launcher would do for a product (no GPU call): macro tile rows and columns, and the split count it would use
+ * given a workspace of workspace_bytes (0: none).  elem_size 8 or 4. */
+int pl_gemm_tile_choice(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero, long workspace_bytes,
+                        int* tile_m, int* tile_n, int* splits);
+
 /* out <- beta*src + acc on an M x N tile (out may alias acc): the ALGO_WR_LAZY reduce of a finished C tile
  * with the caller's original C (dgemm.cpp:173-179; CMakeLists.txt:78-88). */
 int pl_dgeadd_tile(long M, long N, double beta, const double* src, long ld_src, const double* acc, long ld_acc,

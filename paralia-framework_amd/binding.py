@@ -20,6 +20,14 @@ class atc_info(C.Structure):
                 ("pipe_h2d", C.c_double), ("pipe_exec", C.c_double), ("pipe_d2h", C.c_double)]
 
 
+class gemm_fit(C.Structure):
+    """pl_gemm_fit of include/paralia_hip.h."""
+    _fields_ = [("lone_us_per_k", C.c_double * 2), ("lone_fixed_k", C.c_double), ("splitk_launch_us", C.c_double),
+                ("pass_bytes_per_us", C.c_double), ("f32_small_us_per_k", C.c_double), ("f32_small_fixed_us", C.c_double),
+                ("f32_wide_gain", C.c_double), ("f32_wide_fixed_us", C.c_double * 2), ("f32_large_gain", C.c_double * 4),
+                ("f32_large_fixed_us", (C.c_double * 2) * 4)]
+
+
 def build_library(jobs=8):
     """Compile every HIP and C++ source for gfx950 (hipcc cross-compiles without a GPU)."""
     subprocess.run(["make", "-C", PKG_DIR, "-j%d" % jobs], check=True)
@@ -63,6 +71,10 @@ _SIGS = {
     "pl_dgemm_tile": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp]),
     "pl_sgemm_tile": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp]),
     "pl_gemm_tile_workspace_bytes": (_l, [_l, _l, _l, _i]),
+    "pl_gemm_fit_defaults": (None, [C.POINTER(gemm_fit)]),
+    "pl_gemm_set_fit": (_i, [C.POINTER(gemm_fit)]),
+    "pl_gemm_get_fit": (_i, [C.POINTER(gemm_fit)]),
+    "pl_gemm_tile_choice": (_i, [_i, _c, _c, _l, _l, _l, _i, _l, _pi, _pi, _pi]),
     "pl_dgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _vp]),
     "pl_sgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _vp]),
     "pl_dgeadd_tile": (_i, [_l, _l, _d, _vp, _l, _vp, _l, _vp, _l, _vp]),

@@ -262,16 +262,19 @@ paralia::StageTimes nominal_stage_times(const ProblemDesc& d, long T) {
 // per launch.  The fp64 kernel runs two workgroups per compute unit that cover each other's ends; there a launch saved
 // is worth the gap between two launches of a stream: dgemm 16384^3 at T = 2048 with 128 launches fewer (448 instead of
 // 576) took 0.55 ms less (123.3 / 123.7 against 123.9 / 124.2 ms), 4 us each.
-static double paralia_merge_saving(const ProblemDesc& d, long T) {
+// Both figures are KernelFit's (merge_saving_us_f64 / _f32): the deploy tool derives them from the launch gap and the
+// large tile's fixed cost it measures.
+static double paralia_merge_saving(const ProblemDesc& d, long T, const KernelFit& fit) {
   const char* env = getenv("PARALIA_MERGE_CHAINS");  // "0": never merge
   if (env && *env && atoi(env) == 0) return 0.0;
   // measured for tiles that fill the device by themselves; smaller ones run split-K kernels whose time a joined k range
   // changes in ways this term does not describe
-  if (d.dtype_sz != 4) return T >= 1792 ? 4e-6 : 0.0;
+  if (d.dtype_sz != 4) return T >= 1792 ? fit.merge_saving_us_f64 * 1e-6 : 0.0;
   // a launch with fewer workgroups than compute units wastes that much less of the device: scale by the rounds of 256
   // workgroups it amounts to, as a fraction
   const double rounds = (double)((T + 255) / 256) * (double)((T + 255) / 256) / 256.0;
-  return 40e-6 * rounds;
+  const int tr = d.TransA == 'N' ? (d.TransB == 'N' ? 0 : 1) : (d.TransB == 'N' ? 2 : 3);
+  return fit.merge_saving_us_f32[tr] * 1e-6 * rounds;
 }
 
 paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
@@ -289,7 +292,7 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   // takes its lone time, which for tiles whose workgroups do not fill whole rounds of the device is a third longer.
   // Measured streamed calls behave as if that were the case for about 7 % of a launch (12288^3: T = 3072 predicted
   // 0.3 % faster than T = 2048 without this term, measured 2.3 % slower; 14336^3 and 20000 x 20000 x 4096 alike).
-  const double lone_share = 0.07;
+  const double lone_share = m->fit.lone_share;
   st.t_exec *= 1 + lone_share * (m->exec->lone_ratio(T, d.TransA, d.TransB) - 1);
   for (auto& e : st.exec_table) e.second *= 1 + lone_share * (m->exec->lone_ratio(e.first, d.TransA, d.TransB) - 1);
   const comm_data* h2d = m->link[idxize(-1)];
@@ -297,8 +300,9 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.h2d_ti = h2d->ti; st.h2d_tb = h2d->tb;
   st.d2h_ti = d2h->ti; st.d2h_tb = d2h->tb;
   st.h2d_sl = std::max(1.0, h2d->sl); st.d2h_sl = std::max(1.0, d2h->sl);
-  st.t_reduce = 3.0 * T * T * d.dtype_sz / 3e12;
-  st.merge_saving = paralia_merge_saving(d, T);
+  st.t_reduce = 3.0 * T * T * d.dtype_sz / m->fit.geadd_bytes_per_s;
+  st.merge_saving = paralia_merge_saving(d, T, m->fit);
+  st.slab_fixed = m->fit.slab_fixed_us * 1e-6;
   const char* thin = getenv("PARALIA_THIN_START");  // "0": never cut the first k tile into slabs
   st.thin_start = !(thin && *thin && atoi(thin) == 0);
   if (d.problem == BLAS3 && m->transient_amplitude > 0) {

@@ -10,6 +10,53 @@
 #include "Autotuner.hpp"
 #include "backend_wrappers.hpp"
 
+// "name: value" lines; names this build does not know are ignored, so are values that do not parse.
+KernelFit KernelFit_load(const std::string& db_dir, int dev_id) {
+  KernelFit k;
+  char filename[1024];
+  snprintf(filename, sizeof filename, "%s/Processed/Kernel-fit_dev-%d.log", db_dir.c_str(), dev_id);
+  FILE* fp = fopen(filename, "r");
+  if (!fp) return k;
+  k.from_file = true;
+  static const char* const trans[4] = {"NN", "NT", "TN", "TT"};
+  char line[512];
+  while (fgets(line, sizeof line, fp)) {
+    char name[128];
+    double v = 0;
+    if (line[0] == '#' || sscanf(line, " %127[^:]: %lf", name, &v) != 2) continue;
+    const std::string n(name);
+    pl_gemm_fit& f = k.launcher;
+    if (n == "lone_us_per_k_f64") f.lone_us_per_k[0] = v;
+    else if (n == "lone_us_per_k_f32") f.lone_us_per_k[1] = v;
+    else if (n == "lone_fixed_k") f.lone_fixed_k = v;
+    else if (n == "splitk_launch_us") f.splitk_launch_us = v;
+    else if (n == "pass_bytes_per_us") f.pass_bytes_per_us = v;
+    else if (n == "f32_small_us_per_k") f.f32_small_us_per_k = v;
+    else if (n == "f32_small_fixed_us") f.f32_small_fixed_us = v;
+    else if (n == "f32_wide_gain") f.f32_wide_gain = v;
+    else if (n == "f32_wide_fixed_us_beta0") f.f32_wide_fixed_us[0] = v;
+    else if (n == "f32_wide_fixed_us_beta1") f.f32_wide_fixed_us[1] = v;
+    else if (n == "merge_saving_us_f64") k.merge_saving_us_f64 = v;
+    else if (n == "merge_saving_us_f32") { for (double& x : k.merge_saving_us_f32) x = v; }
+    else if (n == "lone_share") k.lone_share = v;
+    else if (n == "geadd_bytes_per_s") k.geadd_bytes_per_s = v;
+    else if (n == "slab_fixed_us") k.slab_fixed_us = v;
+    else
+      for (int t = 0; t < 4; ++t) {
+        if (n == std::string("f32_large_gain_") + trans[t]) f.f32_large_gain[t] = v;
+        else if (n == std::string("f32_large_fixed_us_beta0_") + trans[t]) f.f32_large_fixed_us[t][0] = v;
+        else if (n == std::string("f32_large_fixed_us_beta1_") + trans[t]) f.f32_large_fixed_us[t][1] = v;
+        else if (n == std::string("merge_saving_us_f32_") + trans[t]) k.merge_saving_us_f32[t] = v;
+      }
+  }
+  fclose(fp);
+  bool merge_ok = k.merge_saving_us_f64 >= 0;
+  for (double x : k.merge_saving_us_f32) merge_ok = merge_ok && x >= 0;
+  if (!(merge_ok && k.lone_share >= 0 && k.lone_share <= 1 && k.geadd_bytes_per_s > 0 && k.slab_fixed_us >= 0))
+    error("KernelFit_load: %s holds a value out of range\n", filename);
+  return k;
+}
+
 Modeler::Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc) : P(desc), unit_id(dev_id) {
   for (int idx = 0; idx < LOC_NUM; ++idx) {
     const int other = deidxize(idx);
@@ -21,6 +68,9 @@ Modeler::Modeler(const std::string& db_dir, int dev_id, const ProblemDesc& desc)
     }
   }
   exec = GPUexecModel_init(db_dir, dev_id, desc.func);
+  // the launcher prices its macro tiles and split counts with the constants of the database in use
+  fit = KernelFit_load(db_dir, dev_id);
+  if (pl_gemm_set_fit(&fit.launcher) != 0) error("Modeler: Processed/Kernel-fit_dev-%d.log of %s holds a launcher constant out of range\n", dev_id, db_dir.c_str());
   char filename[1024];
   snprintf(filename, sizeof filename, "%s/Processed/Power-transient_dev-%d.log", db_dir.c_str(), dev_id);
   if (FILE* fp = fopen(filename, "r")) {

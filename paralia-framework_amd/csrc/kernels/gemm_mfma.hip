@@ -25,6 +25,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include "paralia_hip.h"
+
 // Build-time switches (timing experiments; the defaults are what ships).
 #ifndef PLK_F64_BK
 #define PLK_F64_BK 16
@@ -699,6 +701,25 @@ __global__ void splitk_reduce_kernel(int M, int N, int splits, T alpha, const T*
 // How many ways to split K so that a product with few C tiles still fills the 256 compute units.
 // The estimate counts rounds of 256 workgroups, each costing its k extent plus a fixed prologue / epilogue share, and
 // the pass that adds the slices (workspace written once and read once).  1 = do not split.
+// The launcher's fitted constants (pl_gemm_fit in the public header): built-in values measured on an MI355X, replaced
+// by what the deploy database holds once the autotuner has loaded it.
+inline void fit_defaults(pl_gemm_fit* f) {
+  f->lone_us_per_k[0] = 0.117; f->lone_us_per_k[1] = 0.0585;
+  f->lone_fixed_k = 48.0;
+  f->splitk_launch_us = 4.0;
+  f->pass_bytes_per_us = 4.0e6;
+  f->f32_small_us_per_k = 0.1207;
+  f->f32_small_fixed_us = 6.0;
+  f->f32_wide_gain = 1.042;
+  f->f32_wide_fixed_us[0] = 5.0; f->f32_wide_fixed_us[1] = 10.6;
+  const double g[4] = {0.072, 0.088, 0.073, 0.076}, f0[4] = {10.0, 10.0, 9.0, 10.0}, f1[4] = {46.0, 44.0, 52.0, 55.0};
+  for (int t = 0; t < 4; ++t) { f->f32_large_gain[t] = g[t]; f->f32_large_fixed_us[t][0] = f0[t]; f->f32_large_fixed_us[t][1] = f1[t]; }
+}
+inline pl_gemm_fit& fit_in_use() {
+  static pl_gemm_fit f = [] { pl_gemm_fit d; fit_defaults(&d); return d; }();
+  return f;
+}
+
 template <typename T>
 int pick_splits(long M, long N, long K, int* kchunk_out) {
   constexpr int BM = 128, BN = 128;
@@ -707,8 +728,9 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
   // with more than about half the compute units covered, a second product running on another stream (the way the
   // scheduler issues subkernels) fills the rest better than a split would
   if (tiles > 160 || K < 256) return 1;
-  const double us_per_k = sizeof(T) == 8 ? 0.117 : 0.0585;  // one workgroup, one unit of k, at the measured tile rate
-  auto main_us = [&](long blocks, long kc) { return (double)((blocks + 255) / 256) * (double)(kc + 48) * us_per_k; };
+  const pl_gemm_fit& fit = fit_in_use();
+  const double us_per_k = fit.lone_us_per_k[sizeof(T) == 8 ? 0 : 1];  // one workgroup, one unit of k, at the measured tile rate
+  auto main_us = [&](long blocks, long kc) { return (double)((blocks + 255) / 256) * ((double)kc + fit.lone_fixed_k) * us_per_k; };
   double best = main_us(tiles, K);
   int best_s = 1;
   const long max_ws = 256L << 20;  // workspace bound: the slices of very long, very thin products stay small anyway
@@ -718,7 +740,7 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
     const long se = (K + kc - 1) / kc;
     if (se < 2) continue;
     if (se * M * N * (long)sizeof(T) > max_ws) break;
-    const double t = main_us(tiles * se, kc) + 4.0 + (double)(2 * se + 1) * (double)M * (double)N * sizeof(T) / 4.0e6;
+    const double t = main_us(tiles * se, kc) + fit.splitk_launch_us + (double)(2 * se + 1) * (double)M * (double)N * sizeof(T) / fit.pass_bytes_per_us;
     if (t < best * 0.95) {
       best = t;
       best_s = (int)se;
@@ -726,6 +748,50 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
     }
   }
   return best_s;
+}
+
+// Macro tile and split count of one product.
+struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; };
+template <typename T>
+TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes) {
+  TileChoice c;
+  c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
+  if (c.splits > 1 && (long)c.splits * M * N * (long)sizeof(T) > workspace_bytes) c.splits = 1, c.kchunk = 0;
+  // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
+  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 7 - 9 % faster per k (all panels global -> LDS
+  //    directly, a 16-byte operand read per block and four k-steps), but a CU holds one such workgroup at a time, so
+  //    nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * c * K / (1 + g), c the
+  //    per-k time of a round of 512 small tiles, with g and f (beta == 0 / beta != 0) fitted per transpose to
+  //    single-stream runs at M = N = 8192, K = 512 .. 8192 (148 - 150 TFLOP/s at K = 8192, beta = 0, for all four).
+  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 4 % faster per k than the small tile with a
+  //    small fixed cost: f_w + 2 * c * K / 1.042 per round of 512; ahead of the large tile for beta != 0 up to K of
+  //    about 5000.
+  //  * a round of 512 small tiles: f_s + c * K.
+  // The constants are pl_gemm_fit's (built-in: c = 0.1207 us, f_s = 6 us, f_w = 5 | 10.6 us, g = 0.07 - 0.09, f = 10 |
+  // 44 - 55 us).  Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD,
+  // 32-cycle MFMAs) measured 70.7 against 73.4 TFLOP/s.
+  const pl_gemm_fit& fit = fit_in_use();
+  const int tr = an ? (bnn ? 0 : 1) : (bnn ? 2 : 3);
+  const int bi = beta_zero ? 0 : 1;
+  auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
+  const double k_us = fit.f32_small_us_per_k * (double)K;
+  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (fit.f32_small_fixed_us + k_us);
+  const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * (fit.f32_large_fixed_us[tr][bi] + 2.0 * k_us / (1.0 + fit.f32_large_gain[tr]));
+  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (fit.f32_wide_fixed_us[bi] + 2.0 * k_us / fit.f32_wide_gain);
+  // PARALIA_GEMM_LARGE_TILE: "0" small tiles only, "1" the large tile for every call, "2" the wide tile wherever it
+  // exists (NN), unset: the model
+  const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");
+  const int pinv = (pin && *pin) ? atoi(pin) : -1;
+  const bool other = sizeof(T) == 4 && c.splits == 1 && pinv != 0;
+  // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
+  auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
+  const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
+  const bool big_ok = other && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
+  c.big = big_ok && (pinv == 1 || (large_us < small_us && (!wide_ok || large_us <= wide_us)));
+  c.wide = !c.big && wide_ok && (pinv == 2 || wide_us < small_us);
+  c.tm = c.big || c.wide ? 256 : 128;
+  c.tn = c.big ? 256 : 128;
+  return c;
 }
 
 template <typename T>
@@ -748,41 +814,10 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (!A || !B || !C) return 5;
-  int kchunk = 0;
-  int splits = workspace ? pick_splits<T>(M, N, K, &kchunk) : 1;
-  if (splits > 1 && (long)splits * M * N * (long)sizeof(T) > workspace_bytes) splits = 1, kchunk = 0;
-  // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
-  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 7 - 9 % faster per k (all panels global -> LDS
-  //    directly, a 16-byte operand read per block and four k-steps), but a CU holds one such workgroup at a time, so
-  //    nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * 0.1207 us * K / (1 + g),
-  //    with g and f (beta == 0 / beta != 0) fitted per transpose to single-stream runs at M = N = 8192, K = 512 .. 8192
-  //    (148 - 150 TFLOP/s at K = 8192, beta = 0, for all four).
-  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 4 % faster per k than the small tile with a
-  //    small fixed cost: (5 | 10.6) us + 2 * 0.1207 us * K / 1.042 per round of 512; ahead of the large tile for
-  //    beta != 0 up to K of about 5000.
-  //  * a round of 512 small tiles: 6 us + 0.1207 us * K.
-  // Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD, 32-cycle MFMAs)
-  // measured 70.7 against 73.4 TFLOP/s.
-  struct LargeTileFit { double g, f0, f1; };
-  const LargeTileFit fit = an ? (bnn ? LargeTileFit{0.072, 10.0, 46.0} : LargeTileFit{0.088, 10.0, 44.0})
-                              : (bnn ? LargeTileFit{0.073, 9.0, 52.0} : LargeTileFit{0.076, 10.0, 55.0});
-  auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
-  const double k_us = 0.1207 * (double)K;
-  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (6.0 + k_us);
-  const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * ((beta == T(0) ? fit.f0 : fit.f1) + 2.0 * k_us / (1.0 + fit.g));
-  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * ((beta == T(0) ? 5.0 : 10.6) + 2.0 * k_us / 1.042);
-  // PARALIA_GEMM_LARGE_TILE: "0" small tiles only, "1" the large tile for every call, "2" the wide tile wherever it
-  // exists (NN), unset: the model
-  const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");
-  const int pinv = (pin && *pin) ? atoi(pin) : -1;
-  const bool other = sizeof(T) == 4 && splits == 1 && pinv != 0;
-  // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
-  auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
-  const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
-  const bool big_ok = other && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
-  const bool big = big_ok && (pinv == 1 || (large_us < small_us && (!wide_ok || large_us <= wide_us)));
-  const bool wide = !big && wide_ok && (pinv == 2 || wide_us < small_us);
-  const int TM_RT = big || wide ? 256 : 128, TN_RT = big ? 256 : 128;
+  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes);
+  const int kchunk = choice.kchunk, splits = choice.splits;
+  const bool big = choice.big, wide = choice.wide;
+  const int TM_RT = choice.tm, TN_RT = choice.tn;
   const int gm = (int)((M + TM_RT - 1) / TM_RT), gn = (int)((N + TN_RT - 1) / TN_RT);
   if ((long)gm * gn > INT32_MAX) return 2;
   const int vecA = ((reinterpret_cast<uintptr_t>(A) & 15) == 0 && lda % Tr::VEC == 0) ? 1 : 0;
@@ -844,6 +879,39 @@ extern "C" int pl_dgemm_tile(char transA, char transB, long M, long N, long K, d
 extern "C" int pl_sgemm_tile(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
                              const float* B, long ldb, float beta, float* C, long ldc, void* stream) {
   return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream);
+}
+
+extern "C" void pl_gemm_fit_defaults(pl_gemm_fit* fit) {
+  if (fit) plk::fit_defaults(fit);
+}
+extern "C" int pl_gemm_set_fit(const pl_gemm_fit* fit) {
+  if (!fit) { plk::fit_defaults(&plk::fit_in_use()); return 0; }
+  // a fit that would divide by zero or run backwards is refused as a whole
+  const bool sane = fit->lone_us_per_k[0] > 0 && fit->lone_us_per_k[1] > 0 && fit->lone_fixed_k >= 0 && fit->splitk_launch_us >= 0 &&
+                    fit->pass_bytes_per_us > 0 && fit->f32_small_us_per_k > 0 && fit->f32_small_fixed_us >= 0 && fit->f32_wide_gain > 0.5;
+  bool large_sane = true;
+  for (int t = 0; t < 4; ++t) large_sane = large_sane && fit->f32_large_gain[t] > -0.5 && fit->f32_large_fixed_us[t][0] >= 0 && fit->f32_large_fixed_us[t][1] >= 0;
+  if (!sane || !large_sane || fit->f32_wide_fixed_us[0] < 0 || fit->f32_wide_fixed_us[1] < 0) return PL_ERR_ARG;
+  plk::fit_in_use() = *fit;
+  return 0;
+}
+extern "C" int pl_gemm_get_fit(pl_gemm_fit* fit) {
+  if (!fit) return PL_ERR_NULL;
+  *fit = plk::fit_in_use();
+  return 0;
+}
+extern "C" int pl_gemm_tile_choice(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero, long workspace_bytes,
+                                   int* tile_m, int* tile_n, int* splits) {
+  const bool at = (transA == 'T' || transA == 't'), an = (transA == 'N' || transA == 'n');
+  const bool bt = (transB == 'T' || transB == 't'), bnn = (transB == 'N' || transB == 'n');
+  if (!(at || an) || !(bt || bnn)) return PL_ERR_TRANS;
+  if (M <= 0 || N <= 0 || K <= 0 || (elem_size != 8 && elem_size != 4)) return PL_ERR_DIM;
+  const plk::TileChoice c = elem_size == 8 ? plk::choose_tile<double>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes)
+                                           : plk::choose_tile<float>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes);
+  if (tile_m) *tile_m = c.tm;
+  if (tile_n) *tile_n = c.tn;
+  if (splits) *splits = c.splits;
+  return 0;
 }
 
 extern "C" long pl_gemm_tile_workspace_bytes(long M, long N, long K, int elem_size) {

@@ -1,10 +1,10 @@
 // Deploy-time microbenchmarks and database builder for one MI355X.
 //
-//   paralia_deploy <db_dir> [--quick] [--only gemm|gemv|blas1|link]
+//   paralia_deploy <db_dir> [--quick] [--only gemm|gemv|blas1|link|fit]
 //
 // Measures (1) the tile GEMM kernels over square T for the four transpose combinations, fp64 and fp32,
 // (2) daxpy / ddot over vector lengths and dgemv over square T for both transposes, (3) pinned-host <-> device 2-D tile copies in both directions and the
-// slowdown of each direction while the other is busy, (4) the power-state transient of the tile kernels after idle time;
+// slowdown of each direction while the other is busy, (4) the power-state transient of the tile kernels after idle time, (5) the constants of the tile-GEMM launcher's cost model;
 // writes the raw logs to <db_dir>/Benchmark-Results and the
 // tables the autotuner reads to <db_dir>/Processed.
 //
@@ -378,6 +378,156 @@ static void bench_transient(const std::string& db) {
   CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
 }
 
+// Least-squares line y = a + b x.
+static void fit_line(const std::vector<double>& x, const std::vector<double>& y, double* a, double* b) {
+  const double n = (double)x.size();
+  double sx = 0, sy = 0, sxx = 0, sxy = 0;
+  for (size_t i = 0; i < x.size(); ++i) { sx += x[i]; sy += y[i]; sxx += x[i] * x[i]; sxy += x[i] * y[i]; }
+  *b = (n * sxy - sx * sy) / (n * sxx - sx * sx);
+  *a = (sy - *b * sx) / n;
+}
+
+// The constants of the tile-GEMM launcher's cost model and of the plan simulator that are not table rows
+// (pl_gemm_fit, KernelFit): time per launch of a product with one workgroup per compute unit over K (per-k cost and
+// fixed part of a lone 128 x 128 workgroup), of M = N = 8192 products over K with each fp32 macro tile pinned (per-k
+// cost and fixed cost per round of the small, wide and large tile, per transpose and for beta == 0 / != 0), the gap
+// between two launches of a stream, the rate of the scale-add pass, and what a slab of a thin start costs beyond its
+// share of the tile.  Written to Processed/Kernel-fit_dev-0.log as "name: value" lines; not a file of the reference.
+static void bench_fit(const std::string& db, bool quick) {
+  const long big = 8192, one_round = 2048;
+  void* A = CoCoMalloc(big * big * 8, 0, 0);
+  void* B = CoCoMalloc(big * big * 8, 0, 0);
+  void* C = CoCoMalloc(big * big * 8, 0, 1);
+  CoCoVecInit((double*)A, big * big, 42, 0);
+  CoCoVecInit((double*)B, big * big, 43, 0);
+  CoCoVecInit((double*)C, big * big, 44, 0);
+  void* st[2];
+  for (auto& s : st) must(pl_stream_create(&s), "stream");
+  const std::vector<long> Ks = quick ? std::vector<long>{1024, 4096, 8192} : std::vector<long>{512, 1024, 2048, 4096, 8192};
+  // time per launch in microseconds: n launches on `queues` streams round-robin, wall time / n
+  auto per_launch_us = [&](bool f64, char ta, char tb, long M, long N, long K, double beta, int queues) {
+    auto launch = [&](int q) {
+      char* c = (char*)C + (size_t)q * M * N * 8;   // a C of its own per stream
+      const long lda = ta == 'N' ? M : K, ldb = tb == 'N' ? K : N;
+      if (f64) must(pl_dgemm_tile(ta, tb, M, N, K, 1e-3, (const double*)A, lda, (const double*)B, ldb, beta, (double*)c, M, st[q]), "gemm");
+      else must(pl_sgemm_tile(ta, tb, M, N, K, 1e-3f, (const float*)A, lda, (const float*)B, ldb, (float)beta, (float*)c, M, st[q]), "gemm");
+    };
+    const double flop = 2.0 * M * N * K;
+    const int n = std::max(2 * queues, std::min(64, (int)(2.0e12 / flop)) / queues * queues);
+    auto run = [&]() {
+      const double t0 = csecond();
+      for (int i = 0; i < n; ++i) launch(i % queues);
+      for (int q = 0; q < queues; ++q) must(pl_stream_sync(st[q]), "sync");
+      return (csecond() - t0) / n;
+    };
+    run();
+    return sample_until_stable(run).mean * 1e6;
+  };
+  auto over_k = [&](bool f64, char ta, char tb, long MN, double beta, double rounds, double* fixed_us, double* us_per_k) {
+    std::vector<double> x, y;
+    for (long K : Ks) { x.push_back((double)K); y.push_back(per_launch_us(f64, ta, tb, MN, MN, K, beta, 1) / rounds); }
+    fit_line(x, y, fixed_us, us_per_k);
+  };
+  KernelFit k;
+  pl_gemm_fit& f = k.launcher;
+  // the gap between two launches of a stream: a scale-add over a 16 x 16 tile, 400 in a row
+  {
+    auto run = [&]() {
+      const double t0 = csecond();
+      for (int i = 0; i < 400; ++i) must(pl_dgeadd_tile(16, 16, 1.0, (const double*)A, 16, (const double*)C, 16, (double*)C, 16, st[0]), "geadd");
+      must(pl_stream_sync(st[0]), "sync");
+      return (csecond() - t0) / 400;
+    };
+    run();
+    f.splitk_launch_us = sample_until_stable(run).mean * 1e6;
+  }
+  // the scale-add pass over a tile, 3 T^2 elements.  At T = 1024 on one and the same tile: the slices a split-K product
+  // adds up were written a moment ago and are still in the caches.  At T = 2048 over twelve different tiles in turn
+  // (768 MiB, more than the memory-side cache holds): the lazy reduce reads a C tile the copy engine has just brought in.
+  auto geadd_rate = [&](long T, int tiles) {
+    auto run = [&]() {
+      const double t0 = csecond();
+      for (int i = 0; i < 48; ++i) {
+        const size_t off = (size_t)(i % tiles) * T * T;
+        must(pl_dgeadd_tile(T, T, 0.5, (const double*)A + off, T, (const double*)C + off, T, (double*)C + off, T, st[0]), "geadd");
+      }
+      must(pl_stream_sync(st[0]), "sync");
+      return (csecond() - t0) / 48;
+    };
+    run();
+    return 3.0 * T * T * 8 / sample_until_stable(run).mean;
+  };
+  f.pass_bytes_per_us = geadd_rate(1024, 1) / 1e6;
+  k.geadd_bytes_per_s = geadd_rate(2048, 12);
+  // one 128 x 128 workgroup per compute unit (2048 x 2048: 256 tiles), small tile, no split: time over K
+  setenv("PARALIA_GEMM_LARGE_TILE", "0", 1);
+  double a = 0, b = 0;
+  // (beta == 0, as the kernels of a split product run: they write their slice and read nothing of C)
+  over_k(true, 'N', 'N', one_round, 0.0, 1.0, &a, &b);
+  f.lone_us_per_k[0] = b;
+  const double fixed_k64 = a / b;
+  over_k(false, 'N', 'N', one_round, 0.0, 1.0, &a, &b);
+  f.lone_us_per_k[1] = b;
+  f.lone_fixed_k = std::max(0.0, 0.5 * (fixed_k64 + a / b));
+  // fp32, M = N = 8192: 8 rounds of 512 small tiles (beta == 0 and != 0 pooled), 4 rounds of 512 wide tiles (NN), 4 rounds
+  // of 256 large tiles per transpose
+  double a0 = 0, b0 = 0, a1 = 0, b1 = 0;
+  over_k(false, 'N', 'N', big, 0.0, 8.0, &a0, &b0);
+  over_k(false, 'N', 'N', big, 1.0, 8.0, &a1, &b1);
+  f.f32_small_us_per_k = 0.5 * (b0 + b1);
+  f.f32_small_fixed_us = std::max(0.0, 0.5 * (a0 + a1));
+  setenv("PARALIA_GEMM_LARGE_TILE", "2", 1);
+  over_k(false, 'N', 'N', big, 0.0, 4.0, &a0, &b0);
+  over_k(false, 'N', 'N', big, 1.0, 4.0, &a1, &b1);
+  f.f32_wide_gain = 2.0 * f.f32_small_us_per_k / (0.5 * (b0 + b1));
+  f.f32_wide_fixed_us[0] = std::max(0.0, a0);
+  f.f32_wide_fixed_us[1] = std::max(0.0, a1);
+  setenv("PARALIA_GEMM_LARGE_TILE", "1", 1);
+  const char tas[4] = {'N', 'N', 'T', 'T'}, tbs[4] = {'N', 'T', 'N', 'T'};
+  for (int t = 0; t < 4; ++t) {
+    over_k(false, tas[t], tbs[t], big, 0.0, 4.0, &a0, &b0);
+    over_k(false, tas[t], tbs[t], big, 1.0, 4.0, &a1, &b1);
+    f.f32_large_gain[t] = 2.0 * f.f32_small_us_per_k / (0.5 * (b0 + b1)) - 1.0;
+    f.f32_large_fixed_us[t][0] = std::max(0.0, a0);
+    f.f32_large_fixed_us[t][1] = std::max(0.0, a1);
+    // a merged chain saves one such fixed cost per launch it saves, less the gap the launches would have had anyway
+    k.merge_saving_us_f32[t] = std::max(0.0, f.f32_large_fixed_us[t][1] - f.splitk_launch_us);
+  }
+  unsetenv("PARALIA_GEMM_LARGE_TILE");
+  k.merge_saving_us_f64 = f.splitk_launch_us;
+  // a slab of a thin start, two launches sharing the device: 2048 x 2048 x 1024 against half of 2048^3
+  {
+    const double full = per_launch_us(true, 'N', 'N', 2048, 2048, 2048, 1.0, 2);
+    const double half = per_launch_us(true, 'N', 'N', 2048, 2048, 1024, 1.0, 2);
+    k.slab_fixed_us = std::max(0.0, half - 0.5 * full);
+  }
+  char out[1024];
+  snprintf(out, sizeof out, "%s/Processed/Kernel-fit_dev-0.log", db.c_str());
+  FILE* fp = fopen(out, "w");
+  if (!fp) { fprintf(stderr, "cannot write %s\n", out); exit(1); }
+  fprintf(fp, "# constants of the tile-GEMM launcher's cost model and of the plan simulator, microseconds unless named otherwise\n");
+  fprintf(fp, "lone_us_per_k_f64: %.6g\nlone_us_per_k_f32: %.6g\nlone_fixed_k: %.6g\nsplitk_launch_us: %.6g\npass_bytes_per_us: %.6g\n",
+          f.lone_us_per_k[0], f.lone_us_per_k[1], f.lone_fixed_k, f.splitk_launch_us, f.pass_bytes_per_us);
+  fprintf(fp, "f32_small_us_per_k: %.6g\nf32_small_fixed_us: %.6g\nf32_wide_gain: %.6g\nf32_wide_fixed_us_beta0: %.6g\nf32_wide_fixed_us_beta1: %.6g\n",
+          f.f32_small_us_per_k, f.f32_small_fixed_us, f.f32_wide_gain, f.f32_wide_fixed_us[0], f.f32_wide_fixed_us[1]);
+  static const char* const trans[4] = {"NN", "NT", "TN", "TT"};
+  for (int t = 0; t < 4; ++t)
+    fprintf(fp, "f32_large_gain_%s: %.6g\nf32_large_fixed_us_beta0_%s: %.6g\nf32_large_fixed_us_beta1_%s: %.6g\nmerge_saving_us_f32_%s: %.6g\n", trans[t],
+            f.f32_large_gain[t], trans[t], f.f32_large_fixed_us[t][0], trans[t], f.f32_large_fixed_us[t][1], trans[t], k.merge_saving_us_f32[t]);
+  fprintf(fp, "merge_saving_us_f64: %.6g\ngeadd_bytes_per_s: %.6g\nslab_fixed_us: %.6g\n", k.merge_saving_us_f64, k.geadd_bytes_per_s, k.slab_fixed_us);
+  fprintf(fp, "# not measured by this tool: the share of a streamed call's launches that run without a partner, fitted to streamed calls\n");
+  fprintf(fp, "lone_share: %.6g\n", k.lone_share);
+  fclose(fp);
+  fprintf(stderr, "kernel fit: lone workgroup %.4f (fp64) / %.4f (fp32) us per k + %.0f k, launch gap %.2f us, scale-add %.2f / %.2f TB/s\n",
+          f.lone_us_per_k[0], f.lone_us_per_k[1], f.lone_fixed_k, f.splitk_launch_us, f.pass_bytes_per_us / 1e6, k.geadd_bytes_per_s / 1e12);
+  fprintf(stderr, "kernel fit: fp32 small %.4f us per k + %.1f us; wide gain %.3f, fixed %.1f | %.1f us; slab +%.2f us\n", f.f32_small_us_per_k,
+          f.f32_small_fixed_us, f.f32_wide_gain, f.f32_wide_fixed_us[0], f.f32_wide_fixed_us[1], k.slab_fixed_us);
+  for (int t = 0; t < 4; ++t)
+    fprintf(stderr, "kernel fit: fp32 large %s gain %.3f, fixed %.1f | %.1f us\n", trans[t], f.f32_large_gain[t], f.f32_large_fixed_us[t][0], f.f32_large_fixed_us[t][1]);
+  for (auto s : st) pl_stream_destroy(s);
+  CoCoFree(A, 0); CoCoFree(B, 0); CoCoFree(C, 0);
+}
+
 static void bench_link(const std::string& db, bool quick) {
   const long maxDim = quick ? 4352 : 10000;
   std::vector<long> dims = sweep(256, 256, maxDim, 8);
@@ -475,7 +625,7 @@ static void bench_link(const std::string& db, bool quick) {
 
 int main(int argc, char** argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: %s <db_dir> [--quick] [--only gemm|gemv|blas1|link]\n", argv[0]);
+    fprintf(stderr, "usage: %s <db_dir> [--quick] [--only gemm|gemv|blas1|link|fit]\n", argv[0]);
     return 2;
   }
   const std::string db = argv[1];
@@ -499,6 +649,7 @@ int main(int argc, char** argv) {
       bench_gemm<float>(db, "Sgemm", quick, queues);
       bench_transient(db);
     }
+    if (only.empty() || only == "gemm" || only == "fit") bench_fit(db, quick);
     if (only.empty() || only == "gemv") bench_gemv(db, quick);
     if (only.empty() || only == "blas1") {
       bench_blas1(db, "Daxpy", quick);

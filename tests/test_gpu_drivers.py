@@ -216,6 +216,24 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
     assert 0.5 * tr_shipped["Amplitude"] < tr["Amplitude"] < 2.0 * tr_shipped["Amplitude"], (tr, tr_shipped)
     for k in ("Recovery", "Idle"):
         assert 0.25 * tr_shipped[k] < tr[k] < 4.0 * tr_shipped[k], (k, tr, tr_shipped)
+    # the constants of the launcher's cost model and of the simulator (Kernel-fit_dev-0.log): per-k costs within 10 % of
+    # the shipped fit, gains within 0.03, fixed costs (intercepts of a line through three to five points, a few
+    # microseconds of tens) and the scale-add rate within a wider band; every name the shipped file has is there
+    def fit(path):
+        return {k.strip(): float(v) for k, v in (line.split(":") for line in open(path) if not line.startswith("#") and ":" in line)}
+    kf, kf_shipped = fit(os.path.join(fresh, "Kernel-fit_dev-0.log")), fit(os.path.join(shipped, "Kernel-fit_dev-0.log"))
+    assert set(kf) == set(kf_shipped), set(kf) ^ set(kf_shipped)
+    for k in ("lone_us_per_k_f64", "lone_us_per_k_f32", "f32_small_us_per_k"):
+        close(kf[k], kf_shipped[k], 0.10, k)
+    for k in kf:
+        if "gain" in k:
+            assert abs(kf[k] - kf_shipped[k]) <= 0.03, (k, kf[k], kf_shipped[k])
+        elif "fixed_us" in k or k.startswith("merge_saving_us_f32"):
+            assert abs(kf[k] - kf_shipped[k]) <= max(4.0, 0.25 * kf_shipped[k]), (k, kf[k], kf_shipped[k])
+    assert 0.5 * kf_shipped["lone_fixed_k"] < kf["lone_fixed_k"] < 2.0 * kf_shipped["lone_fixed_k"]
+    assert 1.0 < kf["splitk_launch_us"] < 10.0 and 0 <= kf["slab_fixed_us"] < 6.0
+    for k in ("pass_bytes_per_us", "geadd_bytes_per_s"):
+        assert 0.5 * kf_shipped[k] < kf[k] < 2.0 * kf_shipped[k], (k, kf[k], kf_shipped[k])
     # matrix-vector and vector kernels take 40 - 80 us at the largest sizes of the quick sweep: launch and
     # synchronisation are a visible part of that, and working sets of 128 - 384 MiB sit partly inside the memory-side
     # cache, so these differ more between machines than the millisecond-scale GEMM tiles: a wider band
@@ -236,3 +254,8 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
         preds.append(info.pred_t)
     L.PARALiA_set_db_dir(None)
     close(preds[0], preds[1], 0.10, "predicted seconds for dgemm 16384^3")
+    # the loaders handed the launcher the fit of the database read last (the shipped one)
+    from paralia_framework_amd import binding
+    got = binding.gemm_fit()
+    pkg.check(L.pl_gemm_get_fit(C.byref(got)), "get fit")
+    assert abs(got.lone_us_per_k[0] - kf_shipped["lone_us_per_k_f64"]) < 1e-9 and abs(got.f32_large_gain[1] - kf_shipped["f32_large_gain_NT"]) < 1e-9

@@ -410,3 +410,65 @@ def test_planner_time_of_a_first_call(L, pkg, monkeypatch):
             best = min(best, (time.perf_counter() - t0) * 1e3)
         print("  planner %s %d x %d x %d: %.2f ms (T = %d, order %d)" % (func.decode(), M, N, K, best, info.T, info.order_id), flush=True)
         assert best <= bound_ms, (func, M, N, K, best)
+
+
+def test_kernel_fit_file_is_optional_and_drives_launcher_and_simulator(L, pkg, tmp_path, monkeypatch):
+    """Processed/Kernel-fit_dev-0.log (not a file of the reference): the fitted constants of the tile-GEMM launcher's cost
+    model and of the plan simulator.  A database without it leaves the built-in values in force; one with it hands
+    them to the launcher when it is loaded, and a perturbed file changes what the launcher and the planner choose."""
+    from paralia_framework_amd import binding
+    monkeypatch.delenv("PARALIA_GEMM_LARGE_TILE", raising=False)
+    monkeypatch.delenv("PARALIA_MERGE_CHAINS", raising=False)
+    info = pkg.atc_info()
+
+    def load(db):
+        assert L.PARALiA_autotune(str(db).encode(), b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+        f = binding.gemm_fit()
+        assert L.pl_gemm_get_fit(C.byref(f)) == 0
+        return f
+
+    def choice(es, tr, M, N, K, beta0, ws):
+        tm, tn, sp = C.c_int(), C.c_int(), C.c_int()
+        assert L.pl_gemm_tile_choice(es, tr[0:1], tr[1:2], M, N, K, beta0, ws, C.byref(tm), C.byref(tn), C.byref(sp)) == 0
+        return tm.value, tn.value, sp.value
+    builtin = binding.gemm_fit()
+    L.pl_gemm_fit_defaults(C.byref(builtin))
+    # no file: the synthetic database has none
+    f = load(DB_SYNTH.decode())
+    assert bytes(f) == bytes(builtin)
+    assert choice(4, b"NT", 8192, 8192, 8192, 1, 0) == (256, 256, 1)          # large fp32 tile for a long k
+    assert choice(8, b"NN", 1024, 1024, 1024, 0, 1 << 30)[2] > 1               # few tiles: K is split
+    # the shipped database has one; its values are what the launcher then holds
+    shipped = _shipped_db(pkg)
+    f = load(shipped)
+    vals = {k.strip(): float(v) for k, v in (l.split(":") for l in open(os.path.join(shipped, "Processed", "Kernel-fit_dev-0.log")) if ":" in l and not l.startswith("#"))}
+    assert abs(f.lone_us_per_k[0] - vals["lone_us_per_k_f64"]) < 1e-12 and abs(f.f32_large_fixed_us[3][1] - vals["f32_large_fixed_us_beta1_TT"]) < 1e-12
+    order_shipped = info.order_id
+    assert order_shipped >= 80000                                               # merged K chains pay at 4 us a launch
+    # a perturbed copy: large tiles that gain nothing and cost a millisecond a round, a split that costs a millisecond
+    # to launch, merging that saves nothing
+    db = tmp_path / "db"
+    shutil.copytree(shipped, db)
+    lines = []
+    for l in open(db / "Processed" / "Kernel-fit_dev-0.log"):
+        k = l.split(":")[0].strip()
+        if k.startswith("f32_large_fixed_us"):
+            l = "%s: 1000\n" % k
+        elif k == "splitk_launch_us":
+            l = "%s: 1000\n" % k
+        elif k == "merge_saving_us_f64":
+            l = "%s: 0\n" % k
+        lines.append(l)
+    open(db / "Processed" / "Kernel-fit_dev-0.log", "w").writelines(lines)
+    f = load(db)
+    assert f.splitk_launch_us == 1000.0
+    assert choice(4, b"NT", 8192, 8192, 8192, 1, 0)[:2] != (256, 256)
+    assert choice(8, b"NN", 1024, 1024, 1024, 0, 1 << 30)[2] == 1
+    assert info.order_id % 160000 < 80000                                       # nothing to gain: chains are not merged
+    # a value out of range makes the database unusable, like any other malformed file of it: the call falls back to the
+    # tile heuristic and says so
+    open(db / "Processed" / "Kernel-fit_dev-0.log", "a").write("lone_share: 7\n")
+    assert L.PARALiA_autotune(str(db).encode(), b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
+    assert info.has_db == 0 and info.selected_by == b"heuristic"
+    assert L.pl_gemm_set_fit(None) == 0                                         # back to the built-in values for the tests that follow
+    L.PARALiA_set_db_dir(None)
