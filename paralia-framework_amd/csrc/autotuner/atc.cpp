@@ -409,13 +409,13 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         return std::max(0.5 * total, total - saved);
       };
       // ... and at both ends nothing overlaps: no kernel starts before the first pair of A and B tiles has crossed the
-      // link (a quarter of each, if the thin start cuts them into four slabs), and the C tile of the last kernel goes
+      // link (an eighth of each, if the graded thin start applies), and the C tile of the last kernel goes
       // back (after its lazy reduce) when every kernel has finished.
       auto call_floor = [&](const paralia::GemmProblem& gp, const paralia::StageTimes& st) {
         double t = compute_floor(gp, st);
-        const double quarter = (double)gp.T * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz;
-        if (gp.a_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(quarter, (double)gp.tm(gp.Mg() - 1) * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz);
-        if (gp.b_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(quarter, (double)gp.tn(gp.Ng() - 1) * std::min<long>(gp.T, problem.D3) / 4.0 * problem.dtype_sz);
+        const double eighth = (double)gp.T * std::min<long>(gp.T, problem.D3) / 8.0 * problem.dtype_sz;
+        if (gp.a_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(eighth, (double)gp.tm(gp.Mg() - 1) * std::min<long>(gp.T, problem.D3) / 8.0 * problem.dtype_sz);
+        if (gp.b_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(eighth, (double)gp.tn(gp.Ng() - 1) * std::min<long>(gp.T, problem.D3) / 8.0 * problem.dtype_sz);
         if (gp.c_remote) {
           const double smallest = (double)std::min(gp.tm(0), gp.tm(gp.Mg() - 1)) * std::min(gp.tn(0), gp.tn(gp.Ng() - 1));
           t += st.d2h_ti + st.d2h_tb * smallest * problem.dtype_sz;

@@ -197,20 +197,32 @@ struct Block {
   bool ever_used = false;
 };
 
-void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w) {
+// What each stream is already known to be behind: covered[s][r] = the latest command of stream r that some earlier
+// command of stream s waited for.  Streams run their commands in order, so a later command of s need not wait for
+// that command of r, or any before it, again.  In a k-outer panel most subkernels read tiles their stream's earlier
+// subkernels already waited for.
+constexpr int PLAN_STREAMS = STREAM_EXEC0 + MAX_EXEC_QUEUES;
+struct Covered {
+  int at[PLAN_STREAMS][PLAN_STREAMS];
+  Covered() { for (auto& row : at) for (int& x : row) x = -1; }
+};
+
+void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w, Covered& cov) {
   if (w < 0) return;
   if (cmds[w].stream == c.stream) return;  // stream order already covers it
+  if (w <= cov.at[c.stream][cmds[w].stream]) return;  // an earlier command of this stream waited for it, or for a later one
   for (int i = 0; i < c.nwait; ++i) {
     if (c.wait[i] == w) return;
     if (cmds[c.wait[i]].stream == cmds[w].stream) {
       // streams run their commands in order: the later of two commands of one stream covers the earlier
-      if (w > c.wait[i]) { c.wait[i] = w; cmds[w].signals = true; }
+      if (w > c.wait[i]) { c.wait[i] = w; cmds[w].signals = true; cov.at[c.stream][cmds[w].stream] = w; }
       return;
     }
   }
   if (c.nwait >= MAX_WAITS) throw std::runtime_error("gemm plan: too many dependencies on one command");
   c.wait[c.nwait++] = w;
   cmds[w].signals = true;
+  cov.at[c.stream][cmds[w].stream] = w;
 }
 
 }  // namespace
@@ -219,7 +231,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   if (p_in.T <= 0 || p_in.M <= 0 || p_in.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
   GemmPlan plan;
   plan.p = p_in;
-  if (order_id < 0 || order_id / ORDER_K_SPLIT > 2) throw std::runtime_error("gemm plan: unknown order id");
+  if (order_id < 0 || order_id / ORDER_K_SPLIT > 3) throw std::runtime_error("gemm plan: unknown order id");
   plan.p.k_split = 1 << (order_id / ORDER_K_SPLIT);
   const GemmProblem& p = plan.p;
   if (order_id >= ORDER_K_SPLIT && p.slabs() == 1) throw std::runtime_error("gemm plan: this problem has no thin start");
@@ -273,6 +285,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   int cur_pos = 0;
   std::vector<Cmd>& cmds = plan.cmds;
   cmds.reserve(plan.task_order.size() * 2 + 16);
+  Covered covered;
 
   auto release = [&](int b, int after_cmd) {
     blocks[b].kind = -1;
@@ -358,7 +371,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
     c.kind = CMD_GEMM; c.mi = open.mi; c.ni = open.ni; c.ki = open.ki0; c.kn = open.kn; c.stream = STREAM_EXEC0 + queue_of[open.ci];
     c.block = p.c_remote ? c_blk[open.ci] : -1; c.a_block = open.ablk; c.b_block = open.bblk; c.beta_mode = open.beta_mode;
     cmds.push_back(c);
-    for (int x : open.waits) add_wait(cmds, cmds.back(), x);
+    for (int x : open.waits) add_wait(cmds, cmds.back(), x, covered);
     open.active = false;
     return (int)cmds.size() - 1;
   };
@@ -382,7 +395,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
         Cmd c;
         c.kind = CMD_FETCH_A; c.mi = mi; c.ki = ki; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
-        for (int x : w) add_wait(cmds, cmds.back(), x);
+        for (int x : w) add_wait(cmds, cmds.back(), x, covered);
         blocks[b].kind = 0; blocks[b].idx = ai; blocks[b].content_cmd = blocks[b].last_touch = (int)cmds.size() - 1;
         a_blk[ai] = b;
         ++plan.n_fetch[0];
@@ -398,7 +411,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
         Cmd c;
         c.kind = CMD_FETCH_B; c.ki = ki; c.ni = ni; c.stream = STREAM_H2D; c.block = b;
         cmds.push_back(c);
-        for (int x : w) add_wait(cmds, cmds.back(), x);
+        for (int x : w) add_wait(cmds, cmds.back(), x, covered);
         blocks[b].kind = 1; blocks[b].idx = bi; blocks[b].content_cmd = blocks[b].last_touch = (int)cmds.size() - 1;
         b_blk[bi] = b;
         ++plan.n_fetch[1];
@@ -464,21 +477,21 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
         Cmd f;
         f.kind = CMD_FETCH_C; f.mi = mi; f.ni = ni; f.stream = STREAM_H2D; f.block = sb;
         cmds.push_back(f);
-        for (int x : w) add_wait(cmds, cmds.back(), x);
+        for (int x : w) add_wait(cmds, cmds.back(), x, covered);
         const int fetch_idx = (int)cmds.size() - 1;
         blocks[sb].kind = 3; blocks[sb].idx = ci; blocks[sb].content_cmd = fetch_idx;
         ++plan.n_fetch[2];
         Cmd r;
         r.kind = CMD_REDUCE; r.mi = mi; r.ni = ni; r.stream = STREAM_EXEC0 + queue_of[ci]; r.block = accb; r.a_block = sb;
         cmds.push_back(r);
-        add_wait(cmds, cmds.back(), fetch_idx);
+        add_wait(cmds, cmds.back(), fetch_idx, covered);
         last = (int)cmds.size() - 1;
         release(sb, last);
       }
       Cmd wb;
       wb.kind = CMD_WRITEBACK; wb.mi = mi; wb.ni = ni; wb.stream = STREAM_D2H; wb.block = accb;
       cmds.push_back(wb);
-      add_wait(cmds, cmds.back(), last);
+      add_wait(cmds, cmds.back(), last, covered);
       release(accb, (int)cmds.size() - 1);
       c_blk[ci] = -1;
     }
@@ -578,7 +591,7 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
         case CMD_GEMM:
           for (int k = c.ki; k < c.ki + c.kn; ++k) {
             if (k < p.slabs() && p.slabs() > 1)
-              dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.T) / p.slabs() + st.slab_fixed * std::max(1.0, 1024.0 / (double)p.tk(k));
+              dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.T) * (double)p.tk(k) / (double)p.T + st.slab_fixed * std::max(1.0, 1024.0 / (double)p.tk(k));
             else dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
           }
           if (c.kn > 1) dur = std::max(0.5 * dur, dur - (c.kn - 1) * st.merge_saving * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2);
@@ -771,10 +784,10 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
   if (st.thin_start && (p.a_remote || p.b_remote) && !probe && p.pool_blocks >= gemm_full_block_num(unsplit))
     for (Group& g : grp) {
       if (g.id < 0) continue;
-      // a thin start takes at most three quarters of the first A and B tiles' fetch off a call: a group that would
-      // still trail the other group's plain best by more than that is not worth the six plans
+      // a thin start takes at most seven eighths of the first A and B tiles' fetch off a call: a group that would
+      // still trail the other group's plain best by more than that is not worth the nine plans
       const Group& other = grp[&g == &grp[0] ? 1 : 0];
-      const double thin_gain = ((p.a_remote ? 1 : 0) + (p.b_remote ? 1 : 0)) * 0.75 * st.h2d_tb * (double)p.T * std::min(p.T, p.K) * p.elem;
+      const double thin_gain = ((p.a_remote ? 1 : 0) + (p.b_remote ? 1 : 0)) * 0.875 * st.h2d_tb * (double)p.T * std::min(p.T, p.K) * p.elem;
       if (!st.exhaustive && other.id >= 0 && g.r.t_total - thin_gain > other.r.t_total) continue;
       // makespans that differ only in the last bits are ties (compared in single precision), and ties keep the
       // candidate order, as the choice above does
@@ -783,7 +796,7 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
       const double unsplit_best = g.r.t_total;
       std::vector<int> thin_ids;
       for (size_t b = 0; b < std::min<size_t>(3, g.ranked.size()); ++b)
-        for (int s = 1; s <= 2; ++s) thin_ids.push_back(g.ranked[b].second + s * ORDER_K_SPLIT);
+        for (int s = 1; s <= 3; ++s) thin_ids.push_back(g.ranked[b].second + s * ORDER_K_SPLIT);
       const std::vector<Evaluated> thin = evaluate_orders(p, st, thin_ids);
       for (size_t i = 0; i < thin_ids.size(); ++i)
         if (thin[i].ok && thin[i].evictions == 0 && thin[i].r.t_total < unsplit_best * (1.0 - 1e-3) && thin[i].r.t_total < g.r.t_total) {

@@ -28,20 +28,29 @@ struct GemmProblem {
   int elem = 8;                                              // bytes per element
   int exec_queues = 2;
   long pool_blocks = 0;                                      // device blocks available (>= 3 when anything is remote)
-  // Thin start: the first k tile is cut into k_split slabs of T / k_split (each its own k tile, fetched and multiplied
-  // separately), so the first subkernels can start after a fraction of the first tiles has crossed the link.  Taken
-  // as 1 when it does not apply (K < T, T not divisible, slabs under 16).
+  // Thin start: the first k tile is cut into slabs (each its own k tile, fetched and multiplied separately), so the
+  // first subkernels can start after a fraction of the first tiles has crossed the link.  k_split = 2 or 4: that many
+  // equal slabs; k_split = 8: a graded start, four slabs of T/8, T/8, T/4 and T/2 -- the first kernels start after an
+  // eighth of a tile, and the slabs grow as the link gets ahead, so the later ones pay less per launch.  Taken as 1
+  // when it does not apply (K < T, T not divisible, slabs under 16).
   int k_split = 1;
-  int slabs() const { return (k_split > 1 && K >= T && T % k_split == 0 && T / k_split >= 16) ? k_split : 1; }
+  int slabs() const {
+    if (k_split == 8) return (K >= T && T % 8 == 0 && T / 8 >= 16) ? 4 : 1;
+    return (k_split > 1 && K >= T && T % k_split == 0 && T / k_split >= 16) ? k_split : 1;
+  }
+  long slab_k0(int i) const {  // first k of slab i of the first tile (i == slabs(): T)
+    if (k_split != 8) return (long)i * (T / slabs());
+    return i == 0 ? 0 : i == 1 ? T / 8 : i == 2 ? T / 4 : i == 3 ? T / 2 : T;
+  }
   int Mg() const { return (int)((M + T - 1) / T); }
   int Ng() const { return (int)((N + T - 1) / T); }
   int Kg() const { return K > 0 ? (int)((K + T - 1) / T) + slabs() - 1 : 1; }
   long tm(int mi) const { return mi == Mg() - 1 ? M - (long)mi * T : T; }
   long tn(int ni) const { return ni == Ng() - 1 ? N - (long)ni * T : T; }
-  long k0(int ki) const { const int s = slabs(); return ki < s ? (long)ki * (T / s) : (long)(ki - s + 1) * T; }  // first k of tile ki
+  long k0(int ki) const { const int s = slabs(); return ki < s ? slab_k0(ki) : (long)(ki - s + 1) * T; }  // first k of tile ki
   long tk(int ki) const {
     if (K <= 0) return 0;
-    if (ki < slabs() && slabs() > 1) return T / slabs();
+    if (ki < slabs() && slabs() > 1) return slab_k0(ki + 1) - slab_k0(ki);
     return ki == Kg() - 1 ? K - k0(ki) : T;
   }
   long subkernels() const { return (long)Mg() * Ng() * Kg(); }
@@ -103,7 +112,7 @@ constexpr int ORDER_BLOCK_ROWS = 100;
 // Panel widths therefore stay below 100, and w = 99 stands for "the whole grid", however many tiles that is (a grid of
 // 128 column tiles would otherwise read as the block 1 x 28).
 constexpr int ORDER_FULL_PANEL = 99;
-// + 160000 * s: thin start (GemmProblem::k_split) with 2^s slabs, s = 1 or 2.
+// + 160000 * s: thin start (GemmProblem::k_split = 2^s): s = 1 or 2: 2^s equal slabs; s = 3: the graded start.
 constexpr int ORDER_K_SPLIT = 160000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);

@@ -80,6 +80,7 @@ def check_daxpy_against_blas(orc, got, blas_result, alpha, x, y0):
 
 def k_tiles(info, K, T=None):
     """k tiles of a streamed GEMM plan: ceil(K / T), plus the extra slabs of a thin start (order id 160000 * s + ...:
-    the first k tile is cut into 2^s slabs that are fetched and multiplied separately)."""
+    the first k tile is cut into 2 (s = 1) or 4 (s = 2: equal, s = 3: graded) slabs that are fetched and multiplied
+    separately)."""
     T = T or info.T
-    return -(-K // T) + (1 << (info.order_id // 160000)) - 1
+    return -(-K // T) + (1, 2, 4, 4)[info.order_id // 160000] - 1

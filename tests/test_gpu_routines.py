@@ -518,7 +518,34 @@ def test_gemm_merged_k_chains_exact_on_integers(pkg, L, orc, ta, tb, order, locs
             bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
             info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 3.0, beta, bA, ra, bB, rb, bC, M, T=T)
             assert info.order_id == order and info.subkernel_num == 5 * 6 * k_tiles(info, K)
-            assert k_tiles(info, K) == 5 + (1 << (order // 160000)) - 1
+            assert k_tiles(info, K) == 5 + (1, 2, 4, 4)[order // 160000] - 1
+            assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("order", [480000, 480002, 560002, 490001, 480202])
+@pytest.mark.parametrize("locs", [(-1, -1, -1), (-2, -1, 0), (0, -2, -2)])
+def test_gemm_graded_start_exact_on_integers(pkg, L, orc, ta, tb, order, locs, monkeypatch):
+    """Order ids of 480000 and above: the graded thin start, the first k tile cut into slabs of T/8, T/8, T/4 and T/2 (T =
+    128: 16, 16, 32, 64 deep; 400 = 3 k tiles + a ragged one become 7), fetched and multiplied as k tiles of their own,
+    alone, with merged K chains (560002) and with a block order (480202).  Integer data, ragged tiles, every transpose,
+    pinned / pageable / device operands, beta = 0 over NaN and beta != 0, both types: bit for bit the untiled result."""
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+    M, N, K, T = 289, 353, 400 + [480000, 480002, 560002, 490001, 480202].index(order), 128   # a new problem for the metadata cache per order
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    rng = np.random.default_rng(order + 5 * len(ta + tb))
+    for dtype, brute in ((np.float64, orc.orc_dgemm_bruteforce), (np.float32, orc.orc_sgemm_bruteforce)):
+        A = rng.integers(-4, 5, ra * ca).astype(dtype)
+        B = rng.integers(-4, 5, rb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, M * N).astype(dtype)
+        for beta in (0.0, -2.0):
+            ref = C0.copy()
+            brute(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M)
+            start = np.full(M * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+            bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
+            info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 2.0, beta, bA, ra, bB, rb, bC, M, T=T)
+            assert info.order_id == order and k_tiles(info, K) == 4 + 3 and info.subkernel_num == 3 * 3 * 7
             assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
 
 
@@ -542,7 +569,7 @@ def test_gemm_thin_start_with_odd_slabs(pkg, L, orc, ta, tb, order, T, monkeypat
             brute(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A), ra, ptr(B), rb, -1.0, ptr(ref), M)
             bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, C0, locs[2])
             info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 2.0, -1.0, bA, ra, bB, rb, bC, M, T=T)
-            assert info.order_id == order and k_tiles(info, K) == -(-K // T) + (1 << (order // 160000)) - 1
+            assert info.order_id == order and k_tiles(info, K) == -(-K // T) + (1, 2, 4, 4)[order // 160000] - 1
             assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, locs)
 
 

@@ -12,12 +12,16 @@ K_AXIS = object()   # marks a slice request along k, whose tiles need not be uni
 
 
 def kbounds(K, T, slabs=1):
-    """First k of every k tile, and K: tiles of T, the first one cut into `slabs` equal slabs by a thin start (order ids
-    of 160000 and above) when K >= T and the slabs are whole and at least 16 deep."""
+    """First k of every k tile, and K: tiles of T, the first one cut by a thin start (order ids of 160000 and above) when
+    K >= T and the slabs are whole and at least 16 deep: slabs = 2 or 4 equal slabs, slabs = 8 the graded start (four
+    slabs of T/8, T/8, T/4, T/2)."""
     if K <= 0:
         return [0, 0]
     b = list(range(0, K, T)) + [K]
-    if slabs > 1 and K >= T and T % slabs == 0 and T // slabs >= 16:
+    if slabs == 8:
+        if K >= T and T % 8 == 0 and T // 8 >= 16:
+            b = [0, T // 8, T // 4, T // 2] + b[1:]
+    elif slabs > 1 and K >= T and T % slabs == 0 and T // slabs >= 16:
         b = [i * (T // slabs) for i in range(slabs)] + b[1:]
     return b
 
@@ -255,8 +259,11 @@ def test_pipeline_simulation(pkg, L):
     # a thin start (order id 160000 * s + ...: first k tile in 2^s slabs) multiplies the same flops in more launches,
     # every slab priced at 2 us on top of its share of the tile time
     slabs = 1 << (picked.value // 160000)
-    assert slabs in (1, 2, 4)
-    assert abs(busy[1] - (512 * 0.24e-3 + (64 * slabs * 2e-6 if slabs > 1 else 0.0))) < 1e-9
+    assert slabs in (1, 2, 4, 8)
+    # (slabs of 1024 and deeper cost 2 us, shallower ones in inverse proportion to their depth; 8 = the graded start:
+    # T/8, T/8, T/4, T/2 of a 2048-tile)
+    extra = {1: 0.0, 2: 64 * 2 * 2e-6, 4: 64 * 4 * 4e-6, 8: 64 * (8e-6 + 8e-6 + 4e-6 + 2e-6)}[slabs]
+    assert abs(busy[1] - (512 * 0.24e-3 + extra)) < 1e-9
     assert abs(busy[0] - 128 * 0.6e-3) < 1e-9 and abs(busy[2] - 64 * 0.6e-3) < 1e-9
     unsplit = L.PARALiA_gemm_plan_simulate(*args, picked.value % 160000, *st, None, None)
     assert best <= unsplit                              # and is only taken when the simulated call gets shorter
@@ -421,24 +428,32 @@ def test_merged_chains_need_the_whole_working_set_and_pay_only_with_a_saving(pkg
     assert picked.value % 160000 < 80000 and best <= plain
 
 
-@pytest.mark.parametrize("order", [160000, 160002, 170001, 320000, 320003, 330002, 240002, 410001, 180002])
+@pytest.mark.parametrize("order", [160000, 160002, 170001, 320000, 320003, 330002, 240002, 410001, 180002, 480000, 490002, 560001, 480203])
 @pytest.mark.parametrize("locs", [(1, 1, 1), (1, 1, 0), (0, 1, 1), (1, 0, 0)])
 @pytest.mark.parametrize("beta_zero", [0, 1])
 def test_thin_start_plans(pkg, order, locs, beta_zero):
-    """Order ids of 160000 * s and above: the first k tile is cut into 2^s slabs, each a k tile of its own (fetched into
-    its own block, multiplied by its own launch, beta' = 0 on a C tile's first slab only).  Every subkernel of the
-    finer k grid fires once, every tile is fetched once, and the plan -- with merged K chains expanded -- keeps the
-    invariants, replays to the exact result on integers and orders every hazard.  K = 110 with T = 32: 4 k tiles become
-    5 (two slabs of 16); four slabs of 8 are too thin, so ids of 320000 and above are refused here, as they are when K < T."""
+    """Order ids of 160000 * s and above: the first k tile is cut into slabs (s = 1: two, s = 2: four equal ones, s = 3:
+    the graded start of T/8, T/8, T/4, T/2), each a k tile of its own (fetched into its own block, multiplied by its
+    own launch, beta' = 0 on a C tile's first slab only).  Every subkernel of the finer k grid fires once, every tile
+    is fetched once, and the plan -- with merged K chains expanded -- keeps the invariants, replays to the exact result
+    on integers and orders every hazard.  K = 110 with T = 32: 4 k tiles become 5 (two slabs of 16); four slabs of 8
+    are too thin, so ids of 320000 and above are refused here, as they are when K < T; the graded start needs T = 128
+    (slabs of 16, 16, 32, 64)."""
     M, N, K, T = 90, 70, 110, 32
     a_r, b_r, c_r = locs
     slabs = 1 << (order // 160000)
-    if slabs == 4:
+    if slabs >= 4:
         with pytest.raises(pkg.ParaliaError, match="thin start"):
             pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
         T = 64                                                   # 2 k tiles become 5: slabs of 16, 16, 16, 16 and 46
+    if slabs == 8:
+        with pytest.raises(pkg.ParaliaError, match="thin start"):
+            pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)     # an eighth of 64 is too thin
+        M, N, K, T = 300, 200, 310, 128                          # 3 k tiles become 6: 16, 16, 32, 64, 128 and 54
     Mg, Ng, Kg = grids(M, N, K, T, slabs)
-    assert Kg == -(-K // T) + slabs - 1
+    assert Kg == -(-K // T) + min(slabs, 4) - 1
+    if slabs == 8:
+        assert kbounds(K, T, 8) == [0, 16, 32, 64, 128, 256, 310]
     rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)
     flat = expand_merged(rows)
     full = 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
@@ -519,6 +534,6 @@ def test_whole_grid_panel_on_grids_of_a_hundred_tiles_and_more(pkg, L):
 
 
 def test_unknown_order_ids_are_refused(pkg):
-    for order in (480000, 640001, -5):
+    for order in (640000, 800001, -5):
         with pytest.raises(pkg.ParaliaError, match="unknown order id"):
             pkg.plan_rows(256, 256, 256, 64, 1, 1, 1, 0, 8, 2, 0, order)
