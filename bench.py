@@ -139,9 +139,10 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
                     help="only the headline configuration (the others take about a minute)")
-    ap.add_argument("--pmc-probe", choices=["host", "tile"], default=None,
+    ap.add_argument("--pmc-probe", choices=["host", "tile", "stile"], default=None,
                     help="for rocprofv3 --pmc runs: 'host' makes three headline calls and nothing else, 'tile' launches one "
-                         "daxpy of N = 2^28 (4 GiB read, 2 GiB written: the counters' scale) and one device-resident tile GEMM")
+                         "daxpy of N = 2^28 (4 GiB read, 2 GiB written: the counters' scale) and one device-resident tile GEMM, "
+                         "'stile' three device-resident fp32 N/T launches of --size (the 256 x 256 tile)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives one GPU; run with --gpus 1 (sharding over several GPUs is a design note only)")
@@ -184,6 +185,15 @@ def main():
         for _ in range(3):
             step_host()
         print(json.dumps({"pmc_probe": "host", "calls": 3, "n": n, "T": int(info.T), "subkernels": int(info.subkernel_num)}))
+        return
+    if args.pmc_probe == "stile":
+        fa, fb, fc = (Buf(pkg, n * n, np.float32, 0) for _ in range(3))
+        for b, seed in ((fa, 0), (fb, 1)):
+            pkg.check(L.PARALiA_vec_init_f32(b.ptr, b.n, seed, 0), "vec init")
+        for _ in range(3):
+            pkg.check(L.pl_sgemm_tile(b"N", b"T", n, n, n, 1.0, fa.ptr, n, fb.ptr, n, 0.0, fc.ptr, n, None), "tile")
+        sync()
+        print(json.dumps({"pmc_probe": "stile", "gemm_n": n}))
         return
     if args.pmc_probe == "tile":
         m = 1 << 28
