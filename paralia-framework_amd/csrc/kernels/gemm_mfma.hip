@@ -204,33 +204,62 @@ __device__ __forceinline__ void lds_store(T* __restrict__ xs, const typename Tra
   for (int i = 0; i < L::NV; ++i) lds_put<L, T>(xs + L::slot_offset(tid, i), regs[i]);
 }
 
+// A wave-uniform pointer pinned to scalar registers.  The address arithmetic in front of it stays on the scalar unit and
+// the compiler cannot merge it with the per-lane offset added behind it, so an LDS-DMA request is issued as
+// "scalar base + 32-bit lane offset": between two MFMAs the wave spends two scalar adds and the request, no vector
+// instruction and one address register instead of two.  With 64-bit per-lane addresses (a v_lshl_add_u64 per request)
+// the requests cost 2 - 3.5 % of the fp32 256 x 256 tile's rate at 8192^3, with this form 0.2 %.
+template <typename T>
+__device__ __forceinline__ const char* scalar_base(const T* p) {
+  const unsigned long long b = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b), hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  return reinterpret_cast<const char*>(((unsigned long long)hi << 32) | lo);
+}
+
 // Row `row` of an MN-major panel straight from global memory into LDS (global_load_lds_dwordx4): the 64 lanes of a wave
 // fetch 16 bytes each and the hardware puts lane l's at the wave's LDS base + 16 l, so one instruction moves one 1 KiB
 // row (256 floats or 128 doubles) and neither staging registers nor LDS store instructions are spent on it.  The LDS
-// base is wave-uniform, which is why the row stride of the padded layout can stay.
+// base is wave-uniform, which is why the row stride of the padded layout can stay.  voff: dma_lane_offset<.., false>.
 template <typename T, int EXT>
-__device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs, int inst, int lane, int s_mn) {
+__device__ __forceinline__ void dma_row(const T* __restrict__ g, long ld, T* xs, int inst, int s_mn, unsigned voff) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int PER = 1024 / (int)sizeof(T), PARTS = EXT / PER > 0 ? EXT / PER : 1;  // elements per instruction, instructions per row
   const int row = inst / PARTS, part = inst % PARTS;
-  const T* p = g + (16 / (int)sizeof(T)) * lane + part * PER + (long)row * ld;
-  __builtin_amdgcn_global_load_lds(p, xs + row * s_mn + part * PER, 16, 0, 0);
+  const char* base = scalar_base(g + part * PER + (long)row * ld);
+  __builtin_amdgcn_global_load_lds(reinterpret_cast<const T*>(base + voff), xs + row * s_mn + part * PER, 16, 0, 0);
 #endif
 }
 
 // Rows of a K-major panel (each BK elements = NC 16-byte chunks) straight into the swizzled layout of Lds<.., SWZ>: wave
 // instruction number `inst` of the panel fills 64 / NC consecutive rows; lane l fills chunk position l % NC of row
-// l / NC with the global chunk (l % NC) ^ swz(row).
+// l / NC with the global chunk (l % NC) ^ swz(row).  voff: dma_lane_offset<.., true>.
 template <typename L, typename T>
-__device__ __forceinline__ void dma_krows(const T* __restrict__ g, long ld, T* xs, int inst, int lane) {
+__device__ __forceinline__ void dma_krows(const T* __restrict__ g, long ld, T* xs, int inst, unsigned voff) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  constexpr int NC = L::NC, RPI = 64 / NC;
-  const int row = inst * RPI + lane / NC;
-  const int gc = (lane % NC) ^ L::swz(row);
-  const T* p = g + (long)row * ld + gc * Traits<T>::VEC;
-  __builtin_amdgcn_global_load_lds(p, xs + inst * RPI * L::S_K, 16, 0, 0);
+  constexpr int RPI = 64 / L::NC;
+  const char* base = scalar_base(g + (long)(inst * RPI) * ld);
+  __builtin_amdgcn_global_load_lds(reinterpret_cast<const T*>(base + voff), xs + inst * RPI * L::S_K, 16, 0, 0);
 #endif
 }
+
+// Where a lane's 16 bytes of a dma_row / dma_krows request sit relative to the request's wave-uniform base, in bytes.
+// The same for every request a wave makes for an operand: its requests are 4 apart and 4 * RPI rows are a whole swizzle
+// period.  K-major: up to 64 / NC - 1 rows of ld elements, which is why the launcher keeps operands whose leading
+// dimension does not fit 32 bits that way on the staged path (PLK_DMA_MAX_LD_BYTES).
+template <typename L, typename T, bool KMAJOR>
+__device__ __forceinline__ unsigned dma_lane_offset(long ld, int wave, int lane) {
+  if constexpr (KMAJOR) {
+    constexpr int NC = L::NC, RPI = 64 / NC;
+    static_assert((4 * RPI / L::RPB) % NC == 0, "the requests of a wave must share their swizzle");
+    const int row = wave * RPI + lane / NC;
+    const int gc = (lane % NC) ^ L::swz(row);
+    return (unsigned)(lane / NC) * (unsigned)ld * (unsigned)sizeof(T) + (unsigned)(gc * 16);
+  } else {
+    return (unsigned)(16 * lane);
+  }
+}
+// largest row stride in bytes of a K-major operand loaded by dma_krows (8 rows of it must stay under 2^32)
+#define PLK_DMA_MAX_LD_BYTES (1L << 29)
 
 // Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
 // give each XCD a contiguous range of logical ids, then walk that range in groups of 8 block rows.
@@ -275,7 +304,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // fp64: only with a K-major A (TN 73.2 -> 74.0, TT 72.6 -> 73.6 TFLOP/s at 8192^3); NN measured the same either way
   // (73.55 / 73.45) and keeps the register path.
   constexpr bool SWZL = DIR && ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
-                        ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16 && AK) ||
+                        ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16) ||
                          (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
   constexpr bool V2 = PLK_V2 && SWZL && sizeof(T) == 4 && (AK || BKM);
   using LA = Lds<T, AK, BM, BK, SWZL>;
@@ -302,6 +331,10 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
 
   int bm, bn;
   block_coords(blockIdx.x, gm, gn, bm, bn);
+  // the divisions above run on the vector unit; back in scalar registers the tile origins and every address derived
+  // from them are scalar arithmetic
+  bm = __builtin_amdgcn_readfirstlane(bm);
+  bn = __builtin_amdgcn_readfirstlane(bn);
   const int m0 = bm * BM, n0 = bn * BN;
   const int mrem = min(M - m0, BM), nrem = min(N - n0, BN);
   const bool fast = (mrem == BM) && (nrem == BN) && vecA && vecB;
@@ -429,6 +462,38 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         bnv[v][i] = (SWZL && BKM) ? b_kp[ks * KV + v][buf * STAGE + i * BLK * LB::S_K] : lane_b[buf * STAGE + (ks * KV + v) * B_KS + b_blk(i)];
     }
   };
+  // one LDS read instruction of read_ops, by its number (A's first); V2 only
+  auto read_one = [&](int buf, int ks, T (&am)[KV][NBM], T (&bnv)[KV][NBN], int e) {
+    if constexpr (V2) {
+      const int g = (ks * KV) / SPG, h = ((ks * KV) % SPG) / KV;
+      if (e < RD_A) {
+        if constexpr (AK) {
+          const vec_t x = *reinterpret_cast<const vec_t*>(a_kp[2 * g + h] + buf * STAGE + e * BLK * LA::S_K);
+#pragma unroll
+          for (int v = 0; v < KV; ++v) am[v][e] = x[v];
+        } else {
+          typedef T opv_t __attribute__((ext_vector_type(PFA)));
+          const int v = e / (NBM / PFA), q = e % (NBM / PFA);
+          const opv_t x = *reinterpret_cast<const opv_t*>(lane_a + buf * STAGE + (g * G + h * KV + v) * LA::S_MN + q * BLK * PFA);
+#pragma unroll
+          for (int f = 0; f < PFA; ++f) am[v][q * PFA + f] = x[f];
+        }
+      } else {
+        const int eb = e - RD_A;
+        if constexpr (BKM) {
+          const vec_t x = *reinterpret_cast<const vec_t*>(b_kp[2 * g + h] + buf * STAGE + eb * BLK * LB::S_K);
+#pragma unroll
+          for (int v = 0; v < KV; ++v) bnv[v][eb] = x[v];
+        } else {
+          typedef T opv_t __attribute__((ext_vector_type(PFB)));
+          const int v = eb / (NBN / PFB), q = eb % (NBN / PFB);
+          const opv_t x = *reinterpret_cast<const opv_t*>(lane_b + buf * STAGE + (g * G + h * KV + v) * LB::S_MN + q * BLK * PFB);
+#pragma unroll
+          for (int f = 0; f < PFB; ++f) bnv[v][q * PFB + f] = x[f];
+        }
+      }
+    }
+  };
   auto mfma_step = [&](const T (&am)[KV][NBM], const T (&bnv)[KV][NBN]) {
 #pragma unroll
     for (int v = 0; v < KV; ++v)
@@ -458,11 +523,12 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     constexpr bool A_DIR = DIR_T && (SWZL || (!AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024));
     constexpr bool B_DIR = A_DIR;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned voff_a0 = dma_lane_offset<LA, T, AK>(lda, wave_u, lane), voff_b0 = dma_lane_offset<LB, T, BKM>(ldb, wave_u, lane);
     if constexpr (A_DIR) {
 #pragma unroll
       for (int i = 0; i < NVA; ++i) {
-        if constexpr (AK) dma_krows<LA, T>(Ab, lda, smem, wave_u + 4 * i, lane);
-        else dma_row<T, BM>(Ab, lda, smem, wave_u + 4 * i, lane, LA::S_MN);
+        if constexpr (AK) dma_krows<LA, T>(Ab, lda, smem, wave_u + 4 * i, voff_a0);
+        else dma_row<T, BM>(Ab, lda, smem, wave_u + 4 * i, LA::S_MN, voff_a0);
       }
     } else {
       gload<LA, T, false>(Ab, lda, 0, 0, true, ra, tid);
@@ -472,8 +538,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     if constexpr (B_DIR) {
 #pragma unroll
       for (int i = 0; i < NVB; ++i) {
-        if constexpr (BKM) dma_krows<LB, T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane);
-        else dma_row<T, BN>(Bb, ldb, smem + ASZ, wave_u + 4 * i, lane, LB::S_MN);
+        if constexpr (BKM) dma_krows<LB, T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, voff_b0);
+        else dma_row<T, BN>(Bb, ldb, smem + ASZ, wave_u + 4 * i, LB::S_MN, voff_b0);
       }
     } else {
       gload<LB, T, false>(Bb, ldb, 0, 0, true, rb, tid);
@@ -493,15 +559,15 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     // staged vector number r -> index into (A vectors, then B vectors)
     constexpr int REG0 = A_DIR ? NVA : 0;
     // one side instruction of the panel (row request, LDS store or global load), by its number in issue order
-    auto side_item = [&](int slot, T* nxt_a, T* nxt_b, const T* ga, const T* gb) {
+    auto side_item = [&](int slot, T* nxt_a, T* nxt_b, const T* ga, const T* gb, unsigned voff_a, unsigned voff_b) {
       if (slot < NDIR) {
         const int vec = (A_DIR ? 0 : NVA) + slot;  // direct rows: A's first when both are direct
         if (vec < NVA) {
-          if constexpr (AK) dma_krows<LA, T>(ga, lda, nxt_a, wave_u + 4 * vec, lane);
-          else dma_row<T, BM>(ga, lda, nxt_a, wave_u + 4 * vec, lane, LA::S_MN);
+          if constexpr (AK) dma_krows<LA, T>(ga, lda, nxt_a, wave_u + 4 * vec, voff_a);
+          else dma_row<T, BM>(ga, lda, nxt_a, wave_u + 4 * vec, LA::S_MN, voff_a);
         } else {
-          if constexpr (BKM) dma_krows<LB, T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane);
-          else dma_row<T, BN>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), lane, LB::S_MN);
+          if constexpr (BKM) dma_krows<LB, T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), voff_b);
+          else dma_row<T, BN>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), LB::S_MN, voff_b);
         }
         return;
       }
@@ -526,13 +592,48 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
       const int kt2 = min(kt + 2, nkt - 1), kt1 = min(kt + 1, nkt - 1);
       const T* const ga = Ab + (A_DIR ? kt1 : kt2) * a_kstep;
       const T* const gb = Bb + (B_DIR ? kt1 : kt2) * b_kstep;
+      // the lane offsets of the row requests, opaque per panel: hoisted out of the loop the compiler widens them to 64
+      // bits once and adds the scalar bases on the vector unit again
+      unsigned voff_a = voff_a0, voff_b = voff_b0;
+      if constexpr (NDIR > 0) asm volatile("" : "+v"(voff_a), "+v"(voff_b));
+      if constexpr (V2 && NREG == 0) {
+        // fp32 256 x 256 with a K-major operand, all panels direct.  The source is written in issue order -- an MFMA, then
+        // the operand read or row request that goes behind it -- because the compiler keeps a row request (an LDS write
+        // as far as it knows) in program order with every LDS read: with all reads of a step in front of its requests
+        // the requests end up three in a row behind the step's last read, and the four waves of the compute unit send
+        // twelve to the one address unit at once.  Spread one at a time, 10 or 11 MFMAs apart: NN 152.3 -> 152.8, TN and
+        // TT 151.8 -> 152.7 TFLOP/s at 8192^3 (NT, which is not V2, loses 0.5 that way and keeps the order below).
+        constexpr int PER_STEP_D = (SIDE + KS - 2) / (KS - 1), DMA_BEHIND = 2;
+#pragma unroll
+        for (int ks = 0; ks < KS - 1; ++ks) {
+#pragma unroll
+          for (int m = 0; m < MFMAS; ++m) {
+            const int v = m / (NBN * NBM), i = (m / NBM) % NBN, j = m % NBM;
+            acc[i][j] = Tr::mfma(bnv[ks & 1][v][i], am[ks & 1][v][j], acc[i][j]);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+            for (int e = 0; e < NREADS; ++e)
+              if (e * MFMAS / NREADS == m) {
+                read_one(cur, ks + 1, am[(ks + 1) & 1], bnv[(ks + 1) & 1], e);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+              }
+#pragma unroll
+            for (int c = 0; c < PER_STEP_D; ++c)
+              if (c * MFMAS / PER_STEP_D + DMA_BEHIND == m && ks * PER_STEP_D + c < SIDE) {
+                side_item(ks * PER_STEP_D + c, nxt_a, nxt_b, ga, gb, voff_a, voff_b);
+                __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+              }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
 #pragma unroll
       for (int ks = 0; ks < KS - 1; ++ks) {
         read_ops(cur, ks + 1, am[(ks + 1) & 1], bnv[(ks + 1) & 1]);
 #pragma unroll
         for (int q = 0; q < PER_STEP; ++q) {
           const int slot = ks * PER_STEP + q;
-          if (slot < SIDE) side_item(slot, nxt_a, nxt_b, ga, gb);
+          if (slot < SIDE) side_item(slot, nxt_a, nxt_b, ga, gb, voff_a, voff_b);
         }
         mfma_step(am[ks & 1], bnv[ks & 1]);
         // Issue order: the NREADS operand reads of the next step and the PER_STEP side instructions alternate and are
@@ -564,6 +665,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
           }
         }
         __builtin_amdgcn_sched_barrier(0);
+      }
       }
       if constexpr (A_DIR || B_DIR) __builtin_amdgcn_s_waitcnt(0x0F70);  // the rows requested during this panel are in LDS
       __syncthreads();
@@ -753,7 +855,7 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
 // Macro tile and split count of one product.
 struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; };
 template <typename T>
-TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes) {
+TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true) {
   TileChoice c;
   c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
   if (c.splits > 1 && (long)c.splits * M * N * (long)sizeof(T) > workspace_bytes) c.splits = 1, c.kchunk = 0;
@@ -786,7 +888,7 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
   auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
   const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
-  const bool big_ok = other && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
+  const bool big_ok = other && large_allowed && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
   c.big = big_ok && (pinv == 1 || (large_us < small_us && (!wide_ok || large_us <= wide_us)));
   c.wide = !c.big && wide_ok && (pinv == 2 || wide_us < small_us);
   c.tm = c.big || c.wide ? 256 : 128;
@@ -814,7 +916,10 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (!A || !B || !C) return 5;
-  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes);
+  // a K-major operand loaded straight into LDS takes eight rows per request with 32-bit lane offsets: leading dimensions
+  // beyond that keep the tiles that stage through registers
+  const bool dma_fits = (!at || lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES) && (!bnn || ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES);
+  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits);
   const int kchunk = choice.kchunk, splits = choice.splits;
   const bool big = choice.big, wide = choice.wide;
   const int TM_RT = choice.tm, TN_RT = choice.tn;
@@ -830,8 +935,8 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   T* const k_C = splits > 1 ? workspace : C;
   const long k_ldc = splits > 1 ? M : ldc;
   constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
-  // fp64 with direct panels (every transpose but NN) only where the k extent of a workgroup is long
-  const bool stage = sizeof(T) == 8 && (splits > 1 ? kchunk : K) < 1536;
+  // fp64 with direct panels only where the k extent of a workgroup is long
+  const bool stage = sizeof(T) == 8 && ((splits > 1 ? kchunk : K) < 1536 || !dma_fits);
 #define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK, DIRF)                                                                            \
   hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK, DIRF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
                      A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)
@@ -841,7 +946,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
       if (big) { PLK_LAUNCH_T(AKF, BKF, 256, 256, PLK_F32_BIG_BK, true); break; }   \
       if (wide) { PLK_LAUNCH_T(AKF, BKF, 256, 128, PLK_F32_BK, true); break; }      \
     }                                                                               \
-    if constexpr (sizeof(T) == 8 && !(!AKF && BKF)) {                               \
+    if constexpr (sizeof(T) == 8) {                                                 \
       if (stage) { PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, false); break; }      \
     }                                                                               \
     PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, true);                               \

@@ -100,6 +100,83 @@ def test_dgemm_tile_exact_on_integers(pkg, L, orc, ta, tb):
         assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+def test_dgemm_tile_direct_panels_exact_on_integers(pkg, L, orc, ta, tb):
+    """K of 1536 and more: every fp64 panel is requested straight into LDS (interior workgroups; the ragged edge
+    workgroups of the same launch take the guarded loop).  Small integers, so the result is exact in any order."""
+    M, N, K = 300, 260, 1552
+    rng = np.random.default_rng(11)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 2, rb + 4, M + 2
+    A = rng.integers(-8, 9, lda * ca).astype(np.float64)
+    B = rng.integers(-8, 9, ldb * cb).astype(np.float64)
+    C0 = rng.integers(-8, 9, ldc * N).astype(np.float64)
+    for alpha, beta in ((1.0, 0.0), (-2.0, 3.0)):
+        got = run_gemm(pkg, L, np.float64, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc)
+        ref = C0.copy()
+        orc.orc_dgemm_bruteforce(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A), lda, ptr(B), ldb, beta, ptr(ref), ldc)
+        assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("operand,extra", [("A", 0), ("A", 2), ("B", 0), ("B", 2)])
+def test_dgemm_tile_k_major_operand_with_a_row_stride_of_half_a_gigabyte(pkg, L, orc, operand, extra):
+    """A K-major operand whose rows are exactly 2^29 bytes apart -- the largest stride whose panels the kernel still
+    requests straight into LDS (eight rows per request, 32-bit lane offsets) -- and one just beyond, where the launcher
+    keeps the tile that stages through registers.  The operand spans 64 GiB of device addresses; its 128 rows of K
+    values are filled by the seeded generator, whose stream the oracle reproduces on the host."""
+    K, ld = 1600, (1 << 26) + extra
+    M, N = (128, 256) if operand == "A" else (256, 128)
+    rows = 128
+    big = Buf(pkg, (rows - 1) * ld + K, np.float64, 0)
+    dense = np.empty((rows, K))
+    for r in range(rows):
+        pkg.check(L.PARALiA_vec_init_f64(big.at(r * ld), K, 100 + r, 0), "vec init")
+        dense[r] = rand_f64(K, 100 + r)
+    other = rand_f64(256 * K, 7)   # the MN-major partner: 256 x K (A, TransA = N) or K x 256 read as B^T (TransB = T)
+    C0 = rand_f64(M * N, 8)
+    dO, dC = Buf(pkg, other.size, np.float64, 0).set(other), Buf(pkg, C0.size, np.float64, 0).set(C0)
+    print("gemm f64 K-major", operand, "ld", ld, flush=True)
+    if operand == "A":   # C = 1.5 A^T B^T + 0.5 C: A is K x M with lda = ld, B is N x K
+        pkg.check(L.pl_dgemm_tile(b"T", b"T", M, N, K, 1.5, big.ptr, ld, dO.ptr, N, 0.5, dC.ptr, M, None), "gemm tile")
+    else:                # C = 1.5 A B + 0.5 C: A is M x K, B is K x N with ldb = ld
+        pkg.check(L.pl_dgemm_tile(b"N", b"N", M, N, K, 1.5, dO.ptr, M, big.ptr, ld, 0.5, dC.ptr, M, None), "gemm tile")
+    sync(pkg)
+    got = dC.get()
+    big.free()
+    ref = C0.copy()
+    flat = dense.ravel()
+    if operand == "A":
+        orc.orc_dgemm_bruteforce(b"T", b"T", M, N, K, 1.5, ptr(flat), K, ptr(other), N, 0.5, ptr(ref), M)
+        d = 1.5 * np.linalg.norm(flat) * np.linalg.norm(other) + 0.5 * np.linalg.norm(C0)
+    else:
+        orc.orc_dgemm_bruteforce(b"N", b"N", M, N, K, 1.5, ptr(other), M, ptr(flat), K, 0.5, ptr(ref), M)
+        d = 1.5 * np.linalg.norm(other) * np.linalg.norm(flat) + 0.5 * np.linalg.norm(C0)
+    assert orc.orc_normwise_err_f64(ptr(got), ptr(ref), M, N, M, M, d) < TOL64
+
+
+def test_sgemm_large_tile_gives_way_to_a_row_stride_beyond_its_lane_offsets(pkg, L, orc):
+    """The 256 x 256 fp32 tile pinned, op(A) K-major with rows more than 2^29 bytes apart: the launcher takes the
+    small tile (and its grid), whatever the pin says."""
+    M, N, K, lda = 3, 300, 600, (1 << 27) + 4
+    dA = Buf(pkg, (M - 1) * lda + K, np.float32, 0)
+    dense = np.empty((M, K), dtype=np.float32)
+    for r in range(M):
+        pkg.check(L.PARALiA_vec_init_f32(dA.at(r * lda), K, 40 + r, 0), "vec init f32")
+        dense[r] = rand_f32(K, 40 + r)
+    B, C0 = rand_f32(K * N, 5), rand_f32(M * N, 6)
+    dB, dC = Buf(pkg, B.size, np.float32, 0).set(B), Buf(pkg, C0.size, np.float32, 0).set(C0)
+    with large_tile("1"):
+        pkg.check(L.pl_sgemm_tile(b"T", b"N", M, N, K, 1.0, dA.ptr, lda, dB.ptr, K, 1.0, dC.ptr, M, None), "gemm tile")
+    sync(pkg)
+    got = dC.get()
+    ref = C0.copy()
+    flat = dense.ravel()
+    orc.orc_sgemm_bruteforce(b"T", b"N", M, N, K, 1.0, ptr(flat), K, ptr(B), K, 1.0, ptr(ref), M)
+    d = float(np.linalg.norm(flat.astype(np.float64)) * np.linalg.norm(B.astype(np.float64)) + np.linalg.norm(C0.astype(np.float64)))
+    assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
+
+
 def test_dgemm_tile_special_scalars(pkg, L):
     M, N, K = 100, 90, 50
     A, B, C0 = rand_f64(M * K, 1), rand_f64(K * N, 2), rand_f64(M * N, 3)
