@@ -47,6 +47,12 @@
 #define PLK_SWZ 3
 #endif
 // 1: the permuted k order of gemm_kernel's V2 (fp32 256 x 256 tiles with a K-major operand)
+// fp64 workgroups whose k extent is shorter than this keep the panels staged through registers (0: none does.  With
+// 64-bit lane addresses in the row requests, short k chunks ran 7 - 12 % slower direct than staged and the limit was
+// 1536; with scalar bases direct panels win or tie from K = 128 on, split-K chunks included)
+#ifndef PLK_F64_STAGE_BELOW
+#define PLK_F64_STAGE_BELOW 0
+#endif
 #ifndef PLK_V2
 #define PLK_V2 1
 #endif
@@ -282,9 +288,8 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, i
 // for two workgroups per CU (two waves per SIMD that fill each other's gaps); larger ones run one workgroup per CU with
 // the whole register file and fewer operand reads and global loads per MFMA.
 // AK: op(A) is K-major in memory (TransA == 'T').  BKM: op(B) is K-major in memory (TransB == 'N').
-// DIR = false: every panel through registers, plain layouts (what the launcher picks for short k: a panel requested
-// straight into LDS is asked for one panel ahead, one staged through registers two, and on the cold first panels of a
-// short k chunk that is the difference: fp64 1024^3 split four ways ran 7 - 12 % slower with direct panels).
+// DIR = false: every panel through registers, plain layouts (what the launcher picks for fp64 operands whose K-major
+// rows are too far apart for the 32-bit lane offsets of a row request).
 template <typename T, bool AK, bool BKM, int BM, int BN, int BK, bool DIR = true>
 __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 8 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
@@ -301,8 +306,8 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // operand then has the values of KV = VEC = 4 consecutive steps side by side in LDS: ONE 16-byte read per block
   // serves four steps, where the plain order needs a read per block and two steps.  MN-major operands do not care which
   // row a step reads.  (For fp64 the same order was slower than the plain one: 71.3 against 73.0 TFLOP/s NN.)
-  // fp64: only with a K-major A (TN 73.2 -> 74.0, TT 72.6 -> 73.6 TFLOP/s at 8192^3); NN measured the same either way
-  // (73.55 / 73.45) and keeps the register path.
+  // fp64, 8192^3: NN 73.2 -> 74.9, NT 73.5 -> 74.6, TN 73.9 -> 74.9, TT 73.6 -> 74.9 TFLOP/s against staging every panel
+  // through registers (with 64-bit lane addresses in the row requests NN had measured the same either way).
   constexpr bool SWZL = DIR && ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
                         ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16) ||
                          (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
@@ -806,15 +811,15 @@ __global__ void splitk_reduce_kernel(int M, int N, int splits, T alpha, const T*
 // The launcher's fitted constants (pl_gemm_fit in the public header): built-in values measured on an MI355X, replaced
 // by what the deploy database holds once the autotuner has loaded it.
 inline void fit_defaults(pl_gemm_fit* f) {
-  f->lone_us_per_k[0] = 0.117; f->lone_us_per_k[1] = 0.0585;
-  f->lone_fixed_k = 48.0;
-  f->splitk_launch_us = 4.0;
-  f->pass_bytes_per_us = 4.0e6;
-  f->f32_small_us_per_k = 0.1207;
-  f->f32_small_fixed_us = 6.0;
-  f->f32_wide_gain = 1.042;
-  f->f32_wide_fixed_us[0] = 5.0; f->f32_wide_fixed_us[1] = 10.6;
-  const double g[4] = {0.072, 0.088, 0.073, 0.076}, f0[4] = {10.0, 10.0, 9.0, 10.0}, f1[4] = {46.0, 44.0, 52.0, 55.0};
+  f->lone_us_per_k[0] = 0.115; f->lone_us_per_k[1] = 0.065;
+  f->lone_fixed_k = 80.0;
+  f->splitk_launch_us = 3.0;
+  f->pass_bytes_per_us = 6.2e6;
+  f->f32_small_us_per_k = 0.1192;
+  f->f32_small_fixed_us = 5.1;
+  f->f32_wide_gain = 1.018;
+  f->f32_wide_fixed_us[0] = 3.4; f->f32_wide_fixed_us[1] = 9.6;
+  const double g[4] = {0.085, 0.089, 0.084, 0.085}, f0[4] = {10.0, 10.4, 10.4, 10.8}, f1[4] = {45.0, 43.5, 52.0, 53.0};
   for (int t = 0; t < 4; ++t) { f->f32_large_gain[t] = g[t]; f->f32_large_fixed_us[t][0] = f0[t]; f->f32_large_fixed_us[t][1] = f1[t]; }
 }
 inline pl_gemm_fit& fit_in_use() {
@@ -860,17 +865,17 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
   if (c.splits > 1 && (long)c.splits * M * N * (long)sizeof(T) > workspace_bytes) c.splits = 1, c.kchunk = 0;
   // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
-  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 7 - 9 % faster per k (all panels global -> LDS
+  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 8 - 9 % faster per k (all panels global -> LDS
   //    directly, a 16-byte operand read per block and four k-steps), but a CU holds one such workgroup at a time, so
   //    nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * c * K / (1 + g), c the
   //    per-k time of a round of 512 small tiles, with g and f (beta == 0 / beta != 0) fitted per transpose to
-  //    single-stream runs at M = N = 8192, K = 512 .. 8192 (148 - 150 TFLOP/s at K = 8192, beta = 0, for all four).
-  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 4 % faster per k than the small tile with a
-  //    small fixed cost: f_w + 2 * c * K / 1.042 per round of 512; ahead of the large tile for beta != 0 up to K of
-  //    about 5000.
+  //    single-stream runs at M = N = 8192, K = 512 .. 8192 (152.6 - 152.8 TFLOP/s at K = 8192, beta = 0, for all four).
+  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 2 % faster per k than the small tile with a
+  //    small fixed cost: f_w + 2 * c * K / 1.018 per round of 512; ahead of the large tile for beta != 0 up to K of
+  //    about 2500.
   //  * a round of 512 small tiles: f_s + c * K.
-  // The constants are pl_gemm_fit's (built-in: c = 0.1207 us, f_s = 6 us, f_w = 5 | 10.6 us, g = 0.07 - 0.09, f = 10 |
-  // 44 - 55 us).  Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD,
+  // The constants are pl_gemm_fit's (built-in: c = 0.1192 us, f_s = 5.1 us, f_w = 3.4 | 9.6 us, g = 0.084 - 0.089, f = 10 |
+  // 44 - 53 us).  Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD,
   // 32-cycle MFMAs) measured 70.7 against 73.4 TFLOP/s.
   const pl_gemm_fit& fit = fit_in_use();
   const int tr = an ? (bnn ? 0 : 1) : (bnn ? 2 : 3);
@@ -935,8 +940,8 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   T* const k_C = splits > 1 ? workspace : C;
   const long k_ldc = splits > 1 ? M : ldc;
   constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
-  // fp64 with direct panels only where the k extent of a workgroup is long
-  const bool stage = sizeof(T) == 8 && ((splits > 1 ? kchunk : K) < 1536 || !dma_fits);
+  // fp64: panels staged through registers only where the row requests cannot address the operand
+  const bool stage = sizeof(T) == 8 && ((splits > 1 ? kchunk : K) < PLK_F64_STAGE_BELOW || !dma_fits);
 #define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK, DIRF)                                                                            \
   hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK, DIRF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
                      A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)

@@ -423,9 +423,9 @@ static void bench_fit(const std::string& db, bool quick) {
     run();
     return sample_until_stable(run).mean * 1e6;
   };
-  auto over_k = [&](bool f64, char ta, char tb, long MN, double beta, double rounds, double* fixed_us, double* us_per_k) {
+  auto over_k = [&](bool f64, char ta, char tb, long MN, double beta, double rounds, double* fixed_us, double* us_per_k, const std::vector<long>* ks = nullptr) {
     std::vector<double> x, y;
-    for (long K : Ks) { x.push_back((double)K); y.push_back(per_launch_us(f64, ta, tb, MN, MN, K, beta, 1) / rounds); }
+    for (long K : (ks ? *ks : Ks)) { x.push_back((double)K); y.push_back(per_launch_us(f64, ta, tb, MN, MN, K, beta, 1) / rounds); }
     fit_line(x, y, fixed_us, us_per_k);
   };
   KernelFit k;
@@ -462,11 +462,14 @@ static void bench_fit(const std::string& db, bool quick) {
   // one 128 x 128 workgroup per compute unit (2048 x 2048: 256 tiles), small tile, no split: time over K
   setenv("PARALIA_GEMM_LARGE_TILE", "0", 1);
   double a = 0, b = 0;
-  // (beta == 0, as the kernels of a split product run: they write their slice and read nothing of C)
-  over_k(true, 'N', 'N', one_round, 0.0, 1.0, &a, &b);
+  // (beta == 0, as the kernels of a split product run: they write their slice and read nothing of C; K up to 4096: the
+  // chunks of a split are short, and from K = 8192 on A and B of these repeated launches no longer fit the memory-side
+  // cache, which a lone workgroup per compute unit feels -- another regime than the one the split decision prices)
+  const std::vector<long> lone_ks = quick ? std::vector<long>{1024, 2048, 4096} : std::vector<long>{512, 1024, 2048, 4096};
+  over_k(true, 'N', 'N', one_round, 0.0, 1.0, &a, &b, &lone_ks);
   f.lone_us_per_k[0] = b;
   const double fixed_k64 = a / b;
-  over_k(false, 'N', 'N', one_round, 0.0, 1.0, &a, &b);
+  over_k(false, 'N', 'N', one_round, 0.0, 1.0, &a, &b, &lone_ks);
   f.lone_us_per_k[1] = b;
   f.lone_fixed_k = std::max(0.0, 0.5 * (fixed_k64 + a / b));
   // fp32, M = N = 8192: 8 rounds of 512 small tiles (beta == 0 and != 0 pooled), 4 rounds of 512 wide tiles (NN), 4 rounds
