@@ -53,6 +53,10 @@
 #ifndef PLK_F64_STAGE_BELOW
 #define PLK_F64_STAGE_BELOW 0
 #endif
+// which MFMA of its stretch a row request of the fp32 256 x 256 tile goes behind (see the V2 loop)
+#ifndef PLK_DMA_BEHIND
+#define PLK_DMA_BEHIND 2
+#endif
 #ifndef PLK_V2
 #define PLK_V2 1
 #endif
@@ -608,7 +612,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         // the requests end up three in a row behind the step's last read, and the four waves of the compute unit send
         // twelve to the one address unit at once.  Spread one at a time, 10 or 11 MFMAs apart: NN 152.3 -> 152.8, TN and
         // TT 151.8 -> 152.7 TFLOP/s at 8192^3 (NT, which is not V2, loses 0.5 that way and keeps the order below).
-        constexpr int PER_STEP_D = (SIDE + KS - 2) / (KS - 1), DMA_BEHIND = 2;
+        constexpr int PER_STEP_D = (SIDE + KS - 2) / (KS - 1), DMA_BEHIND = PLK_DMA_BEHIND;
 #pragma unroll
         for (int ks = 0; ks < KS - 1; ++ks) {
 #pragma unroll
