@@ -34,6 +34,10 @@
 #ifndef PLK_F32_BK
 #define PLK_F32_BK 16
 #endif
+// panel depth of the fp32 128 x 128 tile where k allows it (see launch_gemm)
+#ifndef PLK_F32_DEEP_BK
+#define PLK_F32_DEEP_BK 32
+#endif
 #ifndef PLK_F64_PAIR
 #define PLK_F64_PAIR 0
 #endif
@@ -56,6 +60,10 @@
 // which MFMA of its stretch a row request of the fp32 256 x 256 tile goes behind (see the V2 loop)
 #ifndef PLK_DMA_BEHIND
 #define PLK_DMA_BEHIND 2
+#endif
+// 1: the fp32 128 x 128 tile requests its panels straight into LDS too
+#ifndef PLK_F32_SMALL_DIRECT
+#define PLK_F32_SMALL_DIRECT 1
 #endif
 #ifndef PLK_V2
 #define PLK_V2 1
@@ -118,7 +126,7 @@ template <> struct Traits<float> {
 // [mn][k] layout (K-major operands): rows BK + 2 elements apart.  fp32: lane (idx, kk) of an operand read sits in bank
 // ((BK + 2) * idx + kk) mod 64, all distinct; rows are then only 8-byte aligned, so a 16-byte vector goes to LDS as two
 // 8-byte stores (lds_put).  A 16-byte aligned stride costs two-way conflicts on every operand read.
-template <typename T, bool KMAJOR, int EXT, int BK, bool SWZ = false> struct Lds {
+template <typename T, bool KMAJOR, int EXT, int BK, bool SWZ = false, bool ROW2 = false> struct Lds {
   using Tr = Traits<T>;
   // SWZ (K-major only): rows exactly BK elements apart, no padding, and the 16-byte chunks of row mn stored at chunk
   // position c ^ swz(mn).  That is the layout an LDS-DMA load can write (a wave instruction fills 1 KiB of consecutive
@@ -127,7 +135,10 @@ template <typename T, bool KMAJOR, int EXT, int BK, bool SWZ = false> struct Lds
   static constexpr int NC = BK / Tr::VEC;                         // 16-byte chunks per K-major row
   static constexpr int RPB = 256 / (BK * (int)sizeof(T)) > 0 ? 256 / (BK * (int)sizeof(T)) : 1;  // rows per 256 B (all 64 banks)
   static constexpr __host__ __device__ __forceinline__ int swz(int mn) { return (mn / RPB) % NC; }
-  static constexpr int S_K = (KMAJOR && SWZ) ? BK : BK + 2, S_MN = EXT + Tr::PAD_MN;
+  // ROW2 (MN-major only): rows of 512 bytes kept two by two without padding -- rows 2q and 2q + 1 are the 1 KiB that one
+  // LDS-DMA request fills (dma_row2), pairs 2 * EXT apart.  An operand read of the fp32 MFMA takes k = 2q from lanes
+  // 0 - 31 and k = 2q + 1 from lanes 32 - 63, 8 bytes per lane: each half-wave pass covers 256 contiguous bytes.
+  static constexpr int S_K = (KMAJOR && SWZ) ? BK : BK + 2, S_MN = ROW2 ? EXT : EXT + Tr::PAD_MN;
   static constexpr int SIZE = KMAJOR ? EXT * S_K : BK * S_MN;  // elements, padding included
   static constexpr int NV = EXT * BK / Tr::VEC / NTHREADS;     // 16-byte vectors per thread per panel
   static constexpr bool SPLIT_PUT = KMAJOR && !SWZ && sizeof(T) == 4;  // rows only 8-byte aligned: a vector goes as two halves
@@ -252,13 +263,26 @@ __device__ __forceinline__ void dma_krows(const T* __restrict__ g, long ld, T* x
 #endif
 }
 
-// Where a lane's 16 bytes of a dma_row / dma_krows request sit relative to the request's wave-uniform base, in bytes.
+// Two rows of 512 bytes (128 floats) of an MN-major panel with one request: lanes 0 - 31 fetch row 2 * inst, lanes 32 - 63
+// row 2 * inst + 1, and the 1 KiB lands as those two rows of the unpadded layout (Lds<.., ROW2>).
+template <typename T, int EXT>
+__device__ __forceinline__ void dma_row2(const T* __restrict__ g, long ld, T* xs, int inst, unsigned voff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  static_assert(EXT * sizeof(T) == 512, "dma_row2 moves rows of 512 bytes");
+  const char* base = scalar_base(g + (long)(2 * inst) * ld);
+  __builtin_amdgcn_global_load_lds(reinterpret_cast<const T*>(base + voff), xs + 2 * inst * EXT, 16, 0, 0);
+#endif
+}
+
+// Where a lane's 16 bytes of a dma_row / dma_row2 / dma_krows request sit relative to the request's wave-uniform base, in bytes.
 // The same for every request a wave makes for an operand: its requests are 4 apart and 4 * RPI rows are a whole swizzle
 // period.  K-major: up to 64 / NC - 1 rows of ld elements, which is why the launcher keeps operands whose leading
 // dimension does not fit 32 bits that way on the staged path (PLK_DMA_MAX_LD_BYTES).
-template <typename L, typename T, bool KMAJOR>
+template <typename L, typename T, bool KMAJOR, bool ROW2 = false>
 __device__ __forceinline__ unsigned dma_lane_offset(long ld, int wave, int lane) {
-  if constexpr (KMAJOR) {
+  if constexpr (!KMAJOR && ROW2) {
+    return (unsigned)(lane / 32) * (unsigned)ld * (unsigned)sizeof(T) + (unsigned)(16 * (lane % 32));
+  } else if constexpr (KMAJOR) {
     constexpr int NC = L::NC, RPI = 64 / NC;
     static_assert((4 * RPI / L::RPB) % NC == 0, "the requests of a wave must share their swizzle");
     const int row = wave * RPI + lane / NC;
@@ -314,10 +338,14 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   // through registers (with 64-bit lane addresses in the row requests NN had measured the same either way).
   constexpr bool SWZL = DIR && ((PLK_SWZ >> (sizeof(T) == 4 ? 1 : 0)) & 1) &&
                         ((sizeof(T) == 8 && BM == 128 && BN == 128 && BK == 16) ||
-                         (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0));
+                         (sizeof(T) == 4 && BM == 256 && BN == 256 && BK % 16 == 0) ||
+                         (sizeof(T) == 4 && BM == 128 && BN == 128 && BK % 16 == 0 && PLK_F32_SMALL_DIRECT));
   constexpr bool V2 = PLK_V2 && SWZL && sizeof(T) == 4 && (AK || BKM);
-  using LA = Lds<T, AK, BM, BK, SWZL>;
-  using LB = Lds<T, BKM, BN, BK, SWZL>;
+  // ROW2 (fp32 128 x 128): the 512-byte panel rows of an MN-major operand are requested two per instruction into the
+  // unpadded layout; its K-major operands take the swizzled layout (SWZL) and the permuted k order (V2) of the large tile
+  constexpr bool ROW2 = DIR && PLK_F32_SMALL_DIRECT && sizeof(T) == 4 && BM == 128 && BN == 128;
+  using LA = Lds<T, AK, BM, BK, SWZL, ROW2>;
+  using LB = Lds<T, BKM, BN, BK, SWZL, ROW2>;
   constexpr int BLK = Tr::BLK, WM = BM / 2, WN = BN / 2, NBM = WM / BLK, NBN = WN / BLK;
   if (kchunk > 0) {
     // split K: the workgroups of grid row y multiply k in [y * kchunk, (y + 1) * kchunk) and leave their plain partial
@@ -529,14 +557,15 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
     constexpr bool DIR_T = DIR && ((PLK_DIRECT >> (sizeof(T) == 4 ? 1 : 0)) & 1) != 0;
     // only when both operands qualify: with one operand direct and one staged the wait in front of the barrier also
     // covers the staged operand's newer loads (fp32 256 x 128 NN: 143.8 -> 137.4 TFLOP/s).  SWZL: every operand does.
-    constexpr bool A_DIR = DIR_T && (SWZL || (!AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024));
+    constexpr bool A_DIR = DIR_T && (SWZL || ROW2 || (!AK && !BKM && BM * sizeof(T) == 1024 && BN * sizeof(T) == 1024));
     constexpr bool B_DIR = A_DIR;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const unsigned voff_a0 = dma_lane_offset<LA, T, AK>(lda, wave_u, lane), voff_b0 = dma_lane_offset<LB, T, BKM>(ldb, wave_u, lane);
+    const unsigned voff_a0 = dma_lane_offset<LA, T, AK, ROW2>(lda, wave_u, lane), voff_b0 = dma_lane_offset<LB, T, BKM, ROW2>(ldb, wave_u, lane);
     if constexpr (A_DIR) {
 #pragma unroll
       for (int i = 0; i < NVA; ++i) {
         if constexpr (AK) dma_krows<LA, T>(Ab, lda, smem, wave_u + 4 * i, voff_a0);
+        else if constexpr (ROW2) dma_row2<T, BM>(Ab, lda, smem, wave_u + 4 * i, voff_a0);
         else dma_row<T, BM>(Ab, lda, smem, wave_u + 4 * i, LA::S_MN, voff_a0);
       }
     } else {
@@ -548,6 +577,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
 #pragma unroll
       for (int i = 0; i < NVB; ++i) {
         if constexpr (BKM) dma_krows<LB, T>(Bb, ldb, smem + ASZ, wave_u + 4 * i, voff_b0);
+        else if constexpr (ROW2) dma_row2<T, BN>(Bb, ldb, smem + ASZ, wave_u + 4 * i, voff_b0);
         else dma_row<T, BN>(Bb, ldb, smem + ASZ, wave_u + 4 * i, LB::S_MN, voff_b0);
       }
     } else {
@@ -573,9 +603,11 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
         const int vec = (A_DIR ? 0 : NVA) + slot;  // direct rows: A's first when both are direct
         if (vec < NVA) {
           if constexpr (AK) dma_krows<LA, T>(ga, lda, nxt_a, wave_u + 4 * vec, voff_a);
+          else if constexpr (ROW2) dma_row2<T, BM>(ga, lda, nxt_a, wave_u + 4 * vec, voff_a);
           else dma_row<T, BM>(ga, lda, nxt_a, wave_u + 4 * vec, LA::S_MN, voff_a);
         } else {
           if constexpr (BKM) dma_krows<LB, T>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), voff_b);
+          else if constexpr (ROW2) dma_row2<T, BN>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), voff_b);
           else dma_row<T, BN>(gb, ldb, nxt_b, wave_u + 4 * (vec - NVA), LB::S_MN, voff_b);
         }
         return;
@@ -846,7 +878,9 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
   int best_s = 1;
   const long max_ws = 256L << 20;  // workspace bound: the slices of very long, very thin products stay small anyway
   for (int s = 2; s <= 64; ++s) {
-    const long kc = (((K + s - 1) / s) + 15) / 16 * 16;
+    // whole panels per chunk (fp32: of the 32-deep panels its 128 x 128 tile takes where it can)
+    const long gran = sizeof(T) == 4 ? PLK_F32_DEEP_BK : 16;
+    const long kc = (((K + s - 1) / s) + gran - 1) / gran * gran;
     if (kc < 128) break;
     const long se = (K + kc - 1) / kc;
     if (se < 2) continue;
@@ -945,7 +979,14 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   const long k_ldc = splits > 1 ? M : ldc;
   constexpr int BK_SMALL = sizeof(T) == 4 ? PLK_F32_BK : PLK_F64_BK;
   // fp64: panels staged through registers only where the row requests cannot address the operand
-  const bool stage = sizeof(T) == 8 && ((splits > 1 ? kchunk : K) < PLK_F64_STAGE_BELOW || !dma_fits);
+  // (the fp32 128 x 128 tile: a request covers sixteen rows of a K-major operand, or two of an MN-major one)
+  const bool small_fits = (at ? lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES / 2 : lda * (long)sizeof(T) < (1L << 32) - 1024) &&
+                          (bnn ? ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES / 2 : ldb * (long)sizeof(T) < (1L << 32) - 1024);
+  const bool stage = sizeof(T) == 8 ? ((splits > 1 ? kchunk : K) < PLK_F64_STAGE_BELOW || !dma_fits) : !small_fits;
+  // fp32 128 x 128 with direct panels: 32-deep panels where every workgroup's k extent is a whole number of them (a
+  // K-major row is then a full 128-byte line per request: TN 141.8 -> 148.9, TT 146.8 -> 149.4 TFLOP/s at 8192^3, NN and
+  // NT + 0.5 %; same bits), 16-deep ones otherwise
+  const bool deep = sizeof(T) == 4 && (splits > 1 ? kchunk : K) % PLK_F32_DEEP_BK == 0 && dma_fits;
 #define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK, DIRF)                                                                            \
   hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK, DIRF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
                      A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)
@@ -955,8 +996,9 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
       if (big) { PLK_LAUNCH_T(AKF, BKF, 256, 256, PLK_F32_BIG_BK, true); break; }   \
       if (wide) { PLK_LAUNCH_T(AKF, BKF, 256, 128, PLK_F32_BK, true); break; }      \
     }                                                                               \
-    if constexpr (sizeof(T) == 8) {                                                 \
-      if (stage) { PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, false); break; }      \
+    if (stage) { PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, false); break; }        \
+    if constexpr (sizeof(T) == 4) {                                                 \
+      if (deep) { PLK_LAUNCH_T(AKF, BKF, 128, 128, PLK_F32_DEEP_BK, true); break; } \
     }                                                                               \
     PLK_LAUNCH_T(AKF, BKF, 128, 128, BK_SMALL, true);                               \
   } while (0)

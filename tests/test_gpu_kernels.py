@@ -254,13 +254,36 @@ def test_sgemm_large_tile_exact_on_integers(pkg, L, openblas, ta, tb, dims, off,
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("K,off", [(1536, 0), (1552, 0), (1536, 1), (96, 0), (32, 0)])
+def test_sgemm_small_tile_direct_panels_exact_on_integers(pkg, L, openblas, ta, tb, K, off):
+    """The 128 x 128 fp32 tile pinned: panels requested straight into LDS, 32 deep where K is a multiple of 32 (1536, 96,
+    32), 16 deep otherwise (1552); interior workgroups take the pipelined loop, the ragged edge workgroups of the same
+    launch and operands that are not 16-byte aligned (off = 1) the guarded one over the same LDS layouts.  Small
+    integers: exact in any order, so the result must equal OpenBLAS bit for bit."""
+    M, N = 300, 260
+    rng = np.random.default_rng(21)
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 8, M + 4
+    A = rng.integers(-4, 5, lda * ca + off).astype(np.float32)
+    B = rng.integers(-4, 5, ldb * cb + off).astype(np.float32)
+    C0 = rng.integers(-4, 5, ldc * N + off).astype(np.float32)
+    with large_tile("0"):
+        got = run_gemm(pkg, L, np.float32, ta, tb, M, N, K, 2.0, -1.0, A, lda, B, ldb, C0, ldc, off, off, off)
+    ref = C0.copy()
+    assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 2.0, ptr(A[off:]), lda, ptr(B[off:]), ldb, -1.0, ptr(ref[off:]), ldc) == 0
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
 @pytest.mark.parametrize("beta", [0.5, 0.0])
 @pytest.mark.parametrize("pin", ["1", "2", "0", None])
 def test_sgemm_large_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, pin, beta):
     """Random data at 4096 x 4096 x 8192, where the kernel's cost model picks the large tile by itself (pin None).  Every
     tile is held to OpenBLAS within the fp32 tolerance.  Tiles that multiply k in the same order give the same bits:
-    for NT (no K-major operand) all of them; with a K-major operand the large tile walks each 16-deep group of k in
-    its own order, so there only runs on the same tile are compared."""
+    for NT (no K-major operand) all of them; with a K-major operand the 256 x 256 and the 128 x 128 tile both walk each
+    16-deep group of k in the permuted order of their direct panels and agree, the 256 x 128 tile (NN only, panels
+    staged through registers) keeps the plain order."""
     M, N, K = 4096, 4096, 8192
     ra, ca = (M, K) if ta == "N" else (K, M)
     rb, cb = (K, N) if tb == "N" else (N, K)
@@ -271,7 +294,7 @@ def test_sgemm_large_tile_vs_openblas(pkg, L, orc, openblas, ta, tb, pin, beta):
     assert openblas.orc_openblas_sgemm(ta.encode(), tb.encode(), M, N, K, 1.5, ptr(A), ra, ptr(B), rb, beta, ptr(ref), M) == 0
     d = 1.5 * orc.orc_fro_norm_f32(ptr(A), ra, ca, ra) * orc.orc_fro_norm_f32(ptr(B), rb, cb, rb) + beta * orc.orc_fro_norm_f32(ptr(C0), M, N, M)
     assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
-    same_order = "all" if (ta, tb) == ("N", "T") else ("large" if pin in ("1", None) else "small")
+    same_order = "all" if (ta, tb) == ("N", "T") else ("plain" if (pin == "2" and (ta, tb) == ("N", "N")) else "permuted")
     key = (ta, tb, beta, same_order)
     if key in _LARGE_TILE_BITS:
         assert np.array_equal(got, _LARGE_TILE_BITS[key])
