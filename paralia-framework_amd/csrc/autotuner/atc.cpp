@@ -380,6 +380,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       // building a plan).  The second runs the full order search for the (at most three) T whose penalised probe is
       // within 10 % of the best, best probe first, and skips a T whose floor is above a result already in hand.
       struct Cand { long T; double probe_t, floor_t; };
+      constexpr long PROBE_ABOVE_SUBKERNELS = 48;
       const char* verbose_env = getenv("PARALIA_VERBOSE");
       const bool chatty = verbose_env && atoi(verbose_env) > 1;
       const char* search_env = getenv("PARALIA_PLAN_SEARCH");
@@ -447,7 +448,10 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         if (e.floor_t > best_probe_score && !exhaustive) break;   // and so is every floor behind it
         paralia::PipelineResult r;
         try {
-          paralia::pick_gemm_order(e.gp, paralia_stage_times(this, cand), &r, /*probe=*/true);
+          // a grid of a few dozen subkernels gets the full order search at once: its plans cost microseconds, and the
+          // handful of orders of a probe misses the block orders that win there (sgemm 4096^3 from the host: T = 1536
+          // probed at 3.24 ms, searched at 3.08, and left out of the finalists)
+          paralia::pick_gemm_order(e.gp, paralia_stage_times(this, cand), &r, /*probe=*/e.gp.subkernels() > PROBE_ABOVE_SUBKERNELS);
         } catch (const std::runtime_error&) { continue; }
         cands.push_back({cand, r.t_total * penalty(cand), e.floor_t});
         best_probe = std::min(best_probe, r.t_total);
@@ -474,9 +478,18 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       for (const Cand& c : cands)
         if (!(c.probe_t > 1.1 * best_probe || c.probe_t > cut)) finalists.push_back(&c);
       std::stable_sort(finalists.begin(), finalists.end(), [](const Cand* x, const Cand* y) { return x->probe_t < y->probe_t; });
+      // A tile size that cuts the problem into thousands of subkernels costs its full search 10 - 20 ms and the call as
+      // many launches and copies; it goes on only when its probe is 2 % ahead of the best finalist with fewer (the
+      // full search moves a probe by 1 - 2 %, so anything closer is a tie the lighter plan should win)
+      constexpr long HEAVY_SUBKERNELS = 2048;
+      auto subkernels_of = [&](long cand) { return gemm_problem_of(problem, cand, exec_queues).subkernels(); };
+      double best_light_probe = DBL_MAX;
+      for (const Cand* c : finalists)
+        if (subkernels_of(c->T) <= HEAVY_SUBKERNELS) best_light_probe = std::min(best_light_probe, c->probe_t);
       for (const Cand* c : finalists) {
         if (c->floor_t > best_t && !exhaustive) continue;
         const long cand = c->T;
+        if (!exhaustive && best_light_probe < DBL_MAX && subkernels_of(cand) > HEAVY_SUBKERNELS && c->probe_t > 0.98 * best_light_probe) continue;
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         paralia::PipelineResult r;
         int oid = -1;

@@ -493,10 +493,16 @@ static void bench_fit(const std::string& db, bool quick) {
     f.f32_large_gain[t] = 2.0 * f.f32_small_us_per_k / (0.5 * (b0 + b1)) - 1.0;
     f.f32_large_fixed_us[t][0] = std::max(0.0, a0);
     f.f32_large_fixed_us[t][1] = std::max(0.0, a1);
-    // a merged chain saves one such fixed cost per launch it saves, less the gap the launches would have had anyway
-    k.merge_saving_us_f32[t] = std::max(0.0, f.f32_large_fixed_us[t][1] - f.splitk_launch_us);
   }
   unsetenv("PARALIA_GEMM_LARGE_TILE");
+  // what joining the k-steps of a C tile into one launch saves per launch saved, as the scheduler issues them (beta = 1,
+  // two streams, the launcher's own tile choice): four 4096^3 launches against one 4096 x 4096 x 16384 launch.  Per
+  // 4096 x 4096 of C, i.e. per round of 256 large or two rounds of 512 small tiles; the planner scales it by the area.
+  for (int t = 0; t < 4; ++t) {
+    const double separate = per_launch_us(false, tas[t], tbs[t], 4096, 4096, 4096, 1.0, 2);
+    const double joined = per_launch_us(false, tas[t], tbs[t], 4096, 4096, 16384, 1.0, 2);
+    k.merge_saving_us_f32[t] = std::max(0.0, (4.0 * separate - joined) / 3.0);
+  }
   k.merge_saving_us_f64 = f.splitk_launch_us;
   // a slab of a thin start, two launches sharing the device: 2048 x 2048 x 1024 against half of 2048^3
   {
