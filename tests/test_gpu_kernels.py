@@ -155,6 +155,33 @@ def test_dgemm_tile_k_major_operand_with_a_row_stride_of_half_a_gigabyte(pkg, L,
     assert orc.orc_normwise_err_f64(ptr(got), ptr(ref), M, N, M, M, d) < TOL64
 
 
+@pytest.mark.parametrize("extra,K", [(0, 96), (0, 80), (4, 96)])
+def test_sgemm_small_tile_k_major_operand_with_a_row_stride_of_a_quarter_gigabyte(pkg, L, orc, extra, K):
+    """The 128 x 128 fp32 tile pinned, op(A) K-major with rows exactly 2^28 bytes apart -- the largest stride its row
+    requests span (sixteen rows per request) -- and just beyond, where the launcher keeps the instantiation that stages
+    through registers.  K = 96 takes the 32-deep panels (eight rows per request), K = 80 the 16-deep ones (sixteen).
+    32 GiB of device addresses, 128 rows of K values filled."""
+    M, N, lda = 128, 256, (1 << 26) + extra
+    dA = Buf(pkg, (M - 1) * lda + K, np.float32, 0)
+    dense = np.empty((M, K), dtype=np.float32)
+    for r in range(M):
+        pkg.check(L.PARALiA_vec_init_f32(dA.at(r * lda), K, 300 + r, 0), "vec init f32")
+        dense[r] = rand_f32(K, 300 + r)
+    B, C0 = rand_f32(K * N, 5), rand_f32(M * N, 6)
+    dB, dC = Buf(pkg, B.size, np.float32, 0).set(B), Buf(pkg, C0.size, np.float32, 0).set(C0)
+    print("gemm f32 small tile, K-major A, lda", lda, flush=True)
+    with large_tile("0"):
+        pkg.check(L.pl_sgemm_tile(b"T", b"N", M, N, K, 1.0, dA.ptr, lda, dB.ptr, K, 1.0, dC.ptr, M, None), "gemm tile")
+    sync(pkg)
+    got = dC.get()
+    dA.free()
+    ref = C0.copy()
+    flat = dense.ravel()
+    orc.orc_sgemm_bruteforce(b"T", b"N", M, N, K, 1.0, ptr(flat), K, ptr(B), K, 1.0, ptr(ref), M)
+    d = float(np.linalg.norm(flat.astype(np.float64)) * np.linalg.norm(B.astype(np.float64)) + np.linalg.norm(C0.astype(np.float64)))
+    assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
+
+
 def test_sgemm_large_tile_gives_way_to_a_row_stride_beyond_its_lane_offsets(pkg, L, orc):
     """The 256 x 256 fp32 tile pinned, op(A) K-major with rows more than 2^29 bytes apart: the launcher takes the
     small tile (and its grid), whatever the pin says."""
