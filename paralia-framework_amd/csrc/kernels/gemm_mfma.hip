@@ -847,15 +847,15 @@ __global__ void splitk_reduce_kernel(int M, int N, int splits, T alpha, const T*
 // The launcher's fitted constants (pl_gemm_fit in the public header): built-in values measured on an MI355X, replaced
 // by what the deploy database holds once the autotuner has loaded it.
 inline void fit_defaults(pl_gemm_fit* f) {
-  f->lone_us_per_k[0] = 0.115; f->lone_us_per_k[1] = 0.065;
-  f->lone_fixed_k = 80.0;
-  f->splitk_launch_us = 3.0;
-  f->pass_bytes_per_us = 6.2e6;
-  f->f32_small_us_per_k = 0.1192;
-  f->f32_small_fixed_us = 5.1;
-  f->f32_wide_gain = 1.018;
-  f->f32_wide_fixed_us[0] = 3.4; f->f32_wide_fixed_us[1] = 9.6;
-  const double g[4] = {0.085, 0.089, 0.084, 0.085}, f0[4] = {10.0, 10.4, 10.4, 10.8}, f1[4] = {45.0, 43.5, 52.0, 53.0};
+  f->lone_us_per_k[0] = 0.114; f->lone_us_per_k[1] = 0.056;
+  f->lone_fixed_k = 94.0;
+  f->splitk_launch_us = 3.2;
+  f->pass_bytes_per_us = 6.15e6;
+  f->f32_small_us_per_k = 0.1099;
+  f->f32_small_fixed_us = 7.4;
+  f->f32_wide_gain = 0.949;
+  f->f32_wide_fixed_us[0] = 4.9; f->f32_wide_fixed_us[1] = 10.6;
+  const double g[4] = {0.012, 0.011, 0.010, 0.010}, f0[4] = {11.4, 10.7, 11.1, 11.7}, f1[4] = {45.5, 44.5, 53.0, 54.4};
   for (int t = 0; t < 4; ++t) { f->f32_large_gain[t] = g[t]; f->f32_large_fixed_us[t][0] = f0[t]; f->f32_large_fixed_us[t][1] = f1[t]; }
 }
 inline pl_gemm_fit& fit_in_use() {
@@ -903,17 +903,19 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
   if (c.splits > 1 && (long)c.splits * M * N * (long)sizeof(T) > workspace_bytes) c.splits = 1, c.kchunk = 0;
   // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
-  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 8 - 9 % faster per k (all panels global -> LDS
-  //    directly, a 16-byte operand read per block and four k-steps), but a CU holds one such workgroup at a time, so
+  //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 1 % faster per k (a 16-byte operand read per
+  //    block and four k-steps, half the row requests per MFMA), but a CU holds one such workgroup at a time, so
   //    nothing overlaps its prologue and its epilogue: a round of 256 large tiles takes f + 2 * c * K / (1 + g), c the
   //    per-k time of a round of 512 small tiles, with g and f (beta == 0 / beta != 0) fitted per transpose to
-  //    single-stream runs at M = N = 8192, K = 512 .. 8192 (152.6 - 152.8 TFLOP/s at K = 8192, beta = 0, for all four).
-  //  * 256 x 128 x 16 ("wide", NN only): still two workgroups per CU, 2 % faster per k than the small tile with a
-  //    small fixed cost: f_w + 2 * c * K / 1.018 per round of 512; ahead of the large tile for beta != 0 up to K of
-  //    about 2500.
+  //    single-stream runs at M = N = 8192, K = 512 .. 8192 (152.6 - 153.2 TFLOP/s at K = 8192, beta = 0, for all four;
+  //    the small tile 150 - 151).  With beta == 0 its fixed cost per unit of work is the lower one and it wins from
+  //    K of about 256 on; with beta != 0 (45 - 54 us per round) only beyond K of about 12000.
+  //  * 256 x 128 x 16 ("wide", NN only, panels staged through registers): still two workgroups per CU, 5 % slower per
+  //    k than the small tile since that one loads its panels directly: f_w + 2 * c * K / 0.949 per round of 512; its
+  //    lower fixed cost wins for K of a few hundred.
   //  * a round of 512 small tiles: f_s + c * K.
-  // The constants are pl_gemm_fit's (built-in: c = 0.1192 us, f_s = 5.1 us, f_w = 3.4 | 9.6 us, g = 0.084 - 0.089, f = 10 |
-  // 44 - 53 us).  Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD,
+  // The constants are pl_gemm_fit's (built-in: c = 0.1099 us, f_s = 7.4 us, f_w = 4.9 | 10.6 us, g = 0.010 - 0.012, f = 11 |
+  // 45 - 54 us).  Split K keeps the small tile.  fp64 stays at 128 x 128: a 256 x 128 tile (one wave per SIMD,
   // 32-cycle MFMAs) measured 70.7 against 73.4 TFLOP/s.
   const pl_gemm_fit& fit = fit_in_use();
   const int tr = an ? (bnn ? 0 : 1) : (bnn ? 2 : 3);
