@@ -93,7 +93,7 @@ struct KernelFit {
   double merge_saving_us_f64 = 3.0;    // a launch saved by merging K chains, fp64: the gap between two launches of a stream
   // fp32, per round of 256 large tiles and per transpose (NN, NT, TN, TT): the fixed cost of a launch that accumulates,
   // less the launch gap
-  double merge_saving_us_f32[4] = {21.0, 20.0, 23.0, 26.0};
+  double merge_saving_us_f32[4] = {8.0, 11.0, 6.0, 7.0};
   double lone_share = 0.07;            // share of a streamed call's launches that run without a partner on the device
   double geadd_bytes_per_s = 5e12;     // rate of the lazy-reduce kernel over its 3 T^2 elements
   double slab_fixed_us = 2.0;          // extra time of a thin-start slab launch 1024 deep (deeper: the same, shallower: in inverse proportion)

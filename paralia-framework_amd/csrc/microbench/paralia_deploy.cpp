@@ -496,12 +496,25 @@ static void bench_fit(const std::string& db, bool quick) {
   }
   unsetenv("PARALIA_GEMM_LARGE_TILE");
   // what joining the k-steps of a C tile into one launch saves per launch saved, as the scheduler issues them (beta = 1,
-  // two streams, the launcher's own tile choice): four 4096^3 launches against one 4096 x 4096 x 16384 launch.  Per
-  // 4096 x 4096 of C, i.e. per round of 256 large or two rounds of 512 small tiles; the planner scales it by the area.
+  // two streams, the launcher's own tile choice): 32 launches of 4096^3 against 8 of 4096 x 4096 x 16384, the same
+  // flops, 24 launches fewer.  The saving is 2 % of either time, so the two are timed in turn and the median of the
+  // differences is taken.  Per 4096 x 4096 of C, i.e. per round of 256 large or two rounds of 512 small tiles; the
+  // planner scales it by the area.
   for (int t = 0; t < 4; ++t) {
-    const double separate = per_launch_us(false, tas[t], tbs[t], 4096, 4096, 4096, 1.0, 2);
-    const double joined = per_launch_us(false, tas[t], tbs[t], 4096, 4096, 16384, 1.0, 2);
-    k.merge_saving_us_f32[t] = std::max(0.0, (4.0 * separate - joined) / 3.0);
+    auto timed = [&](long K, int n) {
+      const long lda = tas[t] == 'N' ? 4096 : K, ldb = tbs[t] == 'N' ? K : 4096;
+      const double t0 = csecond();
+      for (int i = 0; i < n; ++i)
+        must(pl_sgemm_tile(tas[t], tbs[t], 4096, 4096, K, 1e-3f, (const float*)A, lda, (const float*)B, ldb, 1.0f,
+                           (float*)((char*)C + (size_t)(i % 2) * 4096 * 4096 * 4), 4096, st[i % 2]), "gemm");
+      for (auto& q : st) must(pl_stream_sync(q), "sync");
+      return csecond() - t0;
+    };
+    timed(4096, 8); timed(16384, 2);
+    std::vector<double> saved;
+    for (int rep = 0; rep < (quick ? 5 : 9); ++rep) saved.push_back((timed(4096, 32) - timed(16384, 8)) / 24.0 * 1e6);
+    std::sort(saved.begin(), saved.end());
+    k.merge_saving_us_f32[t] = std::max(0.0, saved[saved.size() / 2]);
   }
   k.merge_saving_us_f64 = f.splitk_launch_us;
   // a slab of a thin start, two launches sharing the device: 2048 x 2048 x 1024 against half of 2048^3

@@ -228,8 +228,11 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
     for k in kf:
         if "gain" in k:
             assert abs(kf[k] - kf_shipped[k]) <= 0.03, (k, kf[k], kf_shipped[k])
-        elif "fixed_us" in k or k.startswith("merge_saving_us_f32"):
+        elif "fixed_us" in k:
             assert abs(kf[k] - kf_shipped[k]) <= max(4.0, 0.25 * kf_shipped[k]), (k, kf[k], kf_shipped[k])
+        elif k.startswith("merge_saving_us_f32"):
+            # 2 % of the difference of two 30 ms timings (the median of five): a few microseconds either way
+            assert 0.0 <= kf[k] <= 30.0 and abs(kf[k] - kf_shipped[k]) <= 8.0, (k, kf[k], kf_shipped[k])
     assert 0.5 * kf_shipped["lone_fixed_k"] < kf["lone_fixed_k"] < 2.0 * kf_shipped["lone_fixed_k"]
     assert 1.0 < kf["splitk_launch_us"] < 10.0 and 0 <= kf["slab_fixed_us"] < 6.0
     for k in ("pass_bytes_per_us", "geadd_bytes_per_s"):
