@@ -351,4 +351,53 @@ template <typename T> inline T* host_copy(T* src, long long n, short loc) {
   return out;
 }
 
+
+/// The timing protocol the runners share (PARALia/dgemm_runner.cpp:165-215 and its siblings): optionally one timed
+/// first call, `warmups` untimed calls, then `iterations` calls timed one by one, each handed to log_row(seconds,
+/// returned control values).  Where there is a first call the minimum starts from its time, as the reference's does.
+struct ProtocolTimes {
+  double first = -1, avg = 0, min = 1e9, max = 0;
+  ATC_p info = NULL;
+};
+template <typename Call, typename AfterFirst, typename Log>
+inline ProtocolTimes run_protocol(Call&& call, bool timed_first, int warmups, int iterations, AfterFirst&& after_first, Log&& log_row) {
+  ProtocolTimes t;
+  if (timed_first) {
+    const double t0 = csecond();
+    t.info = call();
+    CoCoSyncCheckErr();
+    t.first = t.min = csecond() - t0;
+    after_first(t.info);
+  }
+  for (int it = 0; it < warmups; ++it) t.info = call();
+  CoCoSyncCheckErr();
+  for (int it = 0; it < iterations; ++it) {
+    const double t0 = csecond();
+    t.info = call();
+    CoCoSyncCheckErr();
+    const double dt = csecond() - t0;
+    log_row(dt, t.info);
+    if (dt < t.min) t.min = dt;
+    if (dt > t.max) t.max = dt;
+    t.avg += dt;
+  }
+  t.avg /= iterations;
+  return t;
+}
+
+/// The block every runner ends with: first / avg / min / max in ms with Gflops/s (and GB/s of `bytes` when bytes > 0),
+/// and the predicted time with `selected` behind it when there is one.
+inline void report_protocol(const ProtocolTimes& t, double flops, double bytes, const char* selected) {
+  auto line = [&](const char* name, double seconds) {
+    if (bytes > 0) fprintf(stderr, "\t%s = %lf ms ( %lf Gflops/s, %lf GB/s )\n", name, seconds * 1000, Gval_per_s(flops, seconds), bytes / seconds / 1e9);
+    else fprintf(stderr, "\t%s = %lf ms ( %lf Gflops/s )\n", name, seconds * 1000, Gval_per_s(flops, seconds));
+  };
+  fprintf(stderr, "CoCopeLia (%s):\n", t.info->print_csv());
+  if (t.first >= 0) line("first_it_t", t.first);
+  line("avg_t", t.avg);
+  line("min_t", t.min);
+  line("max_t", t.max);
+  if (selected) fprintf(stderr, "\tpredicted_t = %lf ms [%s]\n", t.info->pred_t * 1000, selected);
+}
+
 #endif

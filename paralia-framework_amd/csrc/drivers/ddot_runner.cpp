@@ -10,7 +10,7 @@ int main(const int argc, const char* argv[]) {
     double alpha;
     long int N, incx, incy;
     short x_loc, y_loc, x_out_loc, y_out_loc;
-    ATC_p predef_control_values = NULL, return_values = NULL;
+    ATC_p predef_control_values = NULL;
     ParseInputLvl1(argc, argv, &predef_control_values, &alpha, &N, &incx, &incy, &x_loc, &y_loc, &x_out_loc, &y_out_loc);
     char filename[1024];
     if (predef_control_values != NULL) {
@@ -35,7 +35,7 @@ int main(const int argc, const char* argv[]) {
     const char* skip = getenv("PARALIA_SKIP_VALIDATION");
     if (!(skip && atoi(skip))) {
       OpenBlas ob;
-      return_values = call();
+      call();
       CoCoSyncCheckErr();
       if (ob.open()) {
         double* hx = host_copy(x, N * ax, x_loc);
@@ -67,25 +67,11 @@ int main(const int argc, const char* argv[]) {
         free(hx); free(hy);
       }
     }
-    for (int it = 0; it < 10; it++) return_values = call();
-    CoCoSyncCheckErr();
-    double min_t = 1e9, max_t = 0, avg_t = 0;
-    const short bench_it = 10;
-    for (int it = 0; it < bench_it; it++) {
-      double t = csecond();
-      return_values = call();
-      CoCoSyncCheckErr();
-      t = csecond() - t;
-      StoreLogLvl1(filename, return_values, alpha, N, incx, incy, x_loc, y_loc, x_out_loc, y_out_loc, t, return_values->pred_t, return_values->pred_J);
-      if (t < min_t) min_t = t;
-      if (t > max_t) max_t = t;
-      avg_t += t;
-    }
-    avg_t /= bench_it;
-    fprintf(stderr, "CoCopeLia (%s):\n\tavg_t = %lf ms ( %lf Gflops/s, %lf GB/s )\n\tmin_t = %lf ms ( %lf Gflops/s, %lf GB/s )\n\tmax_t = %lf ms "
-            "( %lf Gflops/s, %lf GB/s )\n", return_values->print_csv(), avg_t * 1000, Gval_per_s(dot_flops(N), avg_t), 16.0 * N / avg_t / 1e9,
-            min_t * 1000, Gval_per_s(dot_flops(N), min_t), 16.0 * N / min_t / 1e9, max_t * 1000, Gval_per_s(dot_flops(N), max_t),
-            16.0 * N / max_t / 1e9);
+    // 10 warm-ups, 10 timed and logged iterations; GB/s of the algorithmic traffic (x and y read once)
+    const ProtocolTimes times = run_protocol(
+        call, false, 10, 10, [](ATC_p) {},
+        [&](double seconds, ATC_p info) { StoreLogLvl1(filename, info, alpha, N, incx, incy, x_loc, y_loc, x_out_loc, y_out_loc, seconds, info->pred_t, info->pred_J); });
+    report_protocol(times, (double)dot_flops(N), 16.0 * N, NULL);
     for (int i = 0; i < LOC_NUM; i++) PARALiADevCacheFree(deidxize(i));
     CoCoFree(x, x_loc);
     CoCoFree(y, y_loc);

@@ -101,37 +101,18 @@ int main(const int argc, const char* argv[]) {
       free(y_start); free(y_out);
     }
 
-    cpu_timer = csecond();
-    return_values = call();
-    CoCoSyncCheckErr();
-    cpu_timer = csecond() - cpu_timer;
-    const double first_over_t = cpu_timer;
-
-    short warmup_bench_it = 100, bench_it = 100;
-    if (M >= 20000 && N >= 20000) warmup_bench_it = bench_it = 20;
-    for (int it = 0; it < warmup_bench_it; it++) return_values = call();
-    CoCoSyncCheckErr();
-
-    double min_t = first_over_t, max_t = 0, avg_t = 0;
-    for (int it = 0; it < bench_it; it++) {
-      cpu_timer = csecond();
-      return_values = call();
-      CoCoSyncCheckErr();
-      cpu_timer = csecond() - cpu_timer;
-      StoreLogLvl2(filename, return_values, TransA, alpha, beta, M, N, incx, incy, A_loc, x_loc, y_loc, y_out_loc, cpu_timer,
-                   return_values->pred_t, return_values->pred_J);
-      if (cpu_timer < min_t) min_t = cpu_timer;
-      if (cpu_timer > max_t) max_t = cpu_timer;
-      avg_t += cpu_timer;
-    }
-    avg_t /= bench_it;
-    const double bytes = 8.0 * M * N;
-    fprintf(stderr, "CoCopeLia (%s):\n\tfirst_it_t = %lf ms ( %lf Gflops/s, %lf GB/s )\n\tavg_t = %lf ms ( %lf Gflops/s, %lf GB/s )\n\tmin_t = %lf ms "
-            "( %lf Gflops/s, %lf GB/s )\n\tmax_t = %lf ms ( %lf Gflops/s, %lf GB/s )\n\tpredicted_t = %lf ms [T selected by %s]\n",
-            return_values->print_csv(), first_over_t * 1000, Gval_per_s(gemv_flops(M, N), first_over_t), bytes / first_over_t / 1e9,
-            avg_t * 1000, Gval_per_s(gemv_flops(M, N), avg_t), bytes / avg_t / 1e9, min_t * 1000, Gval_per_s(gemv_flops(M, N), min_t),
-            bytes / min_t / 1e9, max_t * 1000, Gval_per_s(gemv_flops(M, N), max_t), bytes / max_t / 1e9, return_values->pred_t * 1000,
-            return_values->T_selected_by);
+    // a timed first call, 100 warm-ups and 100 timed and logged iterations (20 / 20 for the largest problems); rates in
+    // Gflops/s and in GB/s of the matrix bytes the routine must read
+    const int rounds = (M >= 20000 && N >= 20000) ? 20 : 100;
+    const ProtocolTimes times = run_protocol(
+        call, true, rounds, rounds, [](ATC_p) {},
+        [&](double seconds, ATC_p info) {
+          StoreLogLvl2(filename, info, TransA, alpha, beta, M, N, incx, incy, A_loc, x_loc, y_loc, y_out_loc, seconds, info->pred_t, info->pred_J);
+        });
+    return_values = times.info;
+    char selected[128];
+    snprintf(selected, sizeof selected, "T selected by %s", return_values->T_selected_by);
+    report_protocol(times, (double)gemv_flops(M, N), 8.0 * M * N, selected);
 
     for (int i = 0; i < LOC_NUM; i++) PARALiADevCacheFree(deidxize(i));
     CoCoSyncCheckErr();

@@ -138,37 +138,19 @@ template <typename T> int run_gemm_runner(const int argc, const char* argv[]) {
       free(C_start); free(C_out); free(C_out1);
     }
 
-    cpu_timer = csecond();
-    return_values = call();
-    CoCoSyncCheckErr();
-    cpu_timer = csecond() - cpu_timer;
-    const double first_over_t = cpu_timer;
-    if (checklog) CheckLogLvl3(filename, return_values, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc);
-
-    short warmup_bench_it = 10;
-    if (M >= 20000 && N >= 20000 && K >= 20000) warmup_bench_it = 2;
-    for (int it = 0; it < warmup_bench_it; it++) return_values = call();
-    CoCoSyncCheckErr();
-
-    double min_t = first_over_t, max_t = 0, avg_t = 0;
-    const short bench_it = 10;
-    for (int it = 0; it < bench_it; it++) {
-      cpu_timer = csecond();
-      return_values = call();
-      CoCoSyncCheckErr();
-      cpu_timer = csecond() - cpu_timer;
-      StoreLogLvl3(filename, return_values, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc, cpu_timer,
-                   return_values->pred_t, return_values->pred_J);
-      if (cpu_timer < min_t) min_t = cpu_timer;
-      if (cpu_timer > max_t) max_t = cpu_timer;
-      avg_t += cpu_timer;
-    }
-    avg_t /= bench_it;
-    fprintf(stderr, "CoCopeLia (%s):\n\tfirst_it_t = %lf ms ( %lf Gflops/s )\n\tavg_t = %lf ms ( %lf Gflops/s )\n\tmin_t = %lf ms ( %lf "
-            "Gflops/s )\n\tmax_t = %lf ms ( %lf Gflops/s )\n\tpredicted_t = %lf ms [T selected by %s, order %d]\n",
-            return_values->print_csv(), first_over_t * 1000, Gval_per_s(gemm_flops(M, N, K), first_over_t), avg_t * 1000,
-            Gval_per_s(gemm_flops(M, N, K), avg_t), min_t * 1000, Gval_per_s(gemm_flops(M, N, K), min_t), max_t * 1000,
-            Gval_per_s(gemm_flops(M, N, K), max_t), return_values->pred_t * 1000, return_values->T_selected_by, return_values->order_id);
+    // the protocol of the reference's runner: a timed first call, 10 warm-ups (2 for the largest problems), 10 timed
+    // and logged iterations
+    const int warmups = (M >= 20000 && N >= 20000 && K >= 20000) ? 2 : 10;
+    const ProtocolTimes times = run_protocol(
+        call, true, warmups, 10,
+        [&](ATC_p first) { if (checklog) CheckLogLvl3(filename, first, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc); },
+        [&](double seconds, ATC_p info) {
+          StoreLogLvl3(filename, info, TransA, TransB, alpha, beta, M, N, K, A_loc, B_loc, C_loc, C_out_loc, seconds, info->pred_t, info->pred_J);
+        });
+    return_values = times.info;
+    char selected[128];
+    snprintf(selected, sizeof selected, "T selected by %s, order %d", return_values->T_selected_by, return_values->order_id);
+    report_protocol(times, (double)gemm_flops(M, N, K), 0.0, selected);
 
     for (int i = 0; i < LOC_NUM; i++) PARALiADevCacheFree(deidxize(i));
     CoCoSyncCheckErr();
