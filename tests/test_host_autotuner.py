@@ -394,7 +394,7 @@ def test_pruned_search_picks_what_the_exhaustive_search_picks(L, pkg, monkeypatc
 
 
 def test_planner_time_of_a_first_call(L, pkg, monkeypatch):
-    """What a new problem's first call spends in the planner (best of five, database already read): the headline shape
+    """What a new problem's first call spends in the planner (best of six or more, database already read): the headline shape
     within 5 ms, the largest benchmark shapes (32768^3, fp64 and fp32) within 20 ms."""
     import time
     monkeypatch.delenv("PARALIA_PLAN_SEARCH", raising=False)
@@ -404,10 +404,12 @@ def test_planner_time_of_a_first_call(L, pkg, monkeypatch):
                                                  (b"Dgemm", 32768, 32768, 32768, b"NN", (-1, -1, -1), 1, 20.0),
                                                  (b"Sgemm", 32768, 32768, 32768, b"NT", (-1, -1, 0), 0, 20.0)):
         best = 1e9
-        for _ in range(6):
+        for attempt in range(30):   # the best of a few runs; a busy machine gets more of them before the test gives up
             t0 = time.perf_counter()
             assert L.PARALiA_autotune(db, func, M, N, K, tr[0:1], tr[1:2], loc3(*locs), bz, -1, 0, C.byref(info)) == 0
             best = min(best, (time.perf_counter() - t0) * 1e3)
+            if attempt >= 5 and best <= 0.8 * bound_ms:
+                break
         print("  planner %s %d x %d x %d: %.2f ms (T = %d, order %d)" % (func.decode(), M, N, K, best, info.T, info.order_id), flush=True)
         assert best <= bound_ms, (func, M, N, K, best)
 
