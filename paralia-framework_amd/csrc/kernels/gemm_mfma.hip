@@ -8,13 +8,15 @@
 //     workgroups per CU); fp32 also has 256 x 128 (two workgroups per CU) and 256 x 256 (each wave owns 128 x 128
 //     with 256 accumulator registers, one workgroup per CU) for problems with enough such tiles to fill the CUs;
 //   * fp64 uses v_mfma_f64_16x16x4_f64 (4 x 4 blocks per wave), fp32 uses v_mfma_f32_32x32x2_f32 (2 x 2 or 4 x 4);
-//   * A and B k-panels (16 elements deep, 32 for the large tile) sit in LDS, double-buffered, one barrier per k-panel.
-//     They get there through registers (global loads two panels ahead, LDS stores one ahead, both spread between the
-//     MFMAs) or, where every panel of the tile can, straight from global memory (global_load_lds_dwordx4, one panel
-//     ahead): MN-major panels whose rows are exactly 1 KiB (fp64 128 x 128, fp32 256 x 256), K-major panels of those
-//     tiles in a swizzled unpadded layout.  Direct: fp32 256 x 256 (every transpose), fp64 NT, TN, TT; staged: the
-//     fp64 NN tile (no difference measured), the smaller fp32 tiles, every workgroup with a short k;
-//   * LDS rows are padded so the MFMA operand reads of the four 16-lane groups fall in disjoint banks;
+//   * A and B k-panels (16 elements deep; 32 for the fp32 tiles with direct panels) sit in LDS, double-buffered, one
+//     barrier per k-panel.  They get there straight from global memory (global_load_lds_dwordx4, one panel ahead, each
+//     request addressed by a scalar base and a 32-bit lane offset): MN-major panel rows of 1 KiB one per request
+//     (fp64 128 x 128, fp32 256 x 256), of 512 bytes two per request (fp32 128 x 128), K-major panels in a swizzled
+//     unpadded layout, eight or sixteen rows per request.  Direct: fp64 128 x 128 and fp32 128 x 128 and 256 x 256, every
+//     transpose.  Through registers (global loads two panels ahead, LDS stores one ahead, both spread between the
+//     MFMAs): the fp32 256 x 128 tile, and any operand whose leading dimension the lane offsets cannot span;
+//   * LDS rows are padded (or, where a request fills them, swizzled or read in half-wave passes) so that the MFMA
+//     operand reads do not collide in the banks;
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
 //     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
 //   * workgroup ids are re-mapped so the eight XCDs each own a compact block of C tiles (private L2 per XCD),
