@@ -204,6 +204,36 @@ def test_sgemm_large_tile_gives_way_to_a_row_stride_beyond_its_lane_offsets(pkg,
     assert orc.orc_normwise_err_f32(ptr(got), ptr(ref), M, N, M, M, d) < TOL32
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_gemm_tile_random_shapes_exact_on_integers(pkg, L, orc, seed):
+    """Random shapes, transposes, leading dimensions, operand offsets and scalars through the tile kernels of both types,
+    with whatever macro tile the launcher picks or a pinned one: k extents that are multiples of 32, of 16 only, or of
+    neither, so that the 32-deep and 16-deep direct panels and the guarded loop all come up, next to ragged edge
+    workgroups in the same launch.  Small integers, so the brute-force oracle must be matched bit for bit."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = np.float64 if seed % 2 == 0 else np.float32
+    ta, tb = "NT"[rng.integers(2)], "NT"[rng.integers(2)]
+    M, N = int(rng.integers(1, 420)), int(rng.integers(1, 420))
+    K = int([32 * rng.integers(1, 40), 16 * (2 * rng.integers(1, 30) + 1), rng.integers(1, 700)][rng.integers(3)])
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    aligned = bool(rng.integers(2))
+    pad = (lambda: 4 * int(rng.integers(0, 4))) if aligned else (lambda: int(rng.integers(0, 7)))
+    lda, ldb, ldc = ra + pad(), rb + pad(), M + pad()
+    off = 0 if aligned else int(rng.integers(0, 2))
+    A = rng.integers(-4, 5, lda * ca + off).astype(dtype)
+    B = rng.integers(-4, 5, ldb * cb + off).astype(dtype)
+    C0 = rng.integers(-4, 5, ldc * N + off).astype(dtype)
+    alpha, beta = [(1.0, 0.0), (2.0, -1.0), (-1.0, 1.0), (0.5, 2.0)][rng.integers(4)]
+    pin = [None, "0", "1", "2"][rng.integers(4)] if dtype == np.float32 else None
+    with large_tile(pin):
+        got = run_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, A, lda, B, ldb, C0, ldc, off, off, off)
+    ref = C0.copy()
+    brute = orc.orc_dgemm_bruteforce if dtype == np.float64 else orc.orc_sgemm_bruteforce
+    brute(ta.encode(), tb.encode(), M, N, K, alpha, ptr(A[off:]), lda, ptr(B[off:]), ldb, beta, ptr(ref[off:]), ldc)
+    assert np.array_equal(got, ref), (dtype.__name__, ta, tb, M, N, K, lda, ldb, ldc, off, alpha, beta, pin)
+
+
 def test_dgemm_tile_special_scalars(pkg, L):
     M, N, K = 100, 90, 50
     A, B, C0 = rand_f64(M * K, 1), rand_f64(K * N, 2), rand_f64(M * N, 3)
