@@ -104,6 +104,18 @@ int pl_sgemm_tile_ws(char transA, char transB, long M, long N, long K, float alp
                      const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
                      void* stream);
 
+/* The same again with the caller's split count instead of the model's: K goes to `splits` workgroups per tile of C (in
+ * whole panels, so the count used may be lower; 1, or a workspace under splits * M * N elements, launches the unsplit
+ * kernel).  For a scheduler that knows a product will have the device to itself, where the model above assumes a
+ * second product running beside it (the end of a call: the reference's last subkernels of Subkernel.cpp:168 run alone
+ * on their queue). */
+int pl_dgemm_tile_split(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                        const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
+                        int splits, void* stream);
+int pl_sgemm_tile_split(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                        const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
+                        int splits, void* stream);
+
 /* Fitted constants of the tile-GEMM launcher's cost model: how it chooses between its macro tiles (fp32: 128 x 128,
  * 256 x 128 "wide", 256 x 256 "large") and how many ways it splits K for products with few tiles.  They describe one
  * device and one build of the kernels; the deploy tool measures them and writes Processed/Kernel-fit_dev-<id>.log, the
@@ -263,7 +275,7 @@ int PARALiA_autotune(const char* db_dir, const char* func, long D1, long D2, lon
                      int beta_zero, long T_in, long long pool_budget_bytes, pl_atc_info* info);
 /* static GEMM plan (CreateSubkernelsDgemm + request_data + run_operation, dgemm.cpp:123-205, Subkernel.cpp:90-247) */
 #define PL_PLAN_MAX_WAITS 12
-#define PL_PLAN_ROW (11 + PL_PLAN_MAX_WAITS)
+#define PL_PLAN_ROW (14 + PL_PLAN_MAX_WAITS)
 long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
                        int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]);
 /* makespan of one order (order_id >= 0) or of the best candidate (< 0) on the simulated H2D / compute / D2H pipeline;

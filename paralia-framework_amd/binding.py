@@ -6,7 +6,7 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libparalia.so")
 PL_PLAN_MAX_WAITS = 12
-PL_PLAN_ROW = 11 + PL_PLAN_MAX_WAITS
+PL_PLAN_ROW = 14 + PL_PLAN_MAX_WAITS
 
 
 class ParaliaError(RuntimeError):
@@ -77,6 +77,8 @@ _SIGS = {
     "pl_gemm_tile_choice": (_i, [_i, _c, _c, _l, _l, _l, _i, _l, _pi, _pi, _pi]),
     "pl_dgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _vp]),
     "pl_sgemm_tile_ws": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _vp]),
+    "pl_dgemm_tile_split": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _i, _vp]),
+    "pl_sgemm_tile_split": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _i, _vp]),
     "pl_dgeadd_tile": (_i, [_l, _l, _d, _vp, _l, _vp, _l, _vp, _l, _vp]),
     "pl_sgeadd_tile": (_i, [_l, _l, _f, _vp, _l, _vp, _l, _vp, _l, _vp]),
     "pl_daxpy": (_i, [_l, _d, _vp, _l, _vp, _l, _vp]),
@@ -164,5 +166,6 @@ def plan_rows(M, N, K, T, a_remote=1, b_remote=1, c_remote=1, beta_zero=0, elem=
     for i in range(n):
         r = buf[i * PL_PLAN_ROW:(i + 1) * PL_PLAN_ROW]
         rows.append(dict(kind=r[0], mi=r[1], ni=r[2], ki=r[3], stream=r[4], block=r[5], a_block=r[6], b_block=r[7],
-                         beta_mode=r[8], waits=[w for w in r[10:10 + r[9]]], kn=r[10 + PL_PLAN_MAX_WAITS]))
+                         beta_mode=r[8], waits=[w for w in r[10:10 + r[9]]], kn=r[10 + PL_PLAN_MAX_WAITS],
+                         row0=r[11 + PL_PLAN_MAX_WAITS], rows=r[12 + PL_PLAN_MAX_WAITS], splits=r[13 + PL_PLAN_MAX_WAITS]))
     return rows, tuple(stats)

@@ -9,6 +9,7 @@
 //              compute / D2H command streams for the best subkernel order (runtime/gemm_plan.cpp).
 // Without a database only the heuristic is possible.
 #include <cfloat>
+#include <climits>
 #include <cmath>
 #include <cstdlib>
 #include <algorithm>
@@ -305,6 +306,12 @@ paralia::StageTimes paralia_stage_times(const ATC* atc, long T) {
   st.slab_fixed = m->fit.slab_fixed_us * 1e-6;
   const char* thin = getenv("PARALIA_THIN_START");  // "0": never cut the first k tile into slabs
   st.thin_start = !(thin && *thin && atoi(thin) == 0);
+  // a strip of the call's last C tile splits K: one more round of workgroups with its fixed cost, the reduction's
+  // launch, and the reduction's pass over the slices
+  st.split_fixed = (m->fit.launcher.f32_small_fixed_us + m->fit.launcher.splitk_launch_us) * 1e-6;
+  st.split_pass_tb = 1e-6 / m->fit.launcher.pass_bytes_per_us;
+  const char* strip = getenv("PARALIA_STRIP_END");  // "0": the last C tile is never cut into row strips
+  st.strip_end = !(strip && *strip && atoi(strip) == 0);
   if (d.problem == BLAS3 && m->transient_amplitude > 0) {
     st.tr_amp = m->transient_amplitude;
     st.tr_idle = m->transient_idle_s;
@@ -380,6 +387,15 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
       // building a plan).  The second runs the full order search for the (at most three) T whose penalised probe is
       // within 10 % of the best, best probe first, and skips a T whose floor is above a result already in hand.
       struct Cand { long T; double probe_t, floor_t; };
+      // The tile size is chosen without the strip end: row strips take most of the last write-back off every tile size,
+      // and the larger the tile the more -- but a grid of few large tiles also ends with one compute stream idle for
+      // longer, which the simulated device (kernels one at a time) does not see (16384^3: T = 4096 with strips simulated
+      // 0.2 % faster than T = 2048 with strips, measured 1.3 % slower).  The chosen tile's order gets its strips below.
+      auto search_times = [&](long cand) {
+        paralia::StageTimes st = paralia_stage_times(this, cand);
+        st.strip_end = false;
+        return st;
+      };
       constexpr long PROBE_ABOVE_SUBKERNELS = 48;
       const char* verbose_env = getenv("PARALIA_VERBOSE");
       const bool chatty = verbose_env && atoi(verbose_env) > 1;
@@ -419,7 +435,10 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         if (gp.b_remote) t += st.h2d_ti + st.h2d_tb * std::min<double>(eighth, (double)gp.tn(gp.Ng() - 1) * std::min<long>(gp.T, problem.D3) / 8.0 * problem.dtype_sz);
         if (gp.c_remote) {
           const double smallest = (double)std::min(gp.tm(0), gp.tm(gp.Mg() - 1)) * std::min(gp.tn(0), gp.tn(gp.Ng() - 1));
-          t += st.d2h_ti + st.d2h_tb * smallest * problem.dtype_sz;
+          // (of a last tile cut into row strips, one strip: no thinner than a 128-row tile of the kernel)
+          const bool strips = st.strip_end && st.merge_saving > 0;
+          const double last_rows = (double)std::min(std::min(gp.tm(0), gp.tm(gp.Mg() - 1)), strips ? 128L : LONG_MAX);
+          t += st.d2h_ti + st.d2h_tb * last_rows * std::min(gp.tn(0), gp.tn(gp.Ng() - 1)) * problem.dtype_sz;
           if (!gp.beta_zero) t += st.t_reduce * smallest / ((double)gp.T * gp.T);
         }
         return t;
@@ -438,7 +457,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         if (cand < m->getMinT() && std::min(problem.D1, problem.D2) >= m->getMinT()) continue;
         paralia::GemmProblem gp = gemm_problem_of(problem, cand, exec_queues);
         if (gp.pool_blocks < 3 || gp.subkernels() > 20000) continue;
-        entries.push_back({cand, call_floor(gp, paralia_stage_times(this, cand)) * penalty(cand), gp});
+        entries.push_back({cand, call_floor(gp, search_times(cand)) * penalty(cand), gp});
       }
       std::stable_sort(entries.begin(), entries.end(), [](const Entry& x, const Entry& y) { return x.floor_t < y.floor_t; });
       std::vector<Cand> cands;
@@ -451,7 +470,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
           // a grid of a few dozen subkernels gets the full order search at once: its plans cost microseconds, and the
           // handful of orders of a probe misses the block orders that win there (sgemm 4096^3 from the host: T = 1536
           // probed at 3.24 ms, searched at 3.08, and left out of the finalists)
-          paralia::pick_gemm_order(e.gp, paralia_stage_times(this, cand), &r, /*probe=*/e.gp.subkernels() > PROBE_ABOVE_SUBKERNELS);
+          paralia::pick_gemm_order(e.gp, search_times(cand), &r, /*probe=*/e.gp.subkernels() > PROBE_ABOVE_SUBKERNELS);
         } catch (const std::runtime_error&) { continue; }
         cands.push_back({cand, r.t_total * penalty(cand), e.floor_t});
         best_probe = std::min(best_probe, r.t_total);
@@ -494,7 +513,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
         paralia::PipelineResult r;
         int oid = -1;
         try {
-          oid = paralia::pick_gemm_order(gp, paralia_stage_times(this, cand), &r);
+          oid = paralia::pick_gemm_order(gp, search_times(cand), &r);
         } catch (const std::runtime_error&) { continue; }
         const double score = r.t_total * penalty(cand);
         if (chatty) fprintf(stderr, "  full search T = %ld: %.3lf ms, order %d, %ld plans simulated so far\n", cand, r.t_total * 1e3, oid, paralia::plan_simulations.load());
@@ -502,7 +521,11 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
           best_t = score; best_T = cand; best_order = oid; best_r = r;
         }
       }
-      if (best_T >= 0) { searched_order = best_order; searched_r = best_r; }
+      if (best_T >= 0) {
+        const paralia::StageTimes st = paralia_stage_times(this, best_T);
+        if (st.strip_end) best_order = paralia::with_strip_end(gemm_problem_of(problem, best_T, exec_queues), st, best_order, &best_r);
+        searched_order = best_order; searched_r = best_r;
+      }
       if (best_T < 0) {
         // C narrower than every benchmarked tile: one tile across the short side, as square as that allows
         T = std::max(std::min(problem.D1, problem.D2), std::min(max_dim, m->exec->MinT()));
@@ -540,7 +563,7 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     pipeline.t_d2h_busy = r.t_d2h; pipeline.order_id = order_id;
     pred_t = r.t_total;
     pred_t_pesimistic = r.t_h2d + r.t_exec + r.t_d2h;
-    gp.k_split = 1 << (order_id / paralia::ORDER_K_SPLIT);  // a thin start adds k tiles
+    gp.k_split = 1 << (order_id % paralia::ORDER_STRIP_END / paralia::ORDER_K_SPLIT);  // a thin start adds k tiles
     update_sk_num(gp.subkernels());
     distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());
   } else if (problem.problem == BLAS2) {

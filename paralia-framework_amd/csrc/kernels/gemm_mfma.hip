@@ -900,9 +900,18 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
 // Macro tile and split count of one product.
 struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; };
 template <typename T>
-TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true) {
+TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true,
+                       int want_splits = 0) {
   TileChoice c;
-  c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
+  if (want_splits > 1 && have_ws) {
+    // the caller's split count, in whole panels per chunk like the model's own
+    const long gran = sizeof(T) == 4 ? PLK_F32_DEEP_BK : 16;
+    const long kc = (((K + want_splits - 1) / want_splits) + gran - 1) / gran * gran;
+    const long se = (K + kc - 1) / kc;
+    if (se > 1) c.splits = (int)se, c.kchunk = (int)kc;
+  } else {
+    c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
+  }
   if (c.splits > 1 && (long)c.splits * M * N * (long)sizeof(T) > workspace_bytes) c.splits = 1, c.kchunk = 0;
   // fp32 has two more macro tiles, chosen per call by the fitted model below when they are faster than 128 x 128.
   //  * 256 x 256 x 32 ("large", every transpose): its inner loop runs 1 % faster per k (a 16-byte operand read per
@@ -945,7 +954,7 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
 
 template <typename T>
 int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
-                T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0) {
+                T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0, int want_splits = 0) {
   using Tr = Traits<T>;
   const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
   const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
@@ -966,7 +975,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   // a K-major operand loaded straight into LDS takes eight rows per request with 32-bit lane offsets: leading dimensions
   // beyond that keep the tiles that stage through registers
   const bool dma_fits = (!at || lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES) && (!bnn || ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES);
-  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits);
+  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits);
   const int kchunk = choice.kchunk, splits = choice.splits;
   const bool big = choice.big, wide = choice.wide;
   const int TM_RT = choice.tm, TN_RT = choice.tn;
@@ -1076,6 +1085,22 @@ extern "C" int pl_gemm_tile_choice(int elem_size, char transA, char transB, long
 
 extern "C" long pl_gemm_tile_workspace_bytes(long M, long N, long K, int elem_size) {
   return elem_size == 8 ? plk::workspace_bytes_for<double>(M, N, K) : elem_size == 4 ? plk::workspace_bytes_for<float>(M, N, K) : 0;
+}
+
+extern "C" int pl_dgemm_tile_split(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                                   const double* B, long ldb, double beta, double* C, long ldc, void* workspace,
+                                   long workspace_bytes, int splits, void* stream) {
+  if (splits < 1) return PL_ERR_ARG;
+  return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                  (double*)workspace, workspace_bytes, splits);
+}
+
+extern "C" int pl_sgemm_tile_split(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                                   const float* B, long ldb, float beta, float* C, long ldc, void* workspace,
+                                   long workspace_bytes, int splits, void* stream) {
+  if (splits < 1) return PL_ERR_ARG;
+  return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                 (float*)workspace, workspace_bytes, splits);
 }
 
 extern "C" int pl_dgemm_tile_ws(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,

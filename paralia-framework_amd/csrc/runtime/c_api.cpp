@@ -250,7 +250,8 @@ static paralia::GemmProblem gp_of(long M, long N, long K, long T, int a_remote, 
 
 // Builds the static plan and writes it as rows of PL_PLAN_ROW ints:
 // kind, mi, ni, ki, stream, block, a_block, b_block, beta_mode, nwait, wait[0..PL_PLAN_MAX_WAITS-1], kn (k tiles of a
-// GEMM launch; more than 1 only for order ids of 80000 and above, the merged K chains).
+// GEMM launch; more than 1 only for order ids of 80000 and above, the merged K chains), row0, rows (a GEMM or
+// WRITEBACK on a row strip of its C tile; rows = 0: the whole tile), splits (ways a strip's launch splits K).
 // stats: [blocks_used, fetch_A, fetch_B, fetch_C, evictions, subkernels].  Returns the number of commands.
 long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remote, int c_remote, int beta_zero, int elem,
                        int exec_queues, long pool_blocks, int order_id, int* rows, long max_rows, long stats[6]) {
@@ -270,6 +271,7 @@ long PARALiA_gemm_plan(long M, long N, long K, long T, int a_remote, int b_remot
         r[8] = c.beta_mode; r[9] = c.nwait;
         for (int w = 0; w < PL_PLAN_MAX_WAITS; ++w) r[10 + w] = w < c.nwait ? c.wait[w] : -1;
         r[10 + PL_PLAN_MAX_WAITS] = c.kn;
+        r[11 + PL_PLAN_MAX_WAITS] = c.row0; r[12 + PL_PLAN_MAX_WAITS] = c.rows; r[13 + PL_PLAN_MAX_WAITS] = c.splits;
       }
   });
   return n;
@@ -286,6 +288,7 @@ double PARALiA_gemm_plan_simulate(long M, long N, long K, long T, int a_remote, 
     paralia::StageTimes st;
     st.t_exec = t_exec; st.h2d_ti = h2d_ti; st.h2d_tb = h2d_tb; st.d2h_ti = d2h_ti; st.d2h_tb = d2h_tb; st.t_reduce = t_reduce;
     st.h2d_sl = h2d_sl; st.d2h_sl = d2h_sl;
+    st.strip_end = false;   // its price comes with the kernel fit of a database: a pinned id is simulated, the search does not offer it
     paralia::PipelineResult r;
     if (order_id >= 0) {
       r = paralia::simulate_plan(paralia::build_gemm_plan(gp, order_id), st);

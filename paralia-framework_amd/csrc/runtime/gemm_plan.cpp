@@ -20,6 +20,7 @@ namespace paralia {
 
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id) {
   const int Mg = p.Mg(), Ng = p.Ng(), Kg = p.Kg();   // p.k_split is the caller's business (build_gemm_plan sets it)
+  order_id %= ORDER_STRIP_END;             // strips change launches, not the order
   order_id %= ORDER_K_SPLIT;
   order_id %= ORDER_MERGE_CHAINS;          // merging launches does not change the order
   order_id %= 40000;                       // nor does the eviction policy
@@ -225,17 +226,35 @@ void add_wait(std::vector<Cmd>& cmds, Cmd& c, int w, Covered& cov) {
   cov.at[c.stream][cmds[w].stream] = w;
 }
 
+// Row strips for the call's last launch (ORDER_STRIP_END), which multiplies launch_k of k into the C tile (mi, ni): rows
+// per strip, 0 when the tile is too small to cut, and how many ways a strip's launch splits K.  Up to four strips of at
+// least 256 rows, in whole 128-row tiles of the kernel; a strip's workgroups are to fill every compute unit twice (512
+// places) as long as a workgroup keeps 512 of k.
+int strip_rows(const GemmProblem& p, int mi, int ni, long launch_k, int* splits) {
+  const long tm = p.tm(mi), tn = p.tn(ni);
+  const long n = std::min(4L, tm / 256);
+  *splits = 0;
+  if (n < 2) return 0;
+  const long rows = ((tm + n - 1) / n + 127) / 128 * 128;
+  const long tiles = ((rows + 127) / 128) * ((tn + 127) / 128);
+  const long want = (512 + tiles - 1) / tiles;
+  *splits = (int)std::max(1L, std::min(want, launch_k / 512));
+  return (int)rows;
+}
+
 }  // namespace
 
 GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   if (p_in.T <= 0 || p_in.M <= 0 || p_in.N <= 0) throw std::runtime_error("gemm plan: invalid dimensions");
   GemmPlan plan;
   plan.p = p_in;
-  if (order_id < 0 || order_id / ORDER_K_SPLIT > 3) throw std::runtime_error("gemm plan: unknown order id");
+  if (order_id < 0 || order_id / ORDER_STRIP_END > 1) throw std::runtime_error("gemm plan: unknown order id");
+  const bool strip_end = order_id >= ORDER_STRIP_END;
+  order_id %= ORDER_STRIP_END;
   plan.p.k_split = 1 << (order_id / ORDER_K_SPLIT);
   const GemmProblem& p = plan.p;
   if (order_id >= ORDER_K_SPLIT && p.slabs() == 1) throw std::runtime_error("gemm plan: this problem has no thin start");
-  plan.order_id = order_id;
+  plan.order_id = order_id + (strip_end ? ORDER_STRIP_END : 0);
   plan.task_order = gemm_task_order(p, order_id);
   order_id %= ORDER_K_SPLIT;
   const bool merge = order_id >= ORDER_MERGE_CHAINS;
@@ -377,6 +396,7 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
   };
 
   std::vector<int> gemm_waits, w;   // scratch, reused by every subkernel
+  int strip_splits = 0;
   for (int pos = 0; pos < (int)plan.task_order.size(); ++pos) {
     const int t = plan.task_order[pos];
     const int ki = t % Kg, ni = (t / Kg) % Ng, mi = t / (Kg * Ng);
@@ -446,11 +466,17 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
       open.ablk = ablk; open.bblk = bblk; open.beta_mode = beta_mode;
       open.waits = gemm_waits;
     }
+    // The call's last launch on a C tile that goes back to the host (ORDER_STRIP_END): row strips, see below.
+    int rows_per = 0;
+    if (strip_end && p.c_remote && fired[ci] + 1 == Kg && pos + 1 == (int)plan.task_order.size()) {
+      long launch_k = 0;
+      for (int kt = open.ki0; kt < open.ki0 + open.kn; ++kt) launch_k += p.tk(kt);
+      rows_per = strip_rows(p, mi, ni, launch_k, &strip_splits);
+    }
     int gemm_idx = -1;
-    if (!merge) {
-      gemm_idx = close_chain();
-      if (ablk >= 0) note_reader(ablk, gemm_idx);
-      if (bblk >= 0) note_reader(bblk, gemm_idx);
+    auto after_launch = [&](int launch) {
+      if (ablk >= 0) note_reader(ablk, launch);
+      if (bblk >= 0) note_reader(bblk, launch);
       // A tile that no later subkernel reads gives its block back at once (its readers stay pending on the block): the
       // FIFO then hands out the longest-dead block first, so the fetch that reuses it rarely waits and the copy stream
       // can run a whole k-step ahead of the subkernels even when the pool is much smaller than the operands.
@@ -464,9 +490,64 @@ GemmPlan build_gemm_plan(const GemmProblem& p_in, int order_id) {
         b_blk[bi] = -1;
         free_list.push_back(bblk);
       }
+    };
+    if (!merge && rows_per == 0) {
+      gemm_idx = close_chain();
+      after_launch(gemm_idx);
     }
 
-    if (++fired[ci] == Kg && p.c_remote) {
+    if (++fired[ci] == Kg && p.c_remote && rows_per > 0) {
+      // The last launch of the call in row strips, one launch each on the tile's stream, and with it everything that
+      // follows on those rows: the fetch of the caller's C and the lazy reduce (beta != 0), and the write-back.  The
+      // strips' copies and kernels pipeline, so what is left when the last kernel ends is a strip's write-back.
+      const int accb = c_blk[ci];
+      const int tm = (int)p.tm(mi), stream = STREAM_EXEC0 + queue_of[ci];
+      std::vector<int> strip_last;   // per strip: the command its write-back waits for
+      for (int r0 = 0; r0 < tm; r0 += rows_per) {
+        Cmd c;
+        c.kind = CMD_GEMM; c.mi = mi; c.ni = ni; c.ki = open.ki0; c.kn = open.kn; c.stream = stream;
+        c.block = accb; c.a_block = open.ablk; c.b_block = open.bblk; c.beta_mode = open.beta_mode;
+        c.row0 = r0; c.rows = std::min(rows_per, tm - r0); c.splits = strip_splits;
+        cmds.push_back(c);
+        for (int x : open.waits) add_wait(cmds, cmds.back(), x, covered);
+        strip_last.push_back((int)cmds.size() - 1);
+      }
+      open.active = false;
+      if (!merge) after_launch(strip_last.back());   // (the stream's last strip covers the earlier ones)
+      if (!p.beta_zero) {
+        w.clear();
+        const int sb = alloc(accb, -1, w);
+        blocks[sb].kind = 3; blocks[sb].idx = ci;
+        std::vector<int> fetches;
+        for (int r0 = 0; r0 < tm; r0 += rows_per) {
+          Cmd f;
+          f.kind = CMD_FETCH_C; f.mi = mi; f.ni = ni; f.stream = STREAM_H2D; f.block = sb; f.row0 = r0; f.rows = std::min(rows_per, tm - r0);
+          cmds.push_back(f);
+          for (int x : w) add_wait(cmds, cmds.back(), x, covered);
+          fetches.push_back((int)cmds.size() - 1);
+        }
+        blocks[sb].content_cmd = fetches.back();
+        ++plan.n_fetch[2];
+        for (size_t i = 0; i < strip_last.size(); ++i) {
+          Cmd r;
+          r.kind = CMD_REDUCE; r.mi = mi; r.ni = ni; r.stream = stream; r.block = accb; r.a_block = sb;
+          r.row0 = cmds[strip_last[i]].row0; r.rows = cmds[strip_last[i]].rows;
+          cmds.push_back(r);
+          add_wait(cmds, cmds.back(), fetches[i], covered);
+          strip_last[i] = (int)cmds.size() - 1;
+        }
+        release(sb, strip_last.back());
+      }
+      for (size_t i = 0; i < strip_last.size(); ++i) {
+        Cmd wb;
+        wb.kind = CMD_WRITEBACK; wb.mi = mi; wb.ni = ni; wb.stream = STREAM_D2H; wb.block = accb;
+        wb.row0 = cmds[strip_last[i]].row0; wb.rows = cmds[strip_last[i]].rows;
+        cmds.push_back(wb);
+        add_wait(cmds, cmds.back(), strip_last[i], covered);
+      }
+      release(accb, (int)cmds.size() - 1);
+      c_blk[ci] = -1;
+    } else if (fired[ci] == Kg && p.c_remote) {
       if (open.active) gemm_idx = close_chain();
       const int accb = c_blk[ci];
       int last = gemm_idx;
@@ -587,7 +668,7 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
       switch (c.kind) {
         case CMD_FETCH_A: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tk(c.ki) * p.elem; break;
         case CMD_FETCH_B: dur = st.h2d_ti + st.h2d_tb * (double)p.tk(c.ki) * p.tn(c.ni) * p.elem; break;
-        case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+        case CMD_FETCH_C: dur = st.h2d_ti + st.h2d_tb * (double)(c.rows > 0 ? c.rows : p.tm(c.mi)) * p.tn(c.ni) * p.elem; break;
         case CMD_GEMM:
           for (int k = c.ki; k < c.ki + c.kn; ++k) {
             if (k < p.slabs() && p.slabs() > 1)
@@ -595,9 +676,14 @@ PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st) {
             else dur += st.exec_time(p.T, p.tm(c.mi), p.tn(c.ni), p.tk(k));
           }
           if (c.kn > 1) dur = std::max(0.5 * dur, dur - (c.kn - 1) * st.merge_saving * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2);
+          if (c.rows > 0) {
+            // a row strip: its share of the tile's launch, and what splitting K adds
+            dur *= (double)c.rows / (double)p.tm(c.mi);
+            if (c.splits > 1) dur += st.split_fixed + st.split_pass_tb * (2.0 * c.splits + 1.0) * (double)c.rows * p.tn(c.ni) * p.elem;
+          }
           break;
-        case CMD_REDUCE: dur = st.t_reduce * ((double)p.tm(c.mi) * p.tn(c.ni)) / T2; break;
-        case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)p.tm(c.mi) * p.tn(c.ni) * p.elem; break;
+        case CMD_REDUCE: dur = st.t_reduce * ((double)(c.rows > 0 ? c.rows : p.tm(c.mi)) * p.tn(c.ni)) / T2; break;
+        case CMD_WRITEBACK: dur = st.d2h_ti + st.d2h_tb * (double)(c.rows > 0 ? c.rows : p.tm(c.mi)) * p.tn(c.ni) * p.elem; break;
       }
       if (c.stream == STREAM_H2D) {
         const double s = std::max(ready, h2d);
@@ -805,8 +891,24 @@ int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* 
         }
     }
   const Group& pick = (grp[0].id < 0 || (grp[1].id >= 0 && grp[1].r.t_total < 0.99 * grp[0].r.t_total)) ? grp[1] : grp[0];
-  if (best_out) *best_out = pick.r;
-  return pick.id;
+  PipelineResult chosen = pick.r;
+  const int id = (st.strip_end && !probe) ? with_strip_end(p, st, pick.id, &chosen) : pick.id;
+  if (best_out) *best_out = chosen;
+  return id;
+}
+
+int with_strip_end(const GemmProblem& p, const StageTimes& st, int order_id, PipelineResult* r) {
+  // With C on the device nothing is written back and the flag builds the same plan.  Offered to merged K chains only:
+  // there the last launch is long and its strips cost little beside it; the strips of a last k-step took as long as
+  // they saved or longer (dgemm 8192^3: 23.28 -> 23.32 ms, 12288^3: 56.12 -> 56.16 ms, simulated 0.1 ms shorter).
+  if (!p.c_remote || order_id >= ORDER_STRIP_END || order_id % ORDER_K_SPLIT < ORDER_MERGE_CHAINS) return order_id;
+  const std::vector<int> strip_id = {order_id + ORDER_STRIP_END};
+  const std::vector<Evaluated> strip = evaluate_orders(p, st, strip_id);
+  if (strip[0].ok && r && strip[0].r.t_total < r->t_total * (1.0 - 1e-3)) {
+    *r = strip[0].r;
+    return strip_id[0];
+  }
+  return order_id;
 }
 
 }  // namespace paralia

@@ -68,6 +68,10 @@ struct Cmd {
   int a_block = -1;   // GEMM: block of the A tile (-1: caller's memory); REDUCE: block holding the fetched source C
   int b_block = -1;   // GEMM: block of the B tile (-1: caller's memory)
   int kn = 1;         // GEMM: number of consecutive k tiles ki .. ki + kn - 1 multiplied by this one launch
+  // FETCH_C / GEMM / REDUCE / WRITEBACK on a row strip of the C tile: rows row0 .. row0 + rows - 1 of it (rows == 0: the
+  // whole tile)
+  int row0 = 0, rows = 0;
+  int splits = 0;     // GEMM: ways the launch is to split K over workgroups (0: the kernel launcher's own choice)
   int beta_mode = BETA_ONE;
   int nwait = 0;
   int wait[MAX_WAITS];  // earlier commands on other streams that must have completed
@@ -114,6 +118,13 @@ constexpr int ORDER_BLOCK_ROWS = 100;
 constexpr int ORDER_FULL_PANEL = 99;
 // + 160000 * s: thin start (GemmProblem::k_split = 2^s): s = 1 or 2: 2^s equal slabs; s = 3: the graded start.
 constexpr int ORDER_K_SPLIT = 160000;
+// + 640000: strip end.  The last launch of the call -- the last k-step, or the whole merged K chain, of the C tile the
+// order completes last -- is made in row strips of that tile, one launch after the other, and what follows it on those
+// rows (with beta != 0 the fetch of the caller's C and the lazy reduce; the write-back) strip by strip behind them, so
+// that the copies left over when the last kernel ends are a strip's, not a tile's.  A strip alone has too few
+// 128 x 128 tiles for the device, so its launch splits K (Cmd::splits).  Only where C goes back to the host; elsewhere,
+// and for a last tile under 512 rows, the id builds the same plan as without it.
+constexpr int ORDER_STRIP_END = 640000;
 inline int order_id_of(int orient, int w) { return orient * 10000 + w; }
 std::vector<int> gemm_task_order(const GemmProblem& p, int order_id);
 // probe = true: a handful of representative orders, enough to rank tile sizes before the full search
@@ -157,6 +168,10 @@ struct StageTimes {
   // or deeper, in inverse proportion to the depth below that (measured inside streamed calls, two launches sharing the
   // device: 2048 x 2048 x 1024 slabs +2 us, x 512 slabs +4.5 us against a quarter of the whole tile's 231.5 us)
   double slab_fixed = 2e-6;
+  // a launch that splits K s ways (Cmd::splits): one more round's fixed cost and the reduction's launch, and the
+  // reduction's pass over 2 s + 1 copies of the strip
+  double split_fixed = 10.6e-6, split_pass_tb = 1.0 / 6.15e12;
+  bool strip_end = true;             // offer the strip end (order ids of 640000 and above) to the order search
 };
 struct PipelineResult {
   double t_total = 0, t_h2d = 0, t_exec = 0, t_d2h = 0;  // makespan and busy time per resource
@@ -164,7 +179,11 @@ struct PipelineResult {
 PipelineResult simulate_plan(const GemmPlan& plan, const StageTimes& st);
 extern std::atomic<long> plan_simulations;   // plans simulated by this process so far (the order search's unit of work)
 // Builds every candidate order, simulates it, returns the id with the smallest makespan.
+// (with StageTimes::strip_end, and not for a probe, the winner goes through with_strip_end)
 int pick_gemm_order(const GemmProblem& p, const StageTimes& st, PipelineResult* best, bool probe = false);
+// The order also with its last C tile in row strips (ORDER_STRIP_END): that id, and its result in *r, when the simulated
+// call gets shorter than *r by more than a thousandth; else the id as it came.
+int with_strip_end(const GemmProblem& p, const StageTimes& st, int order_id, PipelineResult* r);
 
 }  // namespace paralia
 #endif

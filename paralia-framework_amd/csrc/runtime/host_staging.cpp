@@ -18,6 +18,9 @@ void chk(int rc, const char* what) {
 // A dense block of `cols` columns of `rows` elements between a pinned slot and the device, through the 2-D copy call (on
 // a stream of the 1-D call a copy was seen to start only when the copy running on the opposite-direction stream had
 // finished).  One long column (a vector span) goes as columns of 64 KiB plus a short tail.
+// device (leading dimension ld_src, 0 or rows = dense) -> a dense pinned slot
+void device_to_slot_async(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream);
+
 void dense_copy_async(void* dst, const void* src, long rows, long cols, int elem, void* stream) {
   if (cols > 1) {
     chk(pl_copy2d_async(dst, rows, src, rows, rows, cols, elem, stream), "staged tile copy");
@@ -27,6 +30,10 @@ void dense_copy_async(void* dst, const void* src, long rows, long cols, int elem
   if (n > 0) chk(pl_copy2d_async(dst, col, src, col, col, n, 1, stream), "staged tile copy");
   if (bytes > done)
     chk(pl_copy2d_async((char*)dst + done, bytes - done, (const char*)src + done, bytes - done, bytes - done, 1, 1, stream), "staged tile copy");
+}
+void device_to_slot_async(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream) {
+  if (ld_src <= 0 || ld_src == rows) dense_copy_async(dst, src, rows, cols, elem, stream);
+  else chk(pl_copy2d_async(dst, rows, src, ld_src, rows, cols, elem, stream), "staged tile copy");
 }
 }  // namespace
 
@@ -181,25 +188,25 @@ void HostStager::flush(int s) {
   p.active = false;
 }
 
-void HostStager::write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream) {
+void HostStager::write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream, long ld_src) {
   if (rows <= 0 || cols <= 0) return;
   const long long bytes = (long long)rows * cols * elem;
   reserve(bytes);
   const int s = (int)(out_next_++ % SLOTS);
   flush(s);
-  dense_copy_async(out_[s], src, rows, cols, elem, stream);
+  device_to_slot_async(out_[s], src, ld_src, rows, cols, elem, stream);
   chk(pl_event_record(out_ev_[s], stream), "event record");
   Pending& p = pending_[s];
   p.dst = dst; p.ld = ld_dst; p.rows = rows; p.cols = cols; p.elem = elem; p.active = true;
 }
 
 void HostStager::write_back_deferred(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream,
-                                     void* const* after, int n_after) {
+                                     void* const* after, int n_after, long ld_src) {
   if (rows <= 0 || cols <= 0) return;
   reserve((long long)rows * cols * elem);
   // a dropped wait would let the copy start before the tile's kernels have finished
   if (n_after < 0 || n_after > MAX_DEFERRED_WAITS) throw paralia_error(PL_ERR_ARG, "deferred write-back: too many events to wait for");
-  Request r{dst, ld_dst, src, rows, cols, elem, stream, {nullptr}, n_after};
+  Request r{dst, ld_dst, src, rows, cols, elem, stream, {nullptr}, n_after, ld_src};
   for (int i = 0; i < r.n_after; ++i) r.after[i] = after[i];
   {
     std::lock_guard<std::mutex> lk(dmu_);
@@ -236,7 +243,7 @@ void HostStager::deferred_loop() {
         lk.unlock();
         try {
           for (int i = 0; i < f.r.n_after; ++i) chk(pl_stream_wait_event(f.r.stream, f.r.after[i]), "stream wait event");
-          dense_copy_async(out_[f.slot], f.r.src, f.r.rows, f.r.cols, f.r.elem, f.r.stream);
+          device_to_slot_async(out_[f.slot], f.r.src, f.r.ld_src, f.r.rows, f.r.cols, f.r.elem, f.r.stream);
           chk(pl_event_record(out_ev_[f.slot], f.r.stream), "event record");
         } catch (...) {
           err = std::current_exception();

@@ -61,9 +61,9 @@ class HostStager {
   // dst (device, leading dimension ld_dst; 0 = dense, i.e. rows)  <-  src (pageable host, leading dimension ld_src), on
   // `stream`.
   void fetch(void* dst, const void* src, long ld_src, long rows, long cols, int elem, void* stream, long ld_dst = 0);
-  // dst (pageable host, leading dimension ld_dst)  <-  src (device, dense) on `stream`; the host-side scatter happens
-  // when the slot is needed again or in finish().
-  void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream);
+  // dst (pageable host, leading dimension ld_dst)  <-  src (device, leading dimension ld_src; 0 = dense, i.e. rows) on
+  // `stream`; the host-side scatter happens when the slot is needed again or in finish().
+  void write_back(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream, long ld_src = 0);
   // The same, handed to a background thread: it makes `stream` wait for the n_after events (the tile's last kernels),
   // copies the tile into a pinned slot as slots come free, waits for the copy and scatters it.  The caller does not
   // wait for a slot, so the thread that enqueues a plan keeps going when many C tiles complete close together (with
@@ -71,7 +71,7 @@ class HostStager {
   // a call with a pageable C took 148 ms instead of 125 ms at 16384^3).  Nothing else may use `stream` or the slots
   // until finish(); the device memory at src must stay untouched until then.
   void write_back_deferred(void* dst, long ld_dst, const void* src, long rows, long cols, int elem, void* stream,
-                           void* const* after, int n_after);
+                           void* const* after, int n_after, long ld_src = 0);
   // Completes every pending scatter, deferred ones included (those need not have been waited for: their copies are
   // synchronised here); rethrows what the background thread ran into.  The blocking ones need the streams synchronised.
   void finish();
@@ -98,7 +98,7 @@ class HostStager {
   // deferred write-backs: requests in call order; the background thread owns the out_ slots while any are open
   struct Request {
     void* dst; long ld; const void* src; long rows, cols; int elem; void* stream;
-    void* after[MAX_DEFERRED_WAITS]; int n_after;
+    void* after[MAX_DEFERRED_WAITS]; int n_after; long ld_src;
   };
   int device_ = 0;             // device that was current when the background thread was started; the thread makes it its own
   void deferred_loop();

@@ -295,6 +295,10 @@ template <> struct GemmFns<double> {
                   double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_dgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
   }
+  static int tile_split(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
+                        double be, double* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
+    return pl_dgemm_tile_split(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, s);
+  }
   static int geadd(long M, long N, double be, const double* s, long lds, const double* a, long lda, double* o, long ldo, void* st) {
     return pl_dgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
   }
@@ -304,6 +308,10 @@ template <> struct GemmFns<float> {
   static int tile(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                   float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_sgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
+  static int tile_split(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
+                        float be, float* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
+    return pl_sgemm_tile_split(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, s);
   }
   static int geadd(long M, long N, float be, const float* s, long lds, const float* a, long lda, float* o, long ldo, void* st) {
     return pl_sgeadd_tile(M, N, be, s, lds, a, lda, o, ldo, st);
@@ -328,8 +336,8 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   if (pageable[0] || pageable[1] || pageable[2]) stager.reserve((long long)Tt * Tt * (long long)sizeof(T));
   StagerScope staged(stager);
   // what the tile kernel can use to split K when a tile product has too few workgroups (small T): the largest need
-  // over the launches of the plan -- full and ragged tile extents, slabs of a thin start, and merged chains, whose one
-  // launch covers the summed k of their tiles
+  // over the launches of the plan -- full and ragged tile extents, slabs of a thin start, merged chains, whose one
+  // launch covers the summed k of their tiles, and row strips, which come with their own split count
   long ws_bytes = 0;
   {
     std::vector<std::array<long, 3>> seen;
@@ -337,7 +345,8 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
       if (c.kind != CMD_GEMM) continue;
       long k = 0;
       for (int kt = c.ki; kt < c.ki + c.kn; ++kt) k += p.tk(kt);
-      const std::array<long, 3> shape = {p.tm(c.mi), p.tn(c.ni), k};
+      const std::array<long, 3> shape = {c.rows > 0 ? (long)c.rows : p.tm(c.mi), p.tn(c.ni), k};
+      if (c.splits > 1) ws_bytes = std::max(ws_bytes, (long)c.splits * shape[0] * shape[1] * (long)sizeof(T));
       if (std::find(seen.begin(), seen.end(), shape) != seen.end()) continue;
       seen.push_back(shape);
       ws_bytes = std::max(ws_bytes, pl_gemm_tile_workspace_bytes(shape[0], shape[1], shape[2], (int)sizeof(T)));
@@ -403,10 +412,12 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         else chk(pl_copy2d_async(dst, ld_dst, src, ldb, rows, cols, sizeof(T), s), "fetch B tile");
       } break;
       case CMD_FETCH_C: {
-        const long rows = p.tm(c.mi), cols = p.tn(c.ni);
-        const T* src = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
-        if (pageable[2]) stager.fetch(R.pool.at(c.block), src, ldc, rows, cols, sizeof(T), s);
-        else chk(pl_copy2d_async(R.pool.at(c.block), rows, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
+        // the tile, or the row strip of it the command names, into those rows of the block (which holds the whole tile)
+        const long m = p.tm(c.mi), rows = c.rows > 0 ? c.rows : m, cols = p.tn(c.ni);
+        const T* src = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc + c.row0;
+        T* dst = (T*)R.pool.at(c.block) + c.row0;
+        if (pageable[2]) stager.fetch(dst, src, ldc, rows, cols, sizeof(T), s, m);
+        else chk(pl_copy2d_async(dst, m, src, ldc, rows, cols, sizeof(T), s), "fetch C tile");
       } break;
       case CMD_GEMM: {
         const long m = p.tm(c.mi), n = p.tn(c.ni);
@@ -427,23 +438,33 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         const T bp = c.beta_mode == BETA_ZERO ? T(0) : c.beta_mode == BETA_ONE ? T(1) : beta;
         if (la < 1) la = 1;
         if (lb < 1) lb = 1;
-        chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, s), "tile gemm launch");
+        if (c.rows > 0) {
+          // a row strip of the tile: those rows of op(A) and of C, the launch splitting K as the plan says
+          a += at ? (long)c.row0 * la : (long)c.row0;
+          cc += c.row0;
+          chk(GemmFns<T>::tile_split(ta, tb, c.rows, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes,
+                                     std::max(1, c.splits), s), "tile gemm launch");
+        } else {
+          chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, s), "tile gemm launch");
+        }
       } break;
       case CMD_REDUCE: {
-        const long m = p.tm(c.mi), n = p.tn(c.ni);
-        T* acc = (T*)R.pool.at(c.block);
-        chk(GemmFns<T>::geadd(m, n, beta, (const T*)R.pool.at(c.a_block), m, acc, m, acc, m, s), "lazy reduce launch");
+        const long m = p.tm(c.mi), n = p.tn(c.ni), rows = c.rows > 0 ? c.rows : m;
+        T* acc = (T*)R.pool.at(c.block) + c.row0;
+        chk(GemmFns<T>::geadd(rows, n, beta, (const T*)R.pool.at(c.a_block) + c.row0, m, acc, m, acc, m, s), "lazy reduce launch");
       } break;
       case CMD_WRITEBACK: {
-        const long m = p.tm(c.mi), n = p.tn(c.ni);
-        T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc;
+        // the tile, or the row strip of it the command names (the accumulator block holds the whole tile, m rows)
+        const long m = p.tm(c.mi), n = p.tn(c.ni), rows = c.rows > 0 ? c.rows : m;
+        T* dst = C + (long)c.mi * Tt + (long)c.ni * Tt * ldc + c.row0;
+        const T* src = (const T*)R.pool.at(c.block) + c.row0;
         if (deferred) {
           static_assert(MAX_WAITS <= HostStager::MAX_DEFERRED_WAITS, "a deferred write-back must be able to carry every wait of a command");
           void* after[MAX_WAITS];
           for (int w = 0; w < c.nwait; ++w) after[w] = ev[c.wait[w]];
-          stager.write_back_deferred(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s, after, c.nwait);
-        } else if (pageable[2]) stager.write_back(dst, ldc, R.pool.at(c.block), m, n, sizeof(T), s);
-        else chk(pl_copy2d_async(dst, ldc, R.pool.at(c.block), m, m, n, sizeof(T), s), "write back C tile");
+          stager.write_back_deferred(dst, ldc, src, rows, n, sizeof(T), s, after, c.nwait, m);
+        } else if (pageable[2]) stager.write_back(dst, ldc, src, rows, n, sizeof(T), s, m);
+        else chk(pl_copy2d_async(dst, ldc, src, m, rows, n, sizeof(T), s), "write back C tile");
       } break;
     }
     if (trace) chk(pl_event_record(R.res.timing_events[2 + 2 * i], s), "event record");

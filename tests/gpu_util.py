@@ -83,4 +83,4 @@ def k_tiles(info, K, T=None):
     the first k tile is cut into 2 (s = 1) or 4 (s = 2: equal, s = 3: graded) slabs that are fetched and multiplied
     separately)."""
     T = T or info.T
-    return -(-K // T) + (1, 2, 4, 4)[info.order_id // 160000] - 1
+    return -(-K // T) + (1, 2, 4, 4)[info.order_id % 640000 // 160000] - 1

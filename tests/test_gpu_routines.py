@@ -573,6 +573,52 @@ def test_gemm_thin_start_with_odd_slabs(pkg, L, orc, ta, tb, order, T, monkeypat
             assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, locs)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("order", [720000, 720001, 880001, 1200001, 720101, 640000, 650001, 800001])
+@pytest.mark.parametrize("locs", [(-1, -1, -1), (-2, -1, -2), (0, 0, -1)])
+def test_gemm_strip_end_exact_on_integers(pkg, L, ta, tb, order, locs, monkeypatch):
+    """Order ids of 640000 and above: the last launch of the call -- on the last C tile, 700 x 76 here at T = 1024, its
+    merged K chain (720000 and above) or its last k-step -- is made in two row strips of 384 and 316 rows (the merged
+    chain's splitting K two ways into the workspace), and the tile's write-back (into pinned or pageable memory), with
+    beta != 0 also the fetch of the caller's C and the lazy reduce, strip by strip behind them.  Alone, with a thin and
+    a graded start, after a one-tile block; every transpose, A and B pinned / pageable / on the device, fp64 and fp32,
+    beta = 0 over NaN and beta != 0: bit for bit the untiled result on integer operands (exact in either type,
+    whatever the order of the sums)."""
+    monkeypatch.setenv("PARALIA_GEMM_ORDER", str(order))
+    M, N, K, T = 1724, 1100, 1200 + [720000, 720001, 880001, 1200001, 720101, 640000, 650001, 800001].index(order), 1024
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    rng = np.random.default_rng(order + 3 * len(ta + tb))
+    for dtype in (np.float64, np.float32):
+        A = rng.integers(-4, 5, ra * ca).astype(dtype)
+        B = rng.integers(-4, 5, rb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, M * N).astype(dtype)
+        opA = A.reshape(ca, ra).T.astype(np.float64) if ta == "N" else A.reshape(ca, ra).astype(np.float64)
+        opB = B.reshape(cb, rb).T.astype(np.float64) if tb == "N" else B.reshape(cb, rb).astype(np.float64)
+        prod = 2.0 * (opA @ opB)                                  # integers far below 2^24: exact in both types
+        for beta in (0.0, -1.0):
+            ref = (prod + beta * C0.reshape(N, M).T.astype(np.float64)).T.reshape(-1).astype(dtype)
+            start = np.full(M * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+            bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
+            info = call_gemm(pkg, L, dtype, ta, tb, M, N, K, 2.0, beta, bA, ra, bB, rb, bC, M, T=T)
+            assert info.order_id == order and info.T == T
+            assert np.array_equal(bC.get(), ref), (np.dtype(dtype).name, beta)
+            if locs[2] == -1:
+                # the library's own timeline of one more call: on the last tile two write-backs, behind two reduces of two
+                # fetched strips of C when there is a beta
+                bC.set(start)
+                L.PARALiA_trace_enable(1)
+                call_gemm(pkg, L, dtype, ta, tb, M, N, K, 2.0, beta, bA, ra, bB, rb, bC, M, T=T)
+                n = int(L.PARALiA_trace_read(None, 0))
+                buf = (C.c_double * (7 * n))()
+                L.PARALiA_trace_read(buf, n)
+                L.PARALiA_trace_enable(0)
+                last = [int(buf[7 * i]) for i in range(n) if (int(buf[7 * i + 1]), int(buf[7 * i + 2])) == (1, 1)]
+                assert (last.count(2), last.count(4), last.count(5)) == ((0, 0, 2) if beta == 0.0 else (2, 2, 2))
+                assert last.count(3) == (2 if order % 160000 >= 80000 else k_tiles(info, K) + 1)
+                assert np.array_equal(bC.get(), ref)
+
+
 def test_sgemm_autotuned_call_merges_k_chains(pkg, L, orc, openblas):
     """No pin: for fp32 with A and B on the host the planner is offered the merged variants and its simulator takes
     one when the product is bound by compute and the chains are long (12288 x 12288 x 16384 here); parity against

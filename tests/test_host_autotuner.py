@@ -112,7 +112,7 @@ def test_autotune_selectors(L, pkg, monkeypatch):
     assert info.T in (512, 1024, 2048, 4096)
     # a thin start (order id 160000 * s + ...) cuts the first k tile into 2, 4 or (s = 3, graded) 4 slabs, each a k tile of its own
     g = 8192 // info.T
-    assert info.subkernel_num == g * g * (g + (1, 2, 4, 4)[info.order_id // 160000] - 1)
+    assert info.subkernel_num == g * g * (g + (1, 2, 4, 4)[info.order_id % 640000 // 160000] - 1)
     assert info.pred_t > 0 and info.pipe_exec <= info.pred_t * 1.0000001
     # the pick is the argmin over the table of the simulated pipeline time, near-ties broken by the reference's
     # penalty terms: score = pred_t * (1 + 0.02 * T_aggregate_sl)
@@ -135,7 +135,7 @@ def test_autotune_selectors(L, pkg, monkeypatch):
     monkeypatch.setenv("PARALIA_T_SELECT", "heuristic")
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 16384, 16384, 16384, b"N", b"N", HOST3, 1, -1, 0, C.byref(info)) == 0
     assert info.selected_by == b"heuristic" and info.T == 2048 and info.slowdowns[0] == 0.00390625
-    assert info.subkernel_num == 64 * (8 + (1, 2, 4, 4)[info.order_id // 160000] - 1)
+    assert info.subkernel_num == 64 * (8 + (1, 2, 4, 4)[info.order_id % 640000 // 160000] - 1)
     # everything resident: nothing to tile
     monkeypatch.delenv("PARALIA_T_SELECT")
     assert L.PARALiA_autotune(DB_SYNTH, b"Dgemm", 4096, 2048, 1024, b"N", b"N", loc3(0, 0, 0), 0, -1, 0, C.byref(info)) == 0

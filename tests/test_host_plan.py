@@ -82,7 +82,15 @@ def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks, slabs=1):
         elif k == FETCH_B:
             blocks[r["block"]] = ("B", r["ki"], r["ni"], B[sl(r["ki"], K_AXIS), sl(r["ni"], N)].copy())
         elif k == FETCH_C:
-            blocks[r["block"]] = ("S", r["mi"], r["ni"], C[sl(r["mi"], M), sl(r["ni"], N)].copy())
+            src = C[sl(r["mi"], M), sl(r["ni"], N)]
+            if r.get("rows", 0) > 0:
+                # a row strip of the caller's tile into those rows of the block
+                if blocks[r["block"]] is None or blocks[r["block"]][:3] != ("S", r["mi"], r["ni"]):
+                    blocks[r["block"]] = ("S", r["mi"], r["ni"], np.full(src.shape, np.nan))
+                rs = slice(r["row0"], r["row0"] + r["rows"])
+                blocks[r["block"]][3][rs] = src[rs]
+            else:
+                blocks[r["block"]] = ("S", r["mi"], r["ni"], src.copy())
         elif k == GEMM:
             if r["a_block"] >= 0:
                 tag, i, j, a = blocks[r["a_block"]]
@@ -94,6 +102,16 @@ def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks, slabs=1):
                 assert (tag, i, j) == ("B", r["ki"], r["ni"])
             else:
                 b = B[sl(r["ki"], K_AXIS), sl(r["ni"], N)]
+            if r.get("rows", 0) > 0:
+                # a row strip of the tile (order ids of 640000 and above): those rows of the accumulator only
+                assert r["block"] >= 0 and 0 <= r["row0"] and r["row0"] + r["rows"] <= a.shape[0]
+                rs = slice(r["row0"], r["row0"] + r["rows"])
+                prod = alpha * (a[rs] @ b)
+                if blocks[r["block"]] is None or blocks[r["block"]][:3] != ("ACC", r["mi"], r["ni"]):
+                    blocks[r["block"]] = ("ACC", r["mi"], r["ni"], np.full((a.shape[0], b.shape[1]), np.nan))
+                acc = blocks[r["block"]][3]
+                acc[rs] = prod if r["beta_mode"] == BETA_ZERO else acc[rs] + prod
+                continue
             prod = alpha * (a @ b)
             if r["block"] >= 0:
                 if r["beta_mode"] == BETA_ZERO:
@@ -109,22 +127,34 @@ def replay(rows, M, N, K, T, alpha, beta, A, B, C, pool_blocks, slabs=1):
             tag, i, j, acc = blocks[r["block"]]
             stag, si, sj, src = blocks[r["a_block"]]
             assert (tag, i, j) == ("ACC", r["mi"], r["ni"]) and (stag, si, sj) == ("S", r["mi"], r["ni"])
-            blocks[r["block"]] = ("ACC", i, j, beta * src + acc)
+            if r.get("rows", 0) > 0:
+                rs = slice(r["row0"], r["row0"] + r["rows"])
+                acc[rs] = beta * src[rs] + acc[rs]
+            else:
+                blocks[r["block"]] = ("ACC", i, j, beta * src + acc)
         elif k == WRITEBACK:
             tag, i, j, acc = blocks[r["block"]]
             assert (tag, i, j) == ("ACC", r["mi"], r["ni"])
-            out[sl(r["mi"], M), sl(r["ni"], N)] = acc
+            if r.get("rows", 0) > 0:
+                rs = slice(r["row0"], r["row0"] + r["rows"])
+                out[sl(r["mi"], M), sl(r["ni"], N)][rs] = acc[rs]
+            else:
+                out[sl(r["mi"], M), sl(r["ni"], N)] = acc
     return out
 
 
 def check_async_safety(rows):
     """Every data hazard on a pool block is ordered by stream order plus the recorded waits (transitively): a reader
     runs after the command that produced what it reads, and a command that overwrites a block runs after every
-    earlier reader and writer of that block.  Happens-before sets are bit masks."""
+    earlier reader and writer of that block.  Commands on a row strip of a C tile touch those rows of the accumulator
+    block only; hazards are between commands whose rows overlap.  Happens-before sets are bit masks."""
+    whole = (0, 1 << 30)
+    span = lambda r: (r["row0"], r["row0"] + r["rows"]) if r.get("rows", 0) > 0 else whole
+    overlap = lambda a, b: a[0] < b[1] and b[0] < a[1]
     before = [0] * len(rows)
     last_on_stream = {}
-    last_write = {}   # block -> command that last wrote it
-    users = {}        # block -> commands that read it since
+    last_write = {}   # block -> [(rows, command that last wrote them)]
+    users = {}        # block -> [(rows, command that read them since)]
     for i, r in enumerate(rows):
         deps = 0
         if r["stream"] in last_on_stream:
@@ -137,30 +167,34 @@ def check_async_safety(rows):
         k = r["kind"]
         reads, writes = [], []
         if k in (FETCH_A, FETCH_B, FETCH_C):
-            writes = [r["block"]]
+            writes = [(r["block"], span(r))]
         elif k == GEMM:
-            reads = [x for x in (r["a_block"], r["b_block"]) if x >= 0]
+            reads = [(x, whole) for x in (r["a_block"], r["b_block"]) if x >= 0]
             if r["block"] >= 0:
-                (writes if r["beta_mode"] == BETA_ZERO else reads).append(r["block"])
+                (writes if r["beta_mode"] == BETA_ZERO else reads).append((r["block"], span(r)))
                 if r["beta_mode"] != BETA_ZERO:
-                    writes.append(r["block"])
+                    writes.append((r["block"], span(r)))
         elif k == REDUCE:
-            reads = [r["block"], r["a_block"]]
-            writes = [r["block"]]
+            reads = [(r["block"], span(r)), (r["a_block"], span(r))]
+            writes = [(r["block"], span(r))]
         elif k == WRITEBACK:
-            reads = [r["block"]]
-        for blk in reads:
-            w = last_write.get(blk)
-            assert w is not None, "cmd %d reads block %d that nothing wrote" % (i, blk)
-            assert w == i or (deps >> w) & 1, "cmd %d reads block %d before its writer %d is known to be done" % (i, blk, w)
-        for blk in writes:
-            for u in users.get(blk, []) + ([last_write[blk]] if blk in last_write else []):
-                assert u == i or (deps >> u) & 1, "block %d overwritten by cmd %d before cmd %d is known to be done" % (blk, i, u)
-        for blk in reads:
-            users.setdefault(blk, []).append(i)
-        for blk in writes:
-            last_write[blk] = i
-            users[blk] = []
+            reads = [(r["block"], span(r))]
+        for blk, sp in reads:
+            ws = [w for wsp, w in last_write.get(blk, []) if overlap(wsp, sp)]
+            assert ws, "cmd %d reads block %d that nothing wrote" % (i, blk)
+            for w in ws:
+                assert w == i or (deps >> w) & 1, "cmd %d reads block %d before its writer %d is known to be done" % (i, blk, w)
+        for blk, sp in writes:
+            for usp, u in users.get(blk, []) + last_write.get(blk, []):
+                if overlap(usp, sp):
+                    assert u == i or (deps >> u) & 1, "block %d overwritten by cmd %d before cmd %d is known to be done" % (blk, i, u)
+        for blk, sp in reads:
+            users.setdefault(blk, []).append((sp, i))
+        for blk, sp in writes:
+            # (what the new rows cover completely is superseded; a tile-wide entry stays beside a strip's)
+            inside = lambda e: sp[0] <= e[0][0] and e[0][1] <= sp[1]
+            last_write[blk] = [e for e in last_write.get(blk, []) if not inside(e)] + [(sp, i)]
+            users[blk] = [e for e in users.get(blk, []) if not inside(e)]
 
 
 ORDERS = [10000, 0, 1, 3, 10002, 10004, 20002, 30001, 50000, 60002, 102, 201, 202, 10201, 10999]
@@ -470,6 +504,63 @@ def test_thin_start_plans(pkg, order, locs, beta_zero):
         pkg.plan_rows(M, N, 20, 32, a_r, b_r, c_r, beta_zero, 8, 2, 0, order)     # K < T: nothing to cut
 
 
+@pytest.mark.parametrize("order", [640000, 650002, 720000, 720002, 730001, 880001, 720203, 660003, 700001])
+@pytest.mark.parametrize("locs", [(1, 1, 1), (0, 1, 1), (1, 0, 1)])
+@pytest.mark.parametrize("beta_zero", [1, 0])
+def test_strip_end_plans(pkg, order, locs, beta_zero):
+    """Order ids of 640000 and above: the last launch of the call -- the last k-step of the C tile the order completes
+    last, or that tile's whole merged K chain -- is made in row strips, each a launch of its own over the same k range
+    that says how many ways it splits K, and what follows on the tile comes strip by strip as well: with beta != 0 the
+    fetch of the caller's C and the lazy reduce, then the write-back.  Everything before that launch is the plan of
+    the id without the flag; the strips cover the tile's rows once; the plan replays to the exact result and orders
+    every hazard, strips against strips by their rows (with a pool smaller than the working set too: 660003, 700001).
+    Where the flag does not apply (C on the device, a last tile under 512 rows) the plan is that of the plain id."""
+    a_r, b_r, c_r = locs
+    M, N, K, T = 1300, 1100, 1200, 512                              # last tile 276 x 76: nothing to cut
+    pool = 14 if order % 80000 >= 20000 else 0
+    plain_id = order - 640000
+    assert pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, pool, order)[0] == pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, pool, plain_id)[0]
+    M = 1536                                                        # last tile 512 x 76 -> strips of 256 rows
+    if order % 10000 == 203:
+        M, N = 2048, 1636                                           # the block order ends on tile (3, 3): 512 x 100
+    assert pkg.plan_rows(M, N, K, T, a_r, b_r, 0, beta_zero, 8, 2, pool, order)[0] == pkg.plan_rows(M, N, K, T, a_r, b_r, 0, beta_zero, 8, 2, pool, plain_id)[0]
+    slabs = 1 << (plain_id // 160000)
+    merged = plain_id % 160000 >= 80000
+    Mg, Ng, Kg = grids(M, N, K, T, slabs)
+    plain, _ = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, pool, plain_id)
+    rows, stats = pkg.plan_rows(M, N, K, T, a_r, b_r, c_r, beta_zero, 8, 2, pool, order)
+    at = max(i for i, r in enumerate(plain) if r["kind"] == GEMM)
+    last = plain[at]
+    assert last["kn"] == (Kg if merged else 1) and last["ki"] + last["kn"] == Kg
+    assert [r["kind"] for r in plain[at:]] == ([GEMM, WRITEBACK] if beta_zero else [GEMM, FETCH_C, REDUCE, WRITEBACK])
+    assert rows[:at] == plain[:at] and all(r["rows"] == 0 and r["splits"] == 0 for r in rows[:at])
+    tail = rows[at:]
+    tm, tn = M - last["mi"] * T, N - last["ni"] * T
+    assert tm == 512 and len(tail) == (4 if beta_zero else 8)       # two strips of 256 rows
+    kinds = [GEMM, WRITEBACK] if beta_zero else [GEMM, FETCH_C, REDUCE, WRITEBACK]
+    assert [r["kind"] for r in tail] == [k for k in kinds for _ in range(2)]
+    launch_k = K if merged else K - (K // T) * T
+    for i, r in enumerate(tail):
+        assert (r["mi"], r["ni"]) == (last["mi"], last["ni"]) and (r["row0"], r["rows"]) == (256 * (i % 2), 256)
+        if r["kind"] == GEMM:
+            assert (r["ki"], r["kn"], r["beta_mode"], r["stream"], r["block"]) == (last["ki"], last["kn"], last["beta_mode"], last["stream"], last["block"])
+            assert (r["a_block"], r["b_block"]) == (last["a_block"], last["b_block"])
+            assert r["splits"] == max(1, min(-(-512 // (2 * -(-tn // 128))), launch_k // 512)) == (2 if merged else 1)
+        elif r["kind"] == WRITEBACK:
+            assert r["block"] == last["block"] and r["waits"] == [at + (4 if not beta_zero else 0) + i % 2]
+        elif r["kind"] == REDUCE:
+            assert r["block"] == last["block"] and r["stream"] == last["stream"] and at + 2 + i % 2 in r["waits"]
+    flat = expand_merged(rows)
+    full = pool if pool else 1 + Mg * Kg + Kg * Ng + 2 * Mg * Ng
+    rng = np.random.default_rng(order)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64)
+    B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C = rng.integers(-5, 6, (M, N)).astype(np.float64)
+    beta = 0.0 if beta_zero else 3.0
+    assert np.array_equal(replay(flat, M, N, K, T, 2.0, beta, A, B, C, full, slabs), 2.0 * (A @ B) + beta * C)
+    check_async_safety(flat)
+
+
 def test_block_orders(pkg):
     """w = rows * 100 + columns: that block of C tiles is the k-outer panel (walked in growing squares in every k-step),
     the rest follows tile by tile with the K chain innermost -- for orient 0 the other rows of the block's columns, then
@@ -534,6 +625,6 @@ def test_whole_grid_panel_on_grids_of_a_hundred_tiles_and_more(pkg, L):
 
 
 def test_unknown_order_ids_are_refused(pkg):
-    for order in (640000, 800001, -5):
+    for order in (1280000, 1440001, -5):
         with pytest.raises(pkg.ParaliaError, match="unknown order id"):
             pkg.plan_rows(256, 256, 256, 64, 1, 1, 1, 0, 8, 2, 0, order)
