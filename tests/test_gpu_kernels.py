@@ -508,6 +508,47 @@ def test_dgemm_tile_split_k_vs_openblas(pkg, L, orc, openblas, ta, tb, dims):
     assert np.array_equal(got, again)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims,splits", [((512, 700, 4096), 8), ((512, 700, 4096), 3), ((384, 76, 1201), 2), ((1024, 1024, 700), 5),
+                                         ((2048, 2048, 600), 2), ((200, 300, 100), 4), ((256, 256, 2048), 1)])
+def test_gemm_tile_with_the_callers_split_count(pkg, L, ta, tb, dims, splits):
+    """pl_dgemm_tile_split / pl_sgemm_tile_split: K goes to the number of workgroups per tile the caller names, also for
+    shapes the launcher's own model would not split (2048 x 2048 tiles fill the device), in whole panels per chunk with
+    a ragged last chunk, with beta = 0 over NaN and beta != 0, padded leading dimensions; a count of 1, a K too short
+    for two chunks, or a workspace under splits * M * N elements run the unsplit kernel; a count below 1 is refused.
+    Integer operands (sums far below 2^24): bit for bit numpy's fp64 product, whichever way K is cut."""
+    M, N, K = dims
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 8, M + 4
+    rng = np.random.default_rng(M + N + K + splits)
+    for dtype in (np.float64, np.float32):
+        esz = np.dtype(dtype).itemsize
+        fn = L.pl_dgemm_tile_split if dtype == np.float64 else L.pl_sgemm_tile_split
+        A = rng.integers(-4, 5, lda * ca).astype(dtype)
+        B = rng.integers(-4, 5, ldb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, ldc * N).astype(dtype)
+        a = A.reshape(ca, lda)[:, :ra].T.astype(np.float64)        # the column-major operands as matrices
+        b = B.reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+        prod = 3.0 * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T))
+        dA, dB = Buf(pkg, A.size, dtype, 0).set(A), Buf(pkg, B.size, dtype, 0).set(B)
+        for beta, ws_slices in ((0.0, splits), (-2.0, splits), (0.0, splits - 1)):
+            n_ws = max(1, ws_slices * M * N)
+            dW = Buf(pkg, n_ws, dtype, 0).set(np.full(n_ws, np.nan, dtype=dtype))
+            start = np.full(ldc * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+            dC = Buf(pkg, start.size, dtype, 0).set(start)
+            ref = (prod + beta * C0.reshape(N, ldc)[:, :M].T.astype(np.float64)).T.astype(dtype)
+            print("gemm_split", np.dtype(dtype).name, ta, tb, M, N, K, "splits", splits, "workspace slices", ws_slices, "beta", beta, flush=True)
+            pkg.check(fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, beta, dC.ptr, ldc, dW.ptr, n_ws * esz, splits, None), "gemm tile split")
+            sync(pkg)
+            got = dC.get().reshape(N, ldc)
+            assert np.array_equal(got[:, :M], ref), (np.dtype(dtype).name, beta, ws_slices)
+            if beta != 0.0:
+                assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])      # the padding of C is never written
+        assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, ldc, dW.ptr, n_ws * esz, 0, None) == 7      # PL_ERR_ARG, refused before any launch
+        sync(pkg)
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N")])
 def test_gemm_tile_split_k_exact_and_fallback(pkg, L, orc, ta, tb):
     """Integer-valued data: the split result equals the unsplit one bit for bit, for fp64 and fp32; beta = 0 with a
