@@ -35,6 +35,7 @@ int main(int argc, char** argv) {
         int id = orient * 10000 + w + ((w > 0 && rng() % 2) ? 20000 : 0) + ((rng() % 2) ? 40000 : 0);
         if (rng() % 3 == 0) id = ORDER_MERGE_CHAINS + orient * 10000 + w;  // merged K chains (refused unless the pool holds everything)
         if (rng() % 3 == 0) id += ORDER_K_SPLIT * (1 + rng() % 3);  // thin start: first k tile in 2 or 4 equal slabs or graded (refused when it does not apply)
+        if (rng() % 3 == 0) id += ORDER_STRIP_END;  // the last launch in row strips (the same plan where the last tile is too small or stays on the device)
         GemmPlan plan = build_gemm_plan(p, id);
         PipelineResult r = simulate_plan(plan, st);
         if (!(r.t_total >= 0)) { printf("bad makespan\n"); return 1; }
