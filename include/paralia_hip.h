@@ -106,7 +106,7 @@ int pl_sgemm_tile_ws(char transA, char transB, long M, long N, long K, float alp
 
 /* The same again with the caller's split count instead of the model's: K goes to `splits` workgroups per tile of C (in
  * whole panels, so the count used may be lower; 1, or a workspace under splits * M * N elements, launches the unsplit
- * kernel).  For a scheduler that knows a product will have the device to itself, where the model above assumes a
+ * kernel; a count below 1 is PL_ERR_ARG).  For a scheduler that knows a product will have the device to itself, where the model above assumes a
  * second product running beside it (the end of a call: the reference's last subkernels of Subkernel.cpp:168 run alone
  * on their queue). */
 int pl_dgemm_tile_split(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
@@ -115,6 +115,22 @@ int pl_dgemm_tile_split(char transA, char transB, long M, long N, long K, double
 int pl_sgemm_tile_split(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
                         const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
                         int splits, void* stream);
+
+/* The product for a caller who knows it has the device to itself (every operand already in HBM and nothing else
+ * running: the reference's call with all data on the GPU is one cublasDgemm, dgemm.cpp:382-395 with a single
+ * subkernel).  The launcher then counts whole rounds of two workgroups per compute unit instead of assuming a second
+ * product beside this one, and splits K where that fills the last round (a 3072 x 3072 x 16384 product: 576 tiles, 52.7
+ * TFLOP/s unsplit, 73.7 split four ways).  pl_gemm_tile_alone_workspace_bytes: what that choice can use (at most 1 GiB;
+ * 0: not split); pl_gemm_tile_choice_alone reports the choice like pl_gemm_tile_choice. */
+long pl_gemm_tile_alone_workspace_bytes(char transA, char transB, long M, long N, long K, int beta_is_zero, int elem_size);
+int pl_dgemm_tile_alone(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                        const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
+                        void* stream);
+int pl_sgemm_tile_alone(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                        const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
+                        void* stream);
+int pl_gemm_tile_choice_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
+                              long workspace_bytes, int* tile_m, int* tile_n, int* splits);
 
 /* Fitted constants of the tile-GEMM launcher's cost model: how it chooses between its macro tiles (fp32: 128 x 128,
  * 256 x 128 "wide", 256 x 256 "large") and how many ways it splits K for products with few tiles.  They describe one

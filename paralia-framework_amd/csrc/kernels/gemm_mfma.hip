@@ -897,18 +897,65 @@ int pick_splits(long M, long N, long K, int* kchunk_out) {
   return best_s;
 }
 
+// The same choice for a product that has the device to itself (a caller's device-resident call, the end of a streamed
+// one).  Nothing else fills the compute units a launch leaves idle, so what counts is whole rounds of 512 workgroups (two
+// per compute unit): 576 tiles are one full round and an eighth of another that takes as long (3072 x 3072 x 16384 fp64
+// alone: 52.7 TFLOP/s unsplit, 73.7 split four ways = 4.5 rounds), 256 tiles leave every unit with one workgroup (2048
+// x 2048 x 16384: 65.8 unsplit, 72.6 split two to four ways).  A round of 512 takes f + kc * c2, a last round of at most
+// 256 workgroups (one per unit) f + kc * c1, with c1 the lone per-k time of the fit, c2 / c1 as measured on the fp32 tile
+// (f32_small_us_per_k / lone_us_per_k[1]) and f the workgroup's fixed cost (lone_fixed_k); a split adds the second launch
+// and the reduction's pass over the slices and C (the slices' way out of the workgroups is part of their epilogue, as the
+// write of C is).  *us_out: the predicted time of the choice.
+template <typename T>
+int pick_splits_alone(long M, long N, long K, long max_ws_bytes, int* kchunk_out, double* us_out) {
+  constexpr int BM = 128, BN = 128;
+  const long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const pl_gemm_fit& fit = fit_in_use();
+  const double c1 = fit.lone_us_per_k[sizeof(T) == 8 ? 0 : 1];
+  const double c2 = c1 * fit.f32_small_us_per_k / fit.lone_us_per_k[1];
+  const double f = fit.lone_fixed_k * c1;
+  auto main_us = [&](long blocks, long kc) {
+    const long full = blocks / 512, rem = blocks % 512;
+    double t = (double)full * (f + (double)kc * c2);
+    if (rem > 0) t += f + (double)kc * (rem <= 256 ? c1 : c2);
+    return t;
+  };
+  *kchunk_out = 0;
+  double best = main_us(tiles, K);
+  int best_s = 1;
+  const long gran = sizeof(T) == 4 ? PLK_F32_DEEP_BK : 16;
+  for (int s = 2; s <= 64 && K >= 256; ++s) {
+    const long kc = (((K + s - 1) / s) + gran - 1) / gran * gran;
+    if (kc < 128) break;
+    const long se = (K + kc - 1) / kc;
+    if (se < 2) continue;
+    if (se * M * N * (long)sizeof(T) > max_ws_bytes) break;
+    const double t = main_us(tiles * se, kc) + fit.splitk_launch_us + ((double)se + 1.0) * (double)M * (double)N * sizeof(T) / fit.pass_bytes_per_us;
+    if (t < best * 0.97) {
+      best = t;
+      best_s = (int)se;
+      *kchunk_out = (int)kc;
+    }
+  }
+  if (us_out) *us_out = best;
+  return best_s;
+}
+
 // Macro tile and split count of one product.
 struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; };
 template <typename T>
 TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true,
-                       int want_splits = 0) {
+                       int want_splits = 0, bool alone = false) {
   TileChoice c;
-  if (want_splits > 1 && have_ws) {
-    // the caller's split count, in whole panels per chunk like the model's own
+  double alone_us = -1;   // alone: the predicted time of the 128 x 128 tile with the split count chosen for it
+  if (want_splits >= 1) {
+    // the caller's split count (1: unsplit), in whole panels per chunk like the model's own
     const long gran = sizeof(T) == 4 ? PLK_F32_DEEP_BK : 16;
     const long kc = (((K + want_splits - 1) / want_splits) + gran - 1) / gran * gran;
     const long se = (K + kc - 1) / kc;
-    if (se > 1) c.splits = (int)se, c.kchunk = (int)kc;
+    if (se > 1 && have_ws && want_splits > 1) c.splits = (int)se, c.kchunk = (int)kc;
+  } else if (alone) {
+    c.splits = pick_splits_alone<T>(M, N, K, have_ws ? workspace_bytes : 0, &c.kchunk, &alone_us);
   } else {
     c.splits = have_ws ? pick_splits<T>(M, N, K, &c.kchunk) : 1;
   }
@@ -933,20 +980,22 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   const int bi = beta_zero ? 0 : 1;
   auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
   const double k_us = fit.f32_small_us_per_k * (double)K;
-  const double small_us = (double)((tiles_of(128, 128) + 511) / 512) * (fit.f32_small_fixed_us + k_us);
+  const double small_us = alone_us >= 0 ? alone_us : (double)((tiles_of(128, 128) + 511) / 512) * (fit.f32_small_fixed_us + k_us);
   const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * (fit.f32_large_fixed_us[tr][bi] + 2.0 * k_us / (1.0 + fit.f32_large_gain[tr]));
   const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (fit.f32_wide_fixed_us[bi] + 2.0 * k_us / fit.f32_wide_gain);
   // PARALIA_GEMM_LARGE_TILE: "0" small tiles only, "1" the large tile for every call, "2" the wide tile wherever it
   // exists (NN), unset: the model
   const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");
   const int pinv = (pin && *pin) ? atoi(pin) : -1;
-  const bool other = sizeof(T) == 4 && c.splits == 1 && pinv != 0;
+  // (alone, the bigger tiles are weighed against the split small tile too; a caller's own split count keeps the small one)
+  const bool other = sizeof(T) == 4 && (c.splits == 1 || alone_us >= 0) && pinv != 0;
   // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
   auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
   const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
   const bool big_ok = other && large_allowed && (pinv == 1 || (pinv < 0 && fills(tiles_of(256, 256), 256)));
   c.big = big_ok && (pinv == 1 || (large_us < small_us && (!wide_ok || large_us <= wide_us)));
   c.wide = !c.big && wide_ok && (pinv == 2 || wide_us < small_us);
+  if (c.big || c.wide) c.splits = 1, c.kchunk = 0;
   c.tm = c.big || c.wide ? 256 : 128;
   c.tn = c.big ? 256 : 128;
   return c;
@@ -954,7 +1003,8 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
 
 template <typename T>
 int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
-                T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0, int want_splits = 0) {
+                T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0, int want_splits = 0,
+                bool alone = false) {
   using Tr = Traits<T>;
   const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
   const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
@@ -975,7 +1025,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   // a K-major operand loaded straight into LDS takes eight rows per request with 32-bit lane offsets: leading dimensions
   // beyond that keep the tiles that stage through registers
   const bool dma_fits = (!at || lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES) && (!bnn || ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES);
-  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits);
+  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits, alone);
   const int kchunk = choice.kchunk, splits = choice.splits;
   const bool big = choice.big, wide = choice.wide;
   const int TM_RT = choice.tm, TN_RT = choice.tn;
@@ -1101,6 +1151,43 @@ extern "C" int pl_sgemm_tile_split(char transA, char transB, long M, long N, lon
   if (splits < 1) return PL_ERR_ARG;
   return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
                                  (float*)workspace, workspace_bytes, splits);
+}
+
+// workspace a product alone on the device is given at most (the slices of its split)
+#define PLK_ALONE_MAX_WS_BYTES (1L << 30)
+
+extern "C" int pl_dgemm_tile_alone(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                                   const double* B, long ldb, double beta, double* C, long ldc, void* workspace,
+                                   long workspace_bytes, void* stream) {
+  return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                  (double*)workspace, workspace_bytes, 0, true);
+}
+
+extern "C" int pl_sgemm_tile_alone(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                                   const float* B, long ldb, float beta, float* C, long ldc, void* workspace,
+                                   long workspace_bytes, void* stream) {
+  return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                 (float*)workspace, workspace_bytes, 0, true);
+}
+
+extern "C" int pl_gemm_tile_choice_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
+                                         long workspace_bytes, int* tile_m, int* tile_n, int* splits) {
+  const bool at = (transA == 'T' || transA == 't'), an = (transA == 'N' || transA == 'n');
+  const bool bt = (transB == 'T' || transB == 't'), bnn = (transB == 'N' || transB == 'n');
+  if (!(at || an) || !(bt || bnn)) return PL_ERR_TRANS;
+  if (M <= 0 || N <= 0 || K <= 0 || (elem_size != 8 && elem_size != 4)) return PL_ERR_DIM;
+  const plk::TileChoice c = elem_size == 8 ? plk::choose_tile<double>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true)
+                                           : plk::choose_tile<float>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true);
+  if (tile_m) *tile_m = c.tm;
+  if (tile_n) *tile_n = c.tn;
+  if (splits) *splits = c.splits;
+  return 0;
+}
+
+extern "C" long pl_gemm_tile_alone_workspace_bytes(char transA, char transB, long M, long N, long K, int beta_is_zero, int elem_size) {
+  int splits = 1;
+  if (pl_gemm_tile_choice_alone(elem_size, transA, transB, M, N, K, beta_is_zero, PLK_ALONE_MAX_WS_BYTES, nullptr, nullptr, &splits) != 0) return 0;
+  return splits > 1 ? (long)splits * M * N * elem_size : 0;
 }
 
 extern "C" int pl_dgemm_tile_ws(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,

@@ -295,6 +295,10 @@ template <> struct GemmFns<double> {
                   double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_dgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
   }
+  static int tile_alone(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
+                        double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
+    return pl_dgemm_tile_alone(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
   static int tile_split(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
                         double be, double* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
     return pl_dgemm_tile_split(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, s);
@@ -308,6 +312,10 @@ template <> struct GemmFns<float> {
   static int tile(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                   float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_sgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
+  static int tile_alone(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
+                        float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
+    return pl_sgemm_tile_alone(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
   }
   static int tile_split(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                         float be, float* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
@@ -595,11 +603,11 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   ATC* atc = entry->atc.get();
   const bool any_remote = key.loc[0] < 0 || key.loc[1] < 0 || key.loc[2] < 0;
   if (!any_remote) {
-    // Every operand already in HBM: one launch over the caller's matrices.
+    // Every operand already in HBM: one launch over the caller's matrices, alone on the device.
     R.res.ensure_streams(1);
-    const long ws_bytes = no_ab ? 0 : pl_gemm_tile_workspace_bytes(M, N, K, (int)sizeof(T));
+    const long ws_bytes = no_ab ? 0 : pl_gemm_tile_alone_workspace_bytes(ta, tb, M, N, K, beta == T(0) ? 1 : 0, (int)sizeof(T));
     void* ws = ws_bytes > 0 ? R.res.gemm_ws[0].ensure(ws_bytes) : nullptr;
-    chk(GemmFns<T>::tile(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, ws, ws_bytes, R.res.exec[0]), "gemm launch");
+    chk(GemmFns<T>::tile_alone(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, ws, ws_bytes, R.res.exec[0]), "gemm launch");
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;

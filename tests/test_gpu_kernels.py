@@ -549,6 +549,45 @@ def test_gemm_tile_with_the_callers_split_count(pkg, L, ta, tb, dims, splits):
         sync(pkg)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(2560, 2560, 4096), (3072, 1400, 2048), (1537, 1500, 1100), (600, 500, 700), (2560, 2560, 1200)])
+def test_gemm_tile_alone_on_the_device(pkg, L, ta, tb, dims):
+    """pl_dgemm_tile_alone / pl_sgemm_tile_alone: the launcher's choice for a product that has the device to itself (K
+    split so that whole rounds of workgroups are filled: every shape here but the last, whose K is too short to pay),
+    with the workspace it asks for, with none (unsplit), beta = 0 over NaN and beta != 0, ragged edges.  Integer operands: bit for bit numpy's
+    fp64 product."""
+    M, N, K = dims
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 8, M + 4
+    rng = np.random.default_rng(M + N + K)
+    for dtype in (np.float64, np.float32):
+        esz = np.dtype(dtype).itemsize
+        fn = L.pl_dgemm_tile_alone if dtype == np.float64 else L.pl_sgemm_tile_alone
+        A = rng.integers(-4, 5, lda * ca).astype(dtype)
+        B = rng.integers(-4, 5, ldb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, ldc * N).astype(dtype)
+        a = A.reshape(ca, lda)[:, :ra].T.astype(np.float64)
+        b = B.reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+        prod = -2.0 * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T))
+        dA, dB = Buf(pkg, A.size, dtype, 0).set(A), Buf(pkg, B.size, dtype, 0).set(B)
+        for beta in (0.0, 3.0):
+            need = int(L.pl_gemm_tile_alone_workspace_bytes(ta.encode(), tb.encode(), M, N, K, 1 if beta == 0.0 else 0, esz))
+            tm, tn, sp = C.c_int(), C.c_int(), C.c_int()
+            assert L.pl_gemm_tile_choice_alone(esz, ta.encode(), tb.encode(), M, N, K, 1 if beta == 0.0 else 0, need, C.byref(tm), C.byref(tn), C.byref(sp)) == 0
+            assert need == (sp.value * M * N * esz if sp.value > 1 else 0) and (sp.value > 1) == (K != 1200)
+            for ws_bytes in (need, 0):
+                n_ws = max(1, ws_bytes // esz)
+                dW = Buf(pkg, n_ws, dtype, 0).set(np.full(n_ws, np.nan, dtype=dtype))
+                start = np.full(ldc * N, np.nan, dtype=dtype) if beta == 0.0 else C0
+                dC = Buf(pkg, start.size, dtype, 0).set(start)
+                ref = (prod + beta * C0.reshape(N, ldc)[:, :M].T.astype(np.float64)).T.astype(dtype)
+                print("gemm_alone", np.dtype(dtype).name, ta, tb, M, N, K, "splits", sp.value, "workspace", ws_bytes, "beta", beta, flush=True)
+                pkg.check(fn(ta.encode(), tb.encode(), M, N, K, -2.0, dA.ptr, lda, dB.ptr, ldb, beta, dC.ptr, ldc, dW.ptr if ws_bytes else None, ws_bytes, None), "gemm tile alone")
+                sync(pkg)
+                assert np.array_equal(dC.get().reshape(N, ldc)[:, :M], ref), (np.dtype(dtype).name, beta, ws_bytes)
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N")])
 def test_gemm_tile_split_k_exact_and_fallback(pkg, L, orc, ta, tb):
     """Integer-valued data: the split result equals the unsplit one bit for bit, for fp64 and fp32; beta = 0 with a

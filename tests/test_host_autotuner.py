@@ -474,3 +474,47 @@ def test_kernel_fit_file_is_optional_and_drives_launcher_and_simulator(L, pkg, t
     assert info.has_db == 0 and info.selected_by == b"heuristic"
     assert L.pl_gemm_set_fit(None) == 0                                         # back to the built-in values for the tests that follow
     L.PARALiA_set_db_dir(None)
+
+
+def test_launcher_choice_for_a_product_alone_on_the_device(L, pkg, monkeypatch):
+    """pl_gemm_tile_choice_alone: the split count (and, for fp32, the macro tile) of a product that has the device to
+    itself.  Whole rounds of 512 workgroups decide: 576 tiles (3072^2) are split so that the last round is filled,
+    1024 tiles (4096^2: two rounds) and 256 large fp32 tiles (one round) are not, a short K is not, tiny products are
+    split as the two-stream model splits them; the workspace figure is the slices of that choice, never above 1 GiB; a
+    workspace too small for any split leaves the product unsplit; a fit that prices a split at a tenth of a second
+    splits nothing."""
+    from paralia_framework_amd import binding
+    monkeypatch.delenv("PARALIA_GEMM_LARGE_TILE", raising=False)
+    assert L.pl_gemm_set_fit(None) == 0
+
+    def alone(es, tr, M, N, K, beta0=1, ws=1 << 30):
+        tm, tn, sp = C.c_int(), C.c_int(), C.c_int()
+        assert L.pl_gemm_tile_choice_alone(es, tr[0:1], tr[1:2], M, N, K, beta0, ws, C.byref(tm), C.byref(tn), C.byref(sp)) == 0
+        return tm.value, tn.value, sp.value
+
+    def two_streams(es, tr, M, N, K, beta0=1, ws=1 << 30):
+        tm, tn, sp = C.c_int(), C.c_int(), C.c_int()
+        assert L.pl_gemm_tile_choice(es, tr[0:1], tr[1:2], M, N, K, beta0, ws, C.byref(tm), C.byref(tn), C.byref(sp)) == 0
+        return tm.value, tn.value, sp.value
+    for es in (8, 4):
+        assert two_streams(es, b"NN", 3072, 3072, 16384) [2] == 1               # a second product would fill the gaps
+        tm, tn, s = alone(es, b"NN", 3072, 3072, 16384)
+        assert (tm, tn) == (128, 128) and s in (4, 8)                            # 576 x 4 = 4.5 rounds, x 8 = 9
+        assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 3072, 3072, 16384, 1, es) == s * 3072 * 3072 * es
+        assert alone(es, b"TN", 2560, 2560, 4096)[2] >= 2                        # 400 tiles: most of a round idle
+        assert alone(es, b"NN", 3072, 3072, 256)[2] == 1                         # nothing to split
+        assert alone(es, b"NN", 3072, 3072, 16384, ws=3072 * 3072 * es)[2] == 1  # room for one slice only
+        assert alone(es, b"NN", 512, 512, 2048) == two_streams(es, b"NN", 512, 512, 2048)
+        assert alone(es, b"NN", 8192, 8192, 8192)[2] == 1 and L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 8192, 8192, 8192, 1, es) == 0
+        assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 6000, 6000, 16384, 1, es) <= 1 << 30
+    assert alone(8, b"NN", 4096, 4096, 16384) == (128, 128, 1)                   # two full rounds
+    assert alone(4, b"NT", 4096, 4096, 16384) == (256, 256, 1)                   # one round of large tiles
+    assert alone(4, b"NT", 4096, 4096, 16384, beta0=0)[2] == 1
+    assert L.pl_gemm_tile_choice_alone(8, b"X", b"N", 10, 10, 10, 1, 0, None, None, None) != 0
+    assert L.pl_gemm_tile_choice_alone(2, b"N", b"N", 10, 10, 10, 1, 0, None, None, None) != 0
+    f = binding.gemm_fit()
+    L.pl_gemm_fit_defaults(C.byref(f))
+    f.splitk_launch_us = 1e5
+    assert L.pl_gemm_set_fit(C.byref(f)) == 0
+    assert alone(8, b"NN", 3072, 3072, 16384)[2] == 1 and alone(4, b"NN", 2560, 2560, 4096)[2] == 1
+    assert L.pl_gemm_set_fit(None) == 0
