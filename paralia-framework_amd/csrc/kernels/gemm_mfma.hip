@@ -931,7 +931,7 @@ int pick_splits_alone(long M, long N, long K, long max_ws_bytes, int* kchunk_out
     if (se < 2) continue;
     if (se * M * N * (long)sizeof(T) > max_ws_bytes) break;
     const double t = main_us(tiles * se, kc) + fit.splitk_launch_us + ((double)se + 1.0) * (double)M * (double)N * sizeof(T) / fit.pass_bytes_per_us;
-    if (t < best * 0.97) {
+    if (t < best * 0.98) {
       best = t;
       best_s = (int)se;
       *kchunk_out = (int)kc;
