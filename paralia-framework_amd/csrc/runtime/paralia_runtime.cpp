@@ -174,6 +174,15 @@ struct Resources {
       cap = bytes;
       return p;
     }
+    // The same for memory the caller can do without: nullptr, and nothing attempted, unless the device has twice the
+    // room to spare (a caller whose matrices fill the device keeps what is left of it).
+    void* ensure_if_room(long long bytes) {
+      if (bytes <= cap) return p;
+      long long free_b = 0, total_b = 0;
+      chk(pl_mem_info(&free_b, &total_b), "mem info");
+      if (2 * (bytes - cap) > free_b) return nullptr;
+      return ensure(bytes);
+    }
     void release() { if (p) pl_free_device(p); p = nullptr; cap = 0; }
   } gemv_x, gemv_y, gemv_ws;
   // split-K workspaces of the tile GEMM, one per exec stream (launches on different streams may overlap)
@@ -605,9 +614,10 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
   if (!any_remote) {
     // Every operand already in HBM: one launch over the caller's matrices, alone on the device.
     R.res.ensure_streams(1);
+    // (the split-K slices are worth having, not needed: without room for them the launch is unsplit)
     const long ws_bytes = no_ab ? 0 : pl_gemm_tile_alone_workspace_bytes(ta, tb, M, N, K, beta == T(0) ? 1 : 0, (int)sizeof(T));
-    void* ws = ws_bytes > 0 ? R.res.gemm_ws[0].ensure(ws_bytes) : nullptr;
-    chk(GemmFns<T>::tile_alone(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, ws, ws_bytes, R.res.exec[0]), "gemm launch");
+    void* ws = ws_bytes > 0 ? R.res.gemm_ws[0].ensure_if_room(ws_bytes) : nullptr;
+    chk(GemmFns<T>::tile_alone(ta, tb, M, N, no_ab ? 0 : K, alpha, A, ldA, B, ldB, beta, C, ldC, ws, ws ? ws_bytes : 0, R.res.exec[0]), "gemm launch");
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;
