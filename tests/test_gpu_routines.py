@@ -619,6 +619,41 @@ def test_gemm_strip_end_exact_on_integers(pkg, L, ta, tb, order, locs, monkeypat
                 assert np.array_equal(bC.get(), ref)
 
 
+@pytest.mark.parametrize("seed", range(60))
+def test_gemm_routines_random_shapes_exact_on_integers(pkg, L, seed, monkeypatch):
+    """PARALiA_dgemm / PARALiA_sgemm on random problems: shapes up to 3500 x 3500 x 3000, tile sizes 256, 512, 1024 or the
+    planner's, every transpose, each operand pinned, pageable or on the device, padded leading dimensions, alpha / beta
+    pairs with beta = 0 over NaN; the planner's own order, or (one case in three) a pinned strip-end order.  Integer
+    operands: bit for bit numpy's fp64 result, and the padding of C untouched."""
+    rng = np.random.default_rng(90000 + seed)
+    dtype = np.float64 if rng.integers(2) else np.float32
+    ta, tb = "NT"[rng.integers(2)], "NT"[rng.integers(2)]
+    T = int([256, 512, 1024, 1024, -1][rng.integers(5)])
+    M, N, K = int(rng.integers(1, 3500)), int(rng.integers(1, 3500)), int(rng.integers(1, 3000))
+    locs = [int([-1, -1, -2, 0][rng.integers(4)]) for _ in range(3)]
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + int(rng.integers(0, 3)) * 2, rb + int(rng.integers(0, 3)) * 2, M + int(rng.integers(0, 3)) * 2
+    A = rng.integers(-3, 4, lda * ca).astype(dtype)
+    B = rng.integers(-3, 4, ldb * cb).astype(dtype)
+    C0 = rng.integers(-3, 4, ldc * N).astype(dtype)
+    alpha, beta = [(1.0, 0.0), (2.0, -1.0), (-1.0, 1.0), (1.0, 0.0)][rng.integers(4)]
+    monkeypatch.delenv("PARALIA_GEMM_ORDER", raising=False)
+    if rng.integers(3) == 0 and T > 0:
+        monkeypatch.setenv("PARALIA_GEMM_ORDER", str(int([720000, 720001, 650001, 880001, 640002][rng.integers(5)])))
+    a = A.reshape(ca, lda)[:, :ra].T.astype(np.float64)
+    b = B.reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+    ref = (alpha * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T)) + beta * C0.reshape(N, ldc)[:, :M].T.astype(np.float64)).T.astype(dtype)
+    start = C0.copy()
+    if beta == 0.0:
+        start.reshape(N, ldc)[:, :M] = np.nan
+    bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
+    call_gemm(pkg, L, dtype, ta, tb, M, N, K, alpha, beta, bA, lda, bB, ldb, bC, ldc, T=T)
+    got = bC.get().reshape(N, ldc)
+    assert np.array_equal(got[:, :M], ref)
+    assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])
+
+
 def test_sgemm_autotuned_call_merges_k_chains(pkg, L, orc, openblas):
     """No pin: for fp32 with A and B on the host the planner is offered the merged variants and its simulator takes
     one when the product is bound by compute and the chains are long (12288 x 12288 x 16384 here); parity against
