@@ -645,6 +645,15 @@ def other_configs(pkg, L, np, Buf, orc, hA, hB, hC, dA, dB, dC, s, e0, e1, cpu, 
              2.0 * 8192 * 8192 * 8 / link["h2d"] * 1e3, "PCIe: H2D of A and B (1.07e9 B) at the H2D rate measured in this run",
              duplex_roof_ms=duplex_bound_ms(2.0 * 8192 * 8192 * 8, 8192.0 * 8192 * 8, link["h2d"], link["d2h"],
                                             link["h2d_while_d2h_runs"], link["d2h_while_h2d_runs"]))
+    # a mid-size product with every operand in HBM: one launch alone on the device, 576 tiles of 128 x 128, which the
+    # launcher splits along K to fill whole rounds of workgroups
+    tag = "dgemm_3072x3072x16384_device"
+    streamed(tag, L.PARALiA_dgemm, np.float64, b"N", b"N", 3072, 3072, 16384, 1.0, 0.0, (0, 0, 0),
+             2.0 * 3072 * 3072 * 16384 / FP64_MFMA_PEAK * 1e3, "fp64 MFMA peak 78.6 TFLOP/s (operands in HBM: one product alone on the device)")
+    if "error" not in other[tag]:
+        tm, tn, sp = C.c_int(), C.c_int(), C.c_int()
+        pkg.check(L.pl_gemm_tile_choice_alone(8, b"N", b"N", 3072, 3072, 16384, 1, 1 << 30, C.byref(tm), C.byref(tn), C.byref(sp)), "tile choice")
+        other[tag].update({"tile": [tm.value, tn.value], "k_splits": sp.value})
     return other
 
 
