@@ -299,16 +299,36 @@ __device__ __forceinline__ unsigned dma_lane_offset(long ld, int wave, int lane)
 
 // Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
 // give each XCD a contiguous range of logical ids, then walk that range in groups of 8 block rows.
-__device__ __forceinline__ void block_coords(int bid, int gm, int gn, int& bm, int& bn) {
+// A ragged last block row (M not a multiple of the tile) is dealt out first and evenly: its workgroups take the
+// guarded loop, about twice the time of an interior one, and in the walk above they would all fall into the last XCD's
+// range, one in eight of its workgroups, so that XCD finished a sixth later than the other seven (8100 x 8192 x 8192
+// fp64: 62.7 TFLOP/s against 73.1 for 8192 x 8100 x 8192, whose ragged column every XCD shares).  Tile j of that row
+// goes to XCD j mod 8 as one of its first workgroups; the rows above it are walked as before.
+__device__ __forceinline__ void block_coords(int bid, int gm, int gn, bool ragged_m, int& bm, int& bn) {
   const int nb = gm * gn;
-  const int q = nb >> 3, r = nb & 7;
   const int xcd = bid & 7, loc = bid >> 3;
-  const int pid = (xcd < r) ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+  int pid, rows = gm;
+  if (ragged_m && gm > 1) {
+    const int mine = (gn - xcd + 7) >> 3;   // tiles of the last row with j mod 8 == xcd
+    if (loc < mine) {
+      bm = gm - 1;
+      bn = xcd + 8 * loc;
+      return;
+    }
+    // the other rows: XCD y keeps the (nb - y + 7) / 8 workgroups the hardware deals it, less its share of the last row
+    rows = gm - 1;
+    int start = 0;
+    for (int y = 0; y < xcd; ++y) start += ((nb - y + 7) >> 3) - ((gn - y + 7) >> 3);
+    pid = start + loc - mine;
+  } else {
+    const int q = nb >> 3, r = nb & 7;
+    pid = (xcd < r) ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
+  }
   constexpr int GM = 8;
   const int width = GM * gn;
   const int group = pid / width;
   const int first_m = group * GM;
-  const int gsz = min(gm - first_m, GM);
+  const int gsz = min(rows - first_m, GM);
   const int in = pid - group * width;
   bm = first_m + in % gsz;
   bn = in / gsz;
@@ -369,7 +389,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   const int wm = (wave & 1) * WM, wn = (wave >> 1) * WN;
 
   int bm, bn;
-  block_coords(blockIdx.x, gm, gn, bm, bn);
+  block_coords(blockIdx.x, gm, gn, M % BM != 0, bm, bn);
   // the divisions above run on the vector unit; back in scalar registers the tile origins and every address derived
   // from them are scalar arithmetic
   bm = __builtin_amdgcn_readfirstlane(bm);
