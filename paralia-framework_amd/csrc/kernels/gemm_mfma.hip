@@ -20,9 +20,11 @@
 //   * the MFMA "row" index is mapped to n and the "column" index (the lane-contiguous one) to m, so that the
 //     16 / 32 lanes of a group write 128 contiguous bytes of a column of the column-major C;
 //   * workgroup ids are re-mapped so the eight XCDs each own a compact block of C tiles (private L2 per XCD),
-//     and inside an XCD neighbouring ids share A row-panels.
+//     and inside an XCD neighbouring ids share A row-panels; the tiles of a ragged last block row, whose workgroups are
+//     slow, go to all eight XCDs first.
 // Arbitrary M, N, K and leading dimensions are handled; 16-byte vector loads are used when pointer and
-// leading dimension allow it and the workgroup's tile is interior, element loads with zero fill otherwise.
+// leading dimension allow it and the workgroup's tile is interior, element loads with zero fill otherwise.  What K
+// leaves beyond its last whole panel is one guarded step behind the pipelined loop.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
