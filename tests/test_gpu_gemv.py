@@ -37,7 +37,7 @@ def kernel_call(pkg, L, ta, M, N, alpha, dA, lda, dx, incx, beta, dy, incy):
                                      (8192, 64, 0), (64, 8192, 2), (5000, 3000, 0), (3, 20000, 0), (20000, 3, 0)])
 @pytest.mark.parametrize("incx,incy", [(1, 1), (2, 3), (-1, -2)])
 def test_kernel_against_oracle(pkg, L, orc, ta, M, N, pad, incx, incy):
-    """Shapes that take the 16-byte-load path (even M and lda) and the scalar one (odd M or lda), single and many
+    """Shapes that take the 16-byte-load path (even lda; op = T: and even M) and the scalar one, single and many
     reduction chunks, fewer than four columns per wave, strided and reversed vectors."""
     lda = M + pad
     lx, ly = (N, M) if ta == "N" else (M, N)
@@ -52,6 +52,30 @@ def test_kernel_against_oracle(pkg, L, orc, ta, M, N, pad, incx, incy):
     gaps = np.ones(y0.size, dtype=bool)
     gaps[::abs(incy)] = False
     assert np.array_equal(got[gaps], y0[gaps])
+
+
+@pytest.mark.parametrize("M,N,lda", [(1001, 777, 1004), (4095, 300, 4096), (129, 5, 130), (127, 64, 128), (1, 9, 2), (3, 1, 4)])
+def test_kernel_n_with_an_odd_last_row_and_16_byte_columns(pkg, L, M, N, lda):
+    """op = N with an odd M and an even lda: the columns start on 16-byte boundaries, so the rows are read in pairs and
+    the lane that holds the last row reads the padding element behind it along with it -- NaN here, and never part
+    of y -- except in the last column, where that element does not exist: A is allocated with exactly lda * (N - 1) + M
+    elements, the least BLAS asks for.  Integer data: exact."""
+    rng = np.random.default_rng(M + N)
+    A = np.full(lda * (N - 1) + M, np.nan)
+    for n in range(N):
+        A[n * lda:n * lda + M] = rng.integers(-8, 9, M)
+    x = rng.integers(-8, 9, N).astype(np.float64)
+    y0 = rng.integers(-8, 9, M).astype(np.float64)
+    cols = np.stack([A[n * lda:n * lda + M] for n in range(N)], axis=1)
+    ref = 2.0 * (cols @ x) - 3.0 * y0
+    dA, dx, dy = place(pkg, A, 0), place(pkg, x, 0), place(pkg, y0, 0)
+    kernel_call(pkg, L, "N", M, N, 2.0, dA, lda, dx, 1, -3.0, dy, 1)
+    assert np.array_equal(dy.get(), ref)
+    # the same through the entry point that brings its own scratch
+    dy.set(y0)
+    pkg.check(L.pl_dgemv_noalloc(b"N", M, N, 2.0, dA.ptr, lda, dx.ptr, 1, -3.0, dy.ptr, 1, None), "pl_dgemv_noalloc")
+    sync(pkg)
+    assert np.array_equal(dy.get(), ref)
 
 
 @pytest.mark.parametrize("ta", ["N", "T"])
