@@ -111,14 +111,18 @@ __global__ __launch_bounds__(B1_THREADS) void ddot_strided_kernel(long n, const 
   if (threadIdx.x == 0) partials[blockIdx.x] = acc;
 }
 
-// result <- (accumulate ? *result : 0) + sum_{b < nparts} partials[b] (+ tail product of an odd last element)
+// result <- (accumulate ? *result : 0) + sum_{b < nparts} partials[b] (+ the products of the elements the 16-byte pairs
+// of the vector kernel left out: the first nh, in front of the cache line the pairs start on, and an odd last one,
+// xt / yt, null when there is none)
 __global__ __launch_bounds__(B1_THREADS) void ddot_final_kernel(int nparts, const double* __restrict__ partials,
+                                                               const double* __restrict__ xh, const double* __restrict__ yh, int nh,
                                                                const double* __restrict__ xt, const double* __restrict__ yt,
                                                                double* __restrict__ result, int accumulate) {
   double acc = 0.0;
   for (int i = threadIdx.x; i < nparts; i += B1_THREADS) acc += partials[i];
   acc = block_sum(acc);
   if (threadIdx.x == 0) {
+    for (int i = 0; i < nh; ++i) acc = fma(xh[i], yh[i], acc);
     if (xt) acc = fma(*xt, *yt, acc);
     *result = accumulate ? *result + acc : acc;
   }
@@ -179,19 +183,27 @@ extern "C" int pl_daxpy(long n, double alpha, const double* x, long incx, double
   if (!x || !y) return 5;
   if (incx == 0 || incy == 0) return 3;
   hipStream_t s = (hipStream_t)stream;
-  const bool aligned = ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
-  if (incx == 1 && incy == 1 && aligned) {
-    const long n2 = n / 2;
+  // 16-byte pairs when x and y sit at the same place in their 16 bytes (both on a boundary, or both 8 bytes past one):
+  // the elements in front of y's next cache line are updated on their own and the pairs start on that line (x and y at
+  // an odd element of an aligned array: 5.0 -> 6.7 TB/s)
+  const bool pairs = incx == 1 && incy == 1 && ((((uintptr_t)x) ^ ((uintptr_t)y)) & 15) == 0 && (((uintptr_t)x) & 7) == 0;
+  if (pairs) {
+    long head = (long)(((128 - ((uintptr_t)y & 127)) & 127) / 8);
+    if (head > n) head = n;
+    if (head) hipLaunchKernelGGL(daxpy_strided_kernel, dim3(1), dim3(B1_THREADS), 0, s, head, alpha, x, 1L, y, 1L);
+    const double* xv = x + head;
+    double* yv = y + head;
+    const long n2 = (n - head) / 2;
     if (n2 > 0) {
       // the grid's x extent caps one launch at 2^31 - 1 workgroups of 64 pairs: split longer vectors
       const long per_launch = (long)AXPY_THREADS * 0x7fffffffL;
       for (long off = 0; off < n2; off += per_launch) {
         const long m = (n2 - off < per_launch) ? n2 - off : per_launch;
         const unsigned blocks = (unsigned)((m + AXPY_THREADS - 1) / AXPY_THREADS);
-        hipLaunchKernelGGL(daxpy_vec_kernel, dim3(blocks), dim3(AXPY_THREADS), 0, s, m, alpha, (const dvec2*)x + off, (dvec2*)y + off);
+        hipLaunchKernelGGL(daxpy_vec_kernel, dim3(blocks), dim3(AXPY_THREADS), 0, s, m, alpha, (const dvec2*)xv + off, (dvec2*)yv + off);
       }
     }
-    if (n & 1) hipLaunchKernelGGL(daxpy_strided_kernel, dim3(1), dim3(B1_THREADS), 0, s, 1L, alpha, x + n - 1, 1L, y + n - 1, 1L);
+    if ((n - head) & 1) hipLaunchKernelGGL(daxpy_strided_kernel, dim3(1), dim3(B1_THREADS), 0, s, 1L, alpha, x + n - 1, 1L, y + n - 1, 1L);
   } else {
     // BLAS convention for negative increments: element 0 sits at the far end
     const double* xs = incx < 0 ? x + (1 - n) * incx : x;
@@ -212,28 +224,35 @@ extern "C" int pl_ddot(long n, const double* x, long incx, const double* y, long
   hipStream_t s = (hipStream_t)stream;
   if (n <= 0) {
     hipLaunchKernelGGL(ddot_final_kernel, dim3(1), dim3(B1_THREADS), 0, s, 0, workspace, (const double*)nullptr,
-                       (const double*)nullptr, result, accumulate);
+                       (const double*)nullptr, 0, (const double*)nullptr, (const double*)nullptr, result, accumulate);
     return hipGetLastError() == hipSuccess ? 0 : 4;
   }
   if (!x || !y) return 5;
   if (incx == 0 || incy == 0) return 3;
-  const bool aligned = ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
+  // 16-byte pairs when x and y sit at the same place in their 16 bytes (both on a boundary, or both 8 bytes past one):
+  // the elements in front of y's next cache line go to the final kernel and the pairs start on that line (x and y at an
+  // odd element of an aligned array: 6.1 -> 7.0 TB/s)
+  const bool pairs = incx == 1 && incy == 1 && ((((uintptr_t)x) ^ ((uintptr_t)y)) & 15) == 0 && (((uintptr_t)x) & 7) == 0;
   int blocks = 0;
-  const double *xt = nullptr, *yt = nullptr;
-  if (incx == 1 && incy == 1 && aligned) {
-    const long n2 = n / 2;
+  const double *xh = nullptr, *yh = nullptr, *xt = nullptr, *yt = nullptr;
+  long head = 0;
+  if (pairs) {
+    head = (long)(((128 - ((uintptr_t)y & 127)) & 127) / 8);
+    if (head > n) head = n;
+    if (head) { xh = x; yh = y; }
+    const long n2 = (n - head) / 2;
     if (n2 > 0) {
       blocks = grid_for(n2, B1_THREADS * B1_UNROLL * 4, DOT_MAX_BLOCKS);
-      hipLaunchKernelGGL(ddot_vec_kernel, dim3(blocks), dim3(B1_THREADS), 0, s, n2, (const dvec2*)x, (const dvec2*)y, workspace);
+      hipLaunchKernelGGL(ddot_vec_kernel, dim3(blocks), dim3(B1_THREADS), 0, s, n2, (const dvec2*)(x + head), (const dvec2*)(y + head), workspace);
     }
-    if (n & 1) { xt = x + n - 1; yt = y + n - 1; }
+    if ((n - head) & 1) { xt = x + n - 1; yt = y + n - 1; }
   } else {
     const double* xs = incx < 0 ? x + (1 - n) * incx : x;
     const double* ys = incy < 0 ? y + (1 - n) * incy : y;
     blocks = grid_for(n, B1_THREADS * 8, DOT_MAX_BLOCKS);
     hipLaunchKernelGGL(ddot_strided_kernel, dim3(blocks), dim3(B1_THREADS), 0, s, n, xs, incx, ys, incy, workspace);
   }
-  hipLaunchKernelGGL(ddot_final_kernel, dim3(1), dim3(B1_THREADS), 0, s, blocks, workspace, xt, yt, result, accumulate);
+  hipLaunchKernelGGL(ddot_final_kernel, dim3(1), dim3(B1_THREADS), 0, s, blocks, workspace, xh, yh, (int)head, xt, yt, result, accumulate);
   return hipGetLastError() == hipSuccess ? 0 : 4;
 }
 

@@ -443,6 +443,29 @@ def test_ddot_exact_and_strided(pkg, L, orc):
     assert res.get()[0] == 0.0
 
 
+@pytest.mark.parametrize("ox,oy", [(1, 1), (3, 3), (15, 15), (5, 21), (16, 16), (2, 4), (1, 0), (0, 7)])
+@pytest.mark.parametrize("n", [1, 2, 7, 14, 15, 16, 40, 1000003])
+def test_daxpy_ddot_vectors_that_start_inside_a_cache_line(pkg, L, ox, oy, n):
+    """x and y starting at element ox / oy of 256-byte aligned arrays.  When both sit at the same place in their 16 bytes
+    the elements in front of y's next cache line are handled one by one and the 16-byte pairs start on that line (also
+    when the vector ends before it); otherwise the element kernels run.  Integer data: exact, and nothing outside the
+    n elements of y is written."""
+    rng = np.random.default_rng(n + 31 * ox + oy)
+    X = rng.integers(-9, 10, n + 64).astype(np.float64)
+    Y = rng.integers(-9, 10, n + 64).astype(np.float64)
+    dx, dy = Buf(pkg, X.size, np.float64, 0).set(X), Buf(pkg, Y.size, np.float64, 0).set(Y)
+    pkg.check(L.pl_daxpy(n, 3.0, dx.at(ox), 1, dy.at(oy), 1, None), "daxpy")
+    sync(pkg)
+    ref = Y.copy()
+    ref[oy:oy + n] += 3.0 * X[ox:ox + n]
+    assert np.array_equal(dy.get(), ref)
+    res = Buf(pkg, 1, np.float64, 0).set(np.array([5.0]))
+    ws = Buf(pkg, int(L.pl_ddot_workspace_doubles()), np.float64, 0)
+    pkg.check(L.pl_ddot(n, dx.at(ox), 1, dy.at(oy), 1, res.ptr, 1, ws.ptr, None), "ddot")
+    sync(pkg)
+    assert res.get()[0] == 5.0 + float(np.dot(X[ox:ox + n], ref[oy:oy + n]))
+
+
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_geadd(pkg, L, dtype):
     M, N = 1001, 77
