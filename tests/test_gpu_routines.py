@@ -654,6 +654,37 @@ def test_gemm_routines_random_shapes_exact_on_integers(pkg, L, seed, monkeypatch
     assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("M,N,K,pads,offs", [(2049, 2051, 301, (0, 0, 0), (0, 0)), (2304, 2100, 500, (1, 3, 1), (0, 0)),
+                                             (2200, 2300, 260, (0, 0, 0), (1, 1)), (2048, 100, 300, (1, 1, 1), (0, 0))])
+def test_gemm_device_resident_operands_that_are_not_16_byte_aligned(pkg, L, ta, tb, M, N, K, pads, offs):
+    """A, B and C in HBM with odd leading dimensions or starting 8 bytes (fp32: 4) into a 16-byte unit: where the other
+    dimension of the product reaches 2048 the call multiplies 16-byte aligned copies of A and B with padded leading
+    dimensions (the last shape, N = 100: B is copied, A is not), C is used where it lies.  Integer operands: bit for
+    bit numpy's fp64 result, the padding of C untouched, and the caller's A and B unchanged."""
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + pads[0], rb + pads[1], M + pads[2]
+    rng = np.random.default_rng(M + N + K)
+    for dtype in (np.float64, np.float32):
+        A = rng.integers(-3, 4, lda * ca + offs[0]).astype(dtype)
+        B = rng.integers(-3, 4, ldb * cb + offs[1]).astype(dtype)
+        C0 = rng.integers(-3, 4, ldc * N).astype(dtype)
+        a = A[offs[0]:].reshape(ca, lda)[:, :ra].T.astype(np.float64)
+        b = B[offs[1]:].reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+        ref = (2.0 * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T)) - C0.reshape(N, ldc)[:, :M].T.astype(np.float64)).T.astype(dtype)
+        bA, bB, bC = place(pkg, A, 0), place(pkg, B, 0), place(pkg, C0, 0)
+        info = pkg.atc_info()
+        fn = L.PARALiA_dgemm if dtype == np.float64 else L.PARALiA_sgemm
+        for _ in range(2):   # the second call finds the copies' buffers in place
+            bC.set(C0)
+            pkg.check(fn(ta.encode(), tb.encode(), M, N, K, 2.0, bA.at(offs[0]), lda, bB.at(offs[1]), ldb, -1.0, bC.ptr, ldc, -1, 0, C.byref(info)), "gemm")
+            got = bC.get().reshape(N, ldc)
+            assert np.array_equal(got[:, :M], ref)
+            assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])
+        assert np.array_equal(bA.get(), A) and np.array_equal(bB.get(), B)
+
+
 def test_sgemm_autotuned_call_merges_k_chains(pkg, L, orc, openblas):
     """No pin: for fp32 with A and B on the host the planner is offered the merged variants and its simulator takes
     one when the product is bound by compute and the chains are long (12288 x 12288 x 16384 here); parity against
