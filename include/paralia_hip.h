@@ -116,6 +116,19 @@ int pl_sgemm_tile_split(char transA, char transB, long M, long N, long K, float 
                         const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
                         int splits, void* stream);
 
+/* The product on operands that live in larger blocks (the scheduler's tiles in its device pool: the reference's tiles
+ * in CBlocks, DataCaching.hpp).  m_readable >= M rows of op(A) and n_readable >= N columns of op(B) may be READ -- the
+ * memory is there, its content beyond M and N is anything -- so the workgroups on the ragged edge of C load whole
+ * 128-wide tiles without guards like the interior ones (what they read from beyond only reaches elements of C that
+ * are not stored).  0 stands for M or N.  splits: 0 the launcher's choice as in pl_dgemm_tile_ws, >= 1 as in
+ * pl_dgemm_tile_split. */
+int pl_dgemm_tile_padded(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                         const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
+                         int splits, long m_readable, long n_readable, void* stream);
+int pl_sgemm_tile_padded(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                         const float* B, long ldb, float beta, float* C, long ldc, void* workspace, long workspace_bytes,
+                         int splits, long m_readable, long n_readable, void* stream);
+
 /* The product for a caller who knows it has the device to itself (every operand already in HBM and nothing else
  * running: the reference's call with all data on the GPU is one cublasDgemm, dgemm.cpp:382-395 with a single
  * subkernel).  The launcher then counts whole rounds of two workgroups per compute unit instead of assuming a second

@@ -345,7 +345,8 @@ __device__ __forceinline__ void block_coords(int bid, int gm, int gn, bool ragge
 template <typename T, bool AK, bool BKM, int BM, int BN, int BK, bool DIR = true>
 __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 8 ? 2 : 1)) void gemm_kernel(int M, int N, int K, T alpha, const T* __restrict__ A, long lda,
                                                           const T* __restrict__ B, long ldb, T beta, T* __restrict__ C,
-                                                          long ldc, int gm, int gn, int vecA, int vecB, int vecC, int kchunk) {
+                                                          long ldc, int gm, int gn, int vecA, int vecB, int vecC, int kchunk,
+                                                          int m_read, int n_read) {
   using Tr = Traits<T>;
   using vec_t = typename Tr::vec_t;
   using acc_t = typename Tr::acc_t;
@@ -398,7 +399,11 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   bn = __builtin_amdgcn_readfirstlane(bn);
   const int m0 = bm * BM, n0 = bn * BN;
   const int mrem = min(M - m0, BM), nrem = min(N - n0, BN);
-  const bool fast = (mrem == BM) && (nrem == BN) && vecA && vecB;
+  // Unguarded loads for every workgroup whose whole tile of op(A) rows and op(B) columns may be READ: the interior
+  // ones, and on the edge of C those for which the caller vouches that the memory behind the operands' last rows is
+  // there (m_read, n_read >= M, N: tiles that live in larger blocks).  What is read from beyond M or N only reaches
+  // elements of C that the guarded epilogue does not store.
+  const bool fast = (m0 + BM <= m_read) && (n0 + BN <= n_read) && vecA && vecB;
 
   // tile origins; element (mn, k) of op(X) lives at base[mn + k*ld] (MN-major) or base[k + mn*ld] (K-major)
   const T* Ab = AK ? A + (long)m0 * lda : A + m0;
@@ -1044,7 +1049,7 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
 template <typename T>
 int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
                 T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0, int want_splits = 0,
-                bool alone = false) {
+                bool alone = false, long m_read = 0, long n_read = 0) {
   using Tr = Traits<T>;
   const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
   const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
@@ -1053,6 +1058,10 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 2;
   const long rowsA = an ? M : K, rowsB = bnn ? K : N;
   if (lda < (rowsA > 1 ? rowsA : 1) || ldb < (rowsB > 1 ? rowsB : 1) || ldc < (M > 1 ? M : 1)) return 3;
+  // rows of op(A) / columns of op(B) that may be read (0: as many as there are)
+  if (m_read == 0) m_read = M;
+  if (n_read == 0) n_read = N;
+  if (m_read < M || n_read < N || m_read > INT32_MAX || n_read > INT32_MAX) return 2;
   if (M == 0 || N == 0) return 0;
   if (K == 0 || alpha == T(0)) {
     if (beta == T(1)) return 0;
@@ -1092,7 +1101,7 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   const bool deep = sizeof(T) == 4 && (splits > 1 ? kchunk : K) % PLK_F32_DEEP_BK == 0 && dma_fits;
 #define PLK_LAUNCH_T(AKF, BKF, TM, TN, TK, DIRF)                                                                            \
   hipLaunchKernelGGL((gemm_kernel<T, AKF, BKF, TM, TN, TK, DIRF>), grid, block, 0, stream, (int)M, (int)N, (int)K, k_alpha, \
-                     A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk)
+                     A, lda, B, ldb, k_beta, k_C, k_ldc, gm, gn, vecA, vecB, vecC, kchunk, (int)m_read, (int)n_read)
 #define PLK_LAUNCH(AKF, BKF)                                                        \
   do {                                                                              \
     if constexpr (sizeof(T) == 4) {                                                 \
@@ -1191,6 +1200,22 @@ extern "C" int pl_sgemm_tile_split(char transA, char transB, long M, long N, lon
   if (splits < 1) return PL_ERR_ARG;
   return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
                                  (float*)workspace, workspace_bytes, splits);
+}
+
+extern "C" int pl_dgemm_tile_padded(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
+                                    const double* B, long ldb, double beta, double* C, long ldc, void* workspace,
+                                    long workspace_bytes, int splits, long m_readable, long n_readable, void* stream) {
+  if (splits < 0) return PL_ERR_ARG;
+  return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                  (double*)workspace, workspace_bytes, splits, false, m_readable, n_readable);
+}
+
+extern "C" int pl_sgemm_tile_padded(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
+                                    const float* B, long ldb, float beta, float* C, long ldc, void* workspace,
+                                    long workspace_bytes, int splits, long m_readable, long n_readable, void* stream) {
+  if (splits < 0) return PL_ERR_ARG;
+  return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
+                                 (float*)workspace, workspace_bytes, splits, false, m_readable, n_readable);
 }
 
 // workspace a product alone on the device is given at most (the slices of its split)

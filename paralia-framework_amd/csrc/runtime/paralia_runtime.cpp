@@ -307,6 +307,10 @@ template <> struct GemmFns<double> {
                   double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_dgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
   }
+  static int tile_padded(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
+                         double be, double* C, long ldc, void* ws, long ws_bytes, int splits, long m_read, long n_read, void* s) {
+    return pl_dgemm_tile_padded(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, m_read, n_read, s);
+  }
   static int tile_alone(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
                         double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_dgemm_tile_alone(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
@@ -324,6 +328,10 @@ template <> struct GemmFns<float> {
   static int tile(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                   float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
     return pl_sgemm_tile_ws(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
+  }
+  static int tile_padded(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
+                         float be, float* C, long ldc, void* ws, long ws_bytes, int splits, long m_read, long n_read, void* s) {
+    return pl_sgemm_tile_padded(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, m_read, n_read, s);
   }
   static int tile_alone(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                         float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
@@ -390,21 +398,26 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   // leading dimension an odd M, N or K left the tiles of the last block row / column / k-step -- with merged chains
   // every K-major panel -- to the element loads (dgemm 16383^3 from the host: 152 ms against 120 ms at 16384^3).  The
   // padded tile still fits its block of T x T elements when T is a multiple of 16; other tile sizes keep dense tiles.
+  // With T a multiple of 128 the m / n extent of a tile is rounded up to whole 128-wide kernel tiles instead: the rows
+  // of op(A) and the columns of op(B) up to there lie inside the tile's block (or panel) whichever way the operand is
+  // stored, so the kernel may read them (pl_dgemm_tile_padded) and the workgroups on a ragged edge of C need no guarded
+  // loads either.
   const int Kg = p.Kg();
-  const bool pad_ld = Tt % 16 == 0;
+  const bool pad_ld = Tt % 16 == 0, whole_tiles = Tt % 128 == 0;
   auto padded = [&](long rows) { return pad_ld ? (rows + 15) / 16 * 16 : rows; };
+  auto readable = [&](long mn) { return whole_tiles ? (mn + 127) / 128 * 128 : mn; };   // <= T
   auto a_tile = [&](int block, int mi, int ki, long* ld) -> T* {
-    if (!plan.panels) { *ld = padded(at ? p.tk(ki) : p.tm(mi)); return (T*)R.pool.at(block); }
+    if (!plan.panels) { *ld = at ? padded(p.tk(ki)) : padded(readable(p.tm(mi))); return (T*)R.pool.at(block); }
     T* base = (T*)R.pool.at(plan.a_first + (long)mi * Kg);
     if (at) { *ld = padded(std::max(1L, p.K)); return base + p.k0(ki); }
-    *ld = padded(p.tm(mi));
+    *ld = padded(readable(p.tm(mi)));
     return base + p.k0(ki) * *ld;
   };
   auto b_tile = [&](int block, int ni, int ki, long* ld) -> T* {
-    if (!plan.panels) { *ld = padded(bt ? p.tn(ni) : p.tk(ki)); return (T*)R.pool.at(block); }
+    if (!plan.panels) { *ld = bt ? padded(readable(p.tn(ni))) : padded(p.tk(ki)); return (T*)R.pool.at(block); }
     T* base = (T*)R.pool.at(plan.b_first + (long)ni * Kg);
     if (!bt) { *ld = padded(std::max(1L, p.K)); return base + p.k0(ki); }
-    *ld = padded(p.tn(ni));
+    *ld = padded(readable(p.tn(ni)));
     return base + p.k0(ki) * *ld;
   };
 
@@ -465,14 +478,18 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
         const T bp = c.beta_mode == BETA_ZERO ? T(0) : c.beta_mode == BETA_ONE ? T(1) : beta;
         if (la < 1) la = 1;
         if (lb < 1) lb = 1;
+        // what of the operands may be read beyond the tile's ragged edge: tiles in pool blocks, see a_tile / b_tile
+        const long m_read = c.a_block >= 0 ? readable(m) : m, n_read = c.b_block >= 0 ? readable(n) : n;
         if (c.rows > 0) {
           // a row strip of the tile: those rows of op(A) and of C, the launch splitting K as the plan says
           a += at ? (long)c.row0 * la : (long)c.row0;
           cc += c.row0;
-          chk(GemmFns<T>::tile_split(ta, tb, c.rows, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes,
-                                     std::max(1, c.splits), s), "tile gemm launch");
+          chk(GemmFns<T>::tile_padded(ta, tb, c.rows, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes,
+                                      std::max(1, c.splits), std::max<long>(c.rows, std::min<long>(m_read - c.row0, (c.rows + 127) / 128 * 128)), n_read, s),
+              "tile gemm launch");
         } else {
-          chk(GemmFns<T>::tile(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, s), "tile gemm launch");
+          chk(GemmFns<T>::tile_padded(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, 0, m_read, n_read, s),
+              "tile gemm launch");
         }
       } break;
       case CMD_REDUCE: {

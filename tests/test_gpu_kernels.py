@@ -611,6 +611,51 @@ def test_gemm_tile_alone_on_the_device(pkg, L, ta, tb, dims):
                 assert np.array_equal(dC.get().reshape(N, ldc)[:, :M], ref), (np.dtype(dtype).name, beta, ws_bytes)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("M,N,K,splits", [(1000, 900, 520, 0), (2047, 2047, 777, 0), (130, 140, 2000, 0), (511, 2048, 4000, 4), (300, 257, 64, 1), (129, 1, 33, 0)])
+def test_gemm_tile_on_operands_that_live_in_larger_blocks(pkg, L, ta, tb, M, N, K, splits):
+    """pl_dgemm_tile_padded / pl_sgemm_tile_padded: the operands lie in blocks that reach up to the next multiple of 128 rows
+    of op(A) and columns of op(B), and the caller says so, so the workgroups on the ragged edge of C load like interior
+    ones.  What lies beyond M and N is NaN here and must not reach C; C itself has no room to spare (ldc = M, exactly
+    M x N elements, NaN where beta = 0), and its result is exact on integer operands.  Also with the launcher's and the
+    caller's split counts, a ragged K, and extents that promise less than M or N (refused)."""
+    Mr, Nr = -(-M // 128) * 128, -(-N // 128) * 128
+    rng = np.random.default_rng(M + N + K)
+    for dtype in (np.float64, np.float32):
+        esz = np.dtype(dtype).itemsize
+        fn = L.pl_dgemm_tile_padded if dtype == np.float64 else L.pl_sgemm_tile_padded
+        # op(A): Mr x K readable, M x K valid; stored M-major (ta = N: Mr x K, ld Mr) or K-major (ta = T: K x Mr, ld K + 16)
+        a = rng.integers(-4, 5, (M, K)).astype(np.float64)
+        b = rng.integers(-4, 5, (K, N)).astype(np.float64)
+        if ta == "N":
+            lda = Mr
+            A = np.full((K, lda), np.nan); A[:, :M] = a.T
+        else:
+            lda = K + 16
+            A = np.full((Mr, lda), np.nan); A[:M, :K] = a
+        if tb == "N":
+            ldb = K + 16
+            B = np.full((Nr, ldb), np.nan); B[:N, :K] = b.T
+        else:
+            ldb = Nr
+            B = np.full((K, ldb), np.nan); B[:, :N] = b
+        C0 = rng.integers(-4, 5, (N, M)).astype(np.float64)
+        dA, dB = Buf(pkg, A.size, dtype, 0).set(A.reshape(-1).astype(dtype)), Buf(pkg, B.size, dtype, 0).set(B.reshape(-1).astype(dtype))
+        n_ws = max(1, max(splits, 16) * M * N)
+        dW = Buf(pkg, n_ws, dtype, 0)
+        for beta in (0.0, 2.0):
+            start = np.full(M * N, np.nan) if beta == 0.0 else C0.reshape(-1)
+            dC = Buf(pkg, M * N, dtype, 0).set(start.astype(dtype))
+            print("gemm_padded", np.dtype(dtype).name, ta, tb, M, N, K, "readable", Mr, Nr, "splits", splits, "beta", beta, flush=True)
+            pkg.check(fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, beta, dC.ptr, M, dW.ptr, n_ws * esz, splits, Mr, Nr, None), "gemm tile padded")
+            sync(pkg)
+            ref = (3.0 * (a @ b) + beta * C0.T).T.astype(dtype)
+            assert np.array_equal(dC.get().reshape(N, M), ref), (np.dtype(dtype).name, beta)
+        assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, M, dW.ptr, n_ws * esz, splits, M - 1, Nr, None) != 0
+        assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, M, dW.ptr, n_ws * esz, -1, Mr, Nr, None) == 7
+        sync(pkg)
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N")])
 def test_gemm_tile_split_k_exact_and_fallback(pkg, L, orc, ta, tb):
     """Integer-valued data: the split result equals the unsplit one bit for bit, for fp64 and fp32; beta = 0 with a
