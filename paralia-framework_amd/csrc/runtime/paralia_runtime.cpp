@@ -403,9 +403,11 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
   // stored, so the kernel may read them (pl_dgemm_tile_padded) and the workgroups on a ragged edge of C need no guarded
   // loads either.
   const int Kg = p.Kg();
-  const bool pad_ld = Tt % 16 == 0, whole_tiles = Tt % 128 == 0;
+  // (whole 256-wide tiles where T allows it: the fp32 kernel's larger macro tiles are 256 wide)
+  const bool pad_ld = Tt % 16 == 0;
+  const long tile_w = Tt % 256 == 0 ? 256 : Tt % 128 == 0 ? 128 : 0;
   auto padded = [&](long rows) { return pad_ld ? (rows + 15) / 16 * 16 : rows; };
-  auto readable = [&](long mn) { return whole_tiles ? (mn + 127) / 128 * 128 : mn; };   // <= T
+  auto readable = [&](long mn) { return tile_w ? (mn + tile_w - 1) / tile_w * tile_w : mn; };   // <= T
   auto a_tile = [&](int block, int mi, int ki, long* ld) -> T* {
     if (!plan.panels) { *ld = at ? padded(p.tk(ki)) : padded(readable(p.tm(mi))); return (T*)R.pool.at(block); }
     T* base = (T*)R.pool.at(plan.a_first + (long)mi * Kg);
@@ -485,7 +487,7 @@ static void execute_gemm_plan(Runtime& R, const GemmPlan& plan, char ta, char tb
           a += at ? (long)c.row0 * la : (long)c.row0;
           cc += c.row0;
           chk(GemmFns<T>::tile_padded(ta, tb, c.rows, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes,
-                                      std::max(1, c.splits), std::max<long>(c.rows, std::min<long>(m_read - c.row0, (c.rows + 127) / 128 * 128)), n_read, s),
+                                      std::max(1, c.splits), std::max<long>(c.rows, m_read - c.row0), n_read, s),
               "tile gemm launch");
         } else {
           chk(GemmFns<T>::tile_padded(ta, tb, m, n, k, alpha, a, la, b, lb, bp, cc, lc, ws[c.stream - STREAM_EXEC0], ws_bytes, 0, m_read, n_read, s),
