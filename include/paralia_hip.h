@@ -121,7 +121,7 @@ int pl_sgemm_tile_split(char transA, char transB, long M, long N, long K, float 
  * memory is there, its content beyond M and N is anything -- so the workgroups on the ragged edge of C load whole
  * 128-wide tiles without guards like the interior ones (what they read from beyond only reaches elements of C that
  * are not stored).  0 stands for M or N.  splits: 0 the launcher's choice as in pl_dgemm_tile_ws, >= 1 as in
- * pl_dgemm_tile_split. */
+ * pl_dgemm_tile_split, -1 its choice for a product alone on the device as in pl_dgemm_tile_alone (declared below). */
 int pl_dgemm_tile_padded(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
                          const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
                          int splits, long m_readable, long n_readable, void* stream);

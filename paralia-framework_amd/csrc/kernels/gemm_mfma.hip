@@ -1205,17 +1205,17 @@ extern "C" int pl_sgemm_tile_split(char transA, char transB, long M, long N, lon
 extern "C" int pl_dgemm_tile_padded(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
                                     const double* B, long ldb, double beta, double* C, long ldc, void* workspace,
                                     long workspace_bytes, int splits, long m_readable, long n_readable, void* stream) {
-  if (splits < 0) return PL_ERR_ARG;
+  if (splits < -1) return PL_ERR_ARG;
   return plk::launch_gemm<double>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
-                                  (double*)workspace, workspace_bytes, splits, false, m_readable, n_readable);
+                                  (double*)workspace, workspace_bytes, splits < 0 ? 0 : splits, splits < 0, m_readable, n_readable);
 }
 
 extern "C" int pl_sgemm_tile_padded(char transA, char transB, long M, long N, long K, float alpha, const float* A, long lda,
                                     const float* B, long ldb, float beta, float* C, long ldc, void* workspace,
                                     long workspace_bytes, int splits, long m_readable, long n_readable, void* stream) {
-  if (splits < 0) return PL_ERR_ARG;
+  if (splits < -1) return PL_ERR_ARG;
   return plk::launch_gemm<float>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, (hipStream_t)stream,
-                                 (float*)workspace, workspace_bytes, splits, false, m_readable, n_readable);
+                                 (float*)workspace, workspace_bytes, splits < 0 ? 0 : splits, splits < 0, m_readable, n_readable);
 }
 
 // workspace a product alone on the device is given at most (the slices of its split)

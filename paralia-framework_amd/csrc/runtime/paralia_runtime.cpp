@@ -311,10 +311,6 @@ template <> struct GemmFns<double> {
                          double be, double* C, long ldc, void* ws, long ws_bytes, int splits, long m_read, long n_read, void* s) {
     return pl_dgemm_tile_padded(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, m_read, n_read, s);
   }
-  static int tile_alone(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
-                        double be, double* C, long ldc, void* ws, long ws_bytes, void* s) {
-    return pl_dgemm_tile_alone(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
-  }
   static int tile_split(char ta, char tb, long M, long N, long K, double al, const double* A, long lda, const double* B, long ldb,
                         double be, double* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
     return pl_dgemm_tile_split(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, s);
@@ -332,10 +328,6 @@ template <> struct GemmFns<float> {
   static int tile_padded(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                          float be, float* C, long ldc, void* ws, long ws_bytes, int splits, long m_read, long n_read, void* s) {
     return pl_sgemm_tile_padded(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, splits, m_read, n_read, s);
-  }
-  static int tile_alone(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
-                        float be, float* C, long ldc, void* ws, long ws_bytes, void* s) {
-    return pl_sgemm_tile_alone(ta, tb, M, N, K, al, A, lda, B, ldb, be, C, ldc, ws, ws_bytes, s);
   }
   static int tile_split(char ta, char tb, long M, long N, long K, float al, const float* A, long lda, const float* B, long ldb,
                         float be, float* C, long ldc, void* ws, long ws_bytes, int splits, void* s) {
@@ -650,25 +642,31 @@ static ATC_p gemm_entry(char TransA, char TransB, long M, long N, long K, T alph
     // 16 bytes) sends every workgroup to the element loads: 8191^3 with ld = 8191 runs at 57 TFLOP/s (fp32: 103) against
     // 75 (152).  A copy with a padded leading dimension costs two passes over the operand at 3 TB/s, a tenth of that
     // difference once the product's other dimension reaches 2048; taken when the device has the room.
+    // The copy is laid out in whole 256-wide kernel tiles along m (or n), like the tiles of the streamed path, so its
+    // edge may be read too (m_read, n_read).
     const T* a_use = A;
     const T* b_use = B;
-    long lda_use = ldA, ldb_use = ldB;
+    long lda_use = ldA, ldb_use = ldB, m_read = M, n_read = N;
     if (!no_ab) {
       constexpr long VEC = 16 / (long)sizeof(T);
-      auto realigned = [&](int which, const T* p, long ld, long rows, long cols, long other_dim, long* ld_out) -> const T* {
+      // mn_major: the operand's rows run along m (or n); else they run along k and its columns along m (or n)
+      auto realigned = [&](int which, const T* p, long ld, long rows, long cols, bool mn_major, long other_dim, long* ld_out, long* read_out) -> const T* {
         const bool unaligned = (reinterpret_cast<uintptr_t>(p) & 15) != 0 || ld % VEC != 0;
         if (!unaligned || other_dim < 2048 || rows < VEC) return p;
-        const long ld2 = (rows + 15) / 16 * 16;
-        void* copy = R.res.gemm_realigned[which].ensure_if_room((long long)ld2 * cols * (long long)sizeof(T));
+        const long mn = mn_major ? rows : cols, mn_tiles = (mn + 255) / 256 * 256;
+        const long ld2 = mn_major ? mn_tiles : (rows + 15) / 16 * 16, cols2 = mn_major ? cols : mn_tiles;
+        void* copy = R.res.gemm_realigned[which].ensure_if_room((long long)ld2 * cols2 * (long long)sizeof(T));
         if (!copy) return p;
         chk(pl_copy2d_async(copy, ld2, p, ld, rows, cols, sizeof(T), R.res.exec[0]), "operand copy");
         *ld_out = ld2;
+        *read_out = mn_tiles;
         return (const T*)copy;
       };
-      a_use = realigned(0, A, ldA, ta == 'N' ? M : K, ta == 'N' ? K : M, N, &lda_use);
-      b_use = realigned(1, B, ldB, tb == 'N' ? K : N, tb == 'N' ? N : K, M, &ldb_use);
+      a_use = realigned(0, A, ldA, ta == 'N' ? M : K, ta == 'N' ? K : M, ta == 'N', N, &lda_use, &m_read);
+      b_use = realigned(1, B, ldB, tb == 'N' ? K : N, tb == 'N' ? N : K, tb != 'N', M, &ldb_use, &n_read);
     }
-    chk(GemmFns<T>::tile_alone(ta, tb, M, N, no_ab ? 0 : K, alpha, a_use, lda_use, b_use, ldb_use, beta, C, ldC, ws, ws ? ws_bytes : 0, R.res.exec[0]), "gemm launch");
+    chk(GemmFns<T>::tile_padded(ta, tb, M, N, no_ab ? 0 : K, alpha, a_use, lda_use, b_use, ldb_use, beta, C, ldC, ws, ws ? ws_bytes : 0, -1, m_read, n_read,
+                                R.res.exec[0]), "gemm launch");
     chk(pl_stream_sync(R.res.exec[0]), "stream sync");
   } else {
     const GemmPlan& plan = entry->plan;

@@ -612,13 +612,15 @@ def test_gemm_tile_alone_on_the_device(pkg, L, ta, tb, dims):
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
-@pytest.mark.parametrize("M,N,K,splits", [(1000, 900, 520, 0), (2047, 2047, 777, 0), (130, 140, 2000, 0), (511, 2048, 4000, 4), (300, 257, 64, 1), (129, 1, 33, 0)])
+@pytest.mark.parametrize("M,N,K,splits", [(1000, 900, 520, 0), (2047, 2047, 777, 0), (130, 140, 2000, 0), (511, 2048, 4000, 4), (300, 257, 64, 1), (129, 1, 33, 0),
+                                          (2500, 2400, 1100, -1)])
 def test_gemm_tile_on_operands_that_live_in_larger_blocks(pkg, L, ta, tb, M, N, K, splits):
     """pl_dgemm_tile_padded / pl_sgemm_tile_padded: the operands lie in blocks that reach up to the next multiple of 128 rows
     of op(A) and columns of op(B), and the caller says so, so the workgroups on the ragged edge of C load like interior
     ones.  What lies beyond M and N is NaN here and must not reach C; C itself has no room to spare (ldc = M, exactly
     M x N elements, NaN where beta = 0), and its result is exact on integer operands.  Also with the launcher's and the
-    caller's split counts, a ragged K, and extents that promise less than M or N (refused)."""
+    caller's split counts and its count for a product alone on the device (-1), a ragged K, and extents that promise less
+    than M or N (refused)."""
     Mr, Nr = -(-M // 128) * 128, -(-N // 128) * 128
     rng = np.random.default_rng(M + N + K)
     for dtype in (np.float64, np.float32):
@@ -652,7 +654,7 @@ def test_gemm_tile_on_operands_that_live_in_larger_blocks(pkg, L, ta, tb, M, N, 
             ref = (3.0 * (a @ b) + beta * C0.T).T.astype(dtype)
             assert np.array_equal(dC.get().reshape(N, M), ref), (np.dtype(dtype).name, beta)
         assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, M, dW.ptr, n_ws * esz, splits, M - 1, Nr, None) != 0
-        assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, M, dW.ptr, n_ws * esz, -1, Mr, Nr, None) == 7
+        assert fn(ta.encode(), tb.encode(), M, N, K, 3.0, dA.ptr, lda, dB.ptr, ldb, 0.0, dC.ptr, M, dW.ptr, n_ws * esz, -2, Mr, Nr, None) == 7
         sync(pkg)
 
 
