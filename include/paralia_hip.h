@@ -247,7 +247,8 @@ int PARALiA_ddot(long N, double* x, long incx, double* y, long incy, double* res
  * ('N') or M ('T') elements, y the other count */
 int PARALiA_dgemv(char TransA, long M, long N, double alpha, double* A, long ldA, double* x, long incx, double beta, double* y,
                   long incy, long T, long long cache_limit, pl_atc_info* info);
-/* PARALiADevCacheFree (Subkernel.cpp:488) */
+/* PARALiADevCacheFree (Subkernel.cpp:488): device 0 gives back the block pool, the split-K workspaces and the
+ * aligned copies of unaligned device-resident GEMM operands; streams, events and the cached problems stay */
 int PARALiA_dev_cache_free(int dev_id);
 /* metadata-cache and pool counters (PMD_cache, dgemm.cpp:342-368); reset drops the cached problems */
 int PARALiA_runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries);

@@ -1028,6 +1028,10 @@ void cache_free_impl(short dev_id) {
   if (dev_id != 0) return;  // the host "cache" of the reference (dev -1) holds nothing here
   R.res.sync_all();
   R.pool.release();
+  // the device memory that grows with the operands goes with the pool: the split-K workspaces and the aligned copies
+  // of unaligned device-resident operands (each is allocated again by the next call that needs it)
+  for (auto& w : R.res.gemm_ws) w.release();
+  for (auto& w : R.res.gemm_realigned) w.release();
 }
 
 void runtime_stats(long* pmd_hits, long* pmd_misses, long long* pool_bytes, long* pmd_entries) {

@@ -676,7 +676,9 @@ def test_gemm_device_resident_operands_that_are_not_16_byte_aligned(pkg, L, ta, 
         bA, bB, bC = place(pkg, A, 0), place(pkg, B, 0), place(pkg, C0, 0)
         info = pkg.atc_info()
         fn = L.PARALiA_dgemm if dtype == np.float64 else L.PARALiA_sgemm
-        for _ in range(2):   # the second call finds the copies' buffers in place
+        for rep in range(3):   # the second call finds the copies' buffers in place, the third allocates them again
+            if rep == 2:
+                L.PARALiA_dev_cache_free(0)
             bC.set(C0)
             pkg.check(fn(ta.encode(), tb.encode(), M, N, K, 2.0, bA.at(offs[0]), lda, bB.at(offs[1]), ldb, -1.0, bC.ptr, ldc, -1, 0, C.byref(info)), "gemm")
             got = bC.get().reshape(N, ldc)
