@@ -134,7 +134,11 @@ int pl_sgemm_tile_padded(char transA, char transB, long M, long N, long K, float
  * subkernel).  The launcher then counts whole rounds of two workgroups per compute unit instead of assuming a second
  * product beside this one, and splits K where that fills the last round (a 3072 x 3072 x 16384 product: 576 tiles, 52.7
  * TFLOP/s unsplit, 73.7 split four ways).  pl_gemm_tile_alone_workspace_bytes: what that choice can use (at most 1 GiB;
- * 0: not split); pl_gemm_tile_choice_alone reports the choice like pl_gemm_tile_choice. */
+ * 0: not split); pl_gemm_tile_choice_alone reports the choice like pl_gemm_tile_choice.  Where the tiles do not fill
+ * whole rounds and K is too short for the slices of all of C to pay, the product is cut along N instead: the first
+ * n_head columns of C (whole tile columns) in one unsplit launch, the rest in a second one that splits K tail_splits
+ * ways (3072^3 fp64: 21 of 24 tile columns, the last three split seven ways).  pl_gemm_tile_cut_alone reports that:
+ * *n_head == N and *tail_splits == 0 when the product stays one launch; PARALIA_GEMM_TAIL=0 switches the cut off. */
 long pl_gemm_tile_alone_workspace_bytes(char transA, char transB, long M, long N, long K, int beta_is_zero, int elem_size);
 int pl_dgemm_tile_alone(char transA, char transB, long M, long N, long K, double alpha, const double* A, long lda,
                         const double* B, long ldb, double beta, double* C, long ldc, void* workspace, long workspace_bytes,
@@ -144,6 +148,8 @@ int pl_sgemm_tile_alone(char transA, char transB, long M, long N, long K, float 
                         void* stream);
 int pl_gemm_tile_choice_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
                               long workspace_bytes, int* tile_m, int* tile_n, int* splits);
+int pl_gemm_tile_cut_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
+                           long workspace_bytes, long* n_head, int* tail_splits);
 
 /* Fitted constants of the tile-GEMM launcher's cost model: how it chooses between its macro tiles (fp32: 128 x 128,
  * 256 x 128 "wide", 256 x 256 "large") and how many ways it splits K for products with few tiles.  They describe one

@@ -301,33 +301,43 @@ __device__ __forceinline__ unsigned dma_lane_offset(long ld, int wave, int lane)
 
 // Workgroup id -> (block row, block column).  Hardware deals workgroup ids round-robin over the 8 XCDs;
 // give each XCD a contiguous range of logical ids, then walk that range in groups of 8 block rows.
-// A ragged last block row (M not a multiple of the tile) is dealt out first and evenly: its workgroups take the
-// guarded loop, about twice the time of an interior one, and in the walk above they would all fall into the last XCD's
-// range, one in eight of its workgroups, so that XCD finished a sixth later than the other seven (8100 x 8192 x 8192
-// fp64: 62.7 TFLOP/s against 73.1 for 8192 x 8100 x 8192, whose ragged column every XCD shares).  Tile j of that row
-// goes to XCD j mod 8 as one of its first workgroups; the rows above it are walked as before.
-__device__ __forceinline__ void block_coords(int bid, int gm, int gn, bool ragged_m, int& bm, int& bn) {
+// A ragged last block row or column (M or N not a multiple of the tile) is dealt out first and evenly: its workgroups
+// take the guarded loop, about twice the time of an interior one.  In the walk above the last row's would all fall into
+// the last XCD's range, one in eight of its workgroups, so that XCD finished a sixth later than the other seven (8100 x
+// 8192 x 8192 fp64: 62.7 TFLOP/s against 73.1 for 8192 x 8100 x 8192), and the last column's close every band of eight
+// rows, so whichever XCD's range ends with a band starts its slowest workgroups last (7808 x 3126 x 16384, three rounds:
+// 63.7 TFLOP/s, 68.1 now).  The slow tiles are numbered along the last row, then up the last column; tile j goes to
+// XCD j mod 8 as one of its first workgroups, and the rectangle that is left is walked as before.
+__device__ __forceinline__ void block_coords(int bid, int gm, int gn, bool ragged_m, bool ragged_n, int& bm, int& bn) {
   const int nb = gm * gn;
   const int xcd = bid & 7, loc = bid >> 3;
-  int pid, rows = gm;
-  if (ragged_m && gm > 1) {
-    const int mine = (gn - xcd + 7) >> 3;   // tiles of the last row with j mod 8 == xcd
-    if (loc < mine) {
-      bm = gm - 1;
-      bn = xcd + 8 * loc;
+  const int rm = (ragged_m && gm > 1) ? 1 : 0, rn = (ragged_n && gn > 1) ? 1 : 0;
+  const int rows = gm - rm, cols = gn - rn;
+  int pid;
+  if (rm | rn) {
+    const int in_row = rm ? gn : 0;                  // the last row, corner included
+    const int slow = in_row + (rn ? rows : 0);       // and the last column above it
+    const int mine = (slow - xcd + 7) >> 3;          // slow tiles with j mod 8 == xcd
+    // every other one of the XCD's first workgroups where it has that many (two slow ones that share a compute unit
+    // would both run at half speed), its first ones otherwise
+    const bool spread = ((nb - xcd + 7) >> 3) >= 2 * mine;
+    const int s = spread ? ((loc & 1) == 0 && (loc >> 1) < mine ? (loc >> 1) : -1) : (loc < mine ? loc : -1);
+    if (s >= 0) {
+      const int j = xcd + 8 * s;
+      if (j < in_row) { bm = gm - 1; bn = j; }
+      else { bm = j - in_row; bn = gn - 1; }
       return;
     }
-    // the other rows: XCD y keeps the (nb - y + 7) / 8 workgroups the hardware deals it, less its share of the last row
-    rows = gm - 1;
+    // the rest: XCD y keeps the (nb - y + 7) / 8 workgroups the hardware deals it, less its share of the slow ones
     int start = 0;
-    for (int y = 0; y < xcd; ++y) start += ((nb - y + 7) >> 3) - ((gn - y + 7) >> 3);
-    pid = start + loc - mine;
+    for (int y = 0; y < xcd; ++y) start += ((nb - y + 7) >> 3) - ((slow - y + 7) >> 3);
+    pid = start + (spread && loc < 2 * mine ? (loc >> 1) : loc - mine);
   } else {
     const int q = nb >> 3, r = nb & 7;
     pid = (xcd < r) ? xcd * (q + 1) + loc : r * (q + 1) + (xcd - r) * q + loc;
   }
   constexpr int GM = 8;
-  const int width = GM * gn;
+  const int width = GM * cols;
   const int group = pid / width;
   const int first_m = group * GM;
   const int gsz = min(rows - first_m, GM);
@@ -392,7 +402,7 @@ __global__ __launch_bounds__(NTHREADS, (BM * BN * (int)sizeof(T) <= 128 * 128 * 
   const int wm = (wave & 1) * WM, wn = (wave >> 1) * WN;
 
   int bm, bn;
-  block_coords(blockIdx.x, gm, gn, M % BM != 0, bm, bn);
+  block_coords(blockIdx.x, gm, gn, M % BM != 0, N % BN != 0, bm, bn);
   // the divisions above run on the vector unit; back in scalar registers the tile origins and every address derived
   // from them are scalar arithmetic
   bm = __builtin_amdgcn_readfirstlane(bm);
@@ -986,8 +996,60 @@ int pick_splits_alone(long M, long N, long K, long max_ws_bytes, int* kchunk_out
   return best_s;
 }
 
-// Macro tile and split count of one product.
-struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; };
+// A product alone on the device whose tiles do not fill whole rounds can also be cut in two along N: the first
+// n_head columns of C (whole tile columns, close to whole rounds of 512 workgroups) as one unsplit launch, the rest as
+// a second launch that splits K, so that only the tail's slices pass through the reduction (3072^3 fp64: 576 tiles,
+// four-way split of everything 874 us, 21 tile columns unsplit and the last 3 split seven ways 820 us).  Priced with
+// the terms of pick_splits_alone plus half a split's launch cost for the extra launch; taken when 3 % ahead of
+// best_us, the best of the one-launch choices.  Returns the tail's split count (0: one launch stays).
+template <typename T>
+int pick_tail_alone(long M, long N, long K, long max_ws_bytes, double best_us, long* n_head_out, double* us_out) {
+  constexpr int BM = 128, BN = 128;
+  const long gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
+  const char* const off = getenv("PARALIA_GEMM_TAIL");
+  if ((off && *off == '0') || gn < 2 || K < 512 || gm * gn <= 512) return 0;
+  const pl_gemm_fit& fit = fit_in_use();
+  const double c1 = fit.lone_us_per_k[sizeof(T) == 8 ? 0 : 1];
+  const double c2 = c1 * fit.f32_small_us_per_k / fit.lone_us_per_k[1];
+  const double f = fit.lone_fixed_k * c1;
+  auto main_us = [&](long blocks, long kc) {
+    const long full = blocks / 512, rem = blocks % 512;
+    double t = (double)full * (f + (double)kc * c2);
+    if (rem > 0) t += f + (double)kc * (rem <= 256 ? c1 : c2);
+    return t;
+  };
+  const long gran = sizeof(T) == 4 ? PLK_F32_DEEP_BK : 16;
+  int best_s = 0;
+  double best = best_us * 0.97;
+  // tails of up to two rounds' worth of tile columns
+  const long h_span = (1024 + gm - 1) / gm;
+  const long h_min = gn - h_span > 1 ? gn - h_span : 1;
+  for (long h = gn - 1; h >= h_min; --h) {
+    const long nt = N - h * BN;
+    const double head = main_us(gm * h, K) + 0.5 * fit.splitk_launch_us;
+    if (head >= best) continue;
+    for (int s = 2; s <= 64; ++s) {
+      const long kc = (((K + s - 1) / s) + gran - 1) / gran * gran;
+      if (kc < 256) break;   // shorter chunks run below the model's rate (2146 x 6400 x 512 in chunks of 176: 3 % lost)
+      const long se = (K + kc - 1) / kc;
+      if (se < 2) continue;
+      if (se * M * nt * (long)sizeof(T) > max_ws_bytes) break;
+      const double t = head + main_us(gm * (gn - h) * se, kc) + fit.splitk_launch_us +
+                       ((double)se + 1.0) * (double)M * (double)nt * sizeof(T) / fit.pass_bytes_per_us;
+      if (t < best) {
+        best = t;
+        best_s = (int)se;
+        *n_head_out = h * BN;
+      }
+    }
+  }
+  if (us_out) *us_out = best;
+  return best_s;
+}
+
+// Macro tile and split count of one product (alone on the device: possibly an unsplit head of n_head columns and a
+// tail that splits K tail_splits ways).
+struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; long n_head = 0; int tail_splits = 0; };
 template <typename T>
 TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true,
                        int want_splits = 0, bool alone = false) {
@@ -1043,6 +1105,11 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   if (c.big || c.wide) c.splits = 1, c.kchunk = 0;
   c.tm = c.big || c.wide ? 256 : 128;
   c.tn = c.big ? 256 : 128;
+  if (alone_us >= 0 && !c.big && !c.wide && have_ws) {
+    // (fp32: the bigger tiles lost against alone_us, so a cut that beats alone_us beats them too)
+    c.tail_splits = pick_tail_alone<T>(M, N, K, workspace_bytes, alone_us, &c.n_head, nullptr);
+    if (c.tail_splits > 1) c.splits = 1, c.kchunk = 0;
+  }
   return c;
 }
 
@@ -1075,6 +1142,14 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   // beyond that keep the tiles that stage through registers
   const bool dma_fits = (!at || lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES) && (!bnn || ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES);
   const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits, alone);
+  if (choice.tail_splits > 1) {
+    // head: whole tile columns, unsplit; tail: the remaining columns of op(B) and C with K split
+    const long nh = choice.n_head;
+    const int rc = launch_gemm<T>(ta, tb, M, nh, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, 0, 1, false, m_read, n_read);
+    if (rc != 0) return rc;
+    return launch_gemm<T>(ta, tb, M, N - nh, K, alpha, A, lda, bnn ? B + nh * ldb : B + nh, ldb, beta, C + nh * ldc, ldc, stream, workspace,
+                          workspace_bytes, choice.tail_splits, false, m_read, n_read - nh);
+  }
   const int kchunk = choice.kchunk, splits = choice.splits;
   const bool big = choice.big, wide = choice.wide;
   const int TM_RT = choice.tm, TN_RT = choice.tn;
@@ -1249,9 +1324,25 @@ extern "C" int pl_gemm_tile_choice_alone(int elem_size, char transA, char transB
   return 0;
 }
 
+extern "C" int pl_gemm_tile_cut_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
+                                      long workspace_bytes, long* n_head, int* tail_splits) {
+  const bool at = (transA == 'T' || transA == 't'), an = (transA == 'N' || transA == 'n');
+  const bool bt = (transB == 'T' || transB == 't'), bnn = (transB == 'N' || transB == 'n');
+  if (!(at || an) || !(bt || bnn)) return PL_ERR_TRANS;
+  if (M <= 0 || N <= 0 || K <= 0 || (elem_size != 8 && elem_size != 4)) return PL_ERR_DIM;
+  const plk::TileChoice c = elem_size == 8 ? plk::choose_tile<double>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true)
+                                           : plk::choose_tile<float>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true);
+  if (n_head) *n_head = c.tail_splits > 1 ? c.n_head : N;
+  if (tail_splits) *tail_splits = c.tail_splits > 1 ? c.tail_splits : 0;
+  return 0;
+}
+
 extern "C" long pl_gemm_tile_alone_workspace_bytes(char transA, char transB, long M, long N, long K, int beta_is_zero, int elem_size) {
-  int splits = 1;
+  int splits = 1, tail_splits = 0;
+  long n_head = N;
   if (pl_gemm_tile_choice_alone(elem_size, transA, transB, M, N, K, beta_is_zero, PLK_ALONE_MAX_WS_BYTES, nullptr, nullptr, &splits) != 0) return 0;
+  if (pl_gemm_tile_cut_alone(elem_size, transA, transB, M, N, K, beta_is_zero, PLK_ALONE_MAX_WS_BYTES, &n_head, &tail_splits) != 0) return 0;
+  if (tail_splits > 1) return (long)tail_splits * M * (N - n_head) * elem_size;
   return splits > 1 ? (long)splits * M * N * elem_size : 0;
 }
 

@@ -612,6 +612,49 @@ def test_gemm_tile_alone_on_the_device(pkg, L, ta, tb, dims):
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
+@pytest.mark.parametrize("dims", [(3072, 3072, 1024), (3000, 3010, 2050), (2816, 3534, 2048), (1408, 7222, 512)])
+def test_gemm_tile_alone_cut_in_head_and_tail(pkg, L, ta, tb, dims):
+    """pl_dgemm_tile_alone / pl_sgemm_tile_alone on products whose tiles do not fill whole rounds and whose K is too short
+    for an even split: the first tile columns of C go out as one unsplit launch, the rest as a second launch that splits
+    K (pl_gemm_tile_cut_alone says where and how).  Leading dimensions with padding, ragged M, N and K, beta = 0 over
+    NaN and beta != 0, the workspace full of NaN and exactly as large as asked for.  Integer operands: bit for bit
+    numpy's fp64 product, the padding of C untouched."""
+    M, N, K = dims
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + 4, rb + 8, M + 4
+    rng = np.random.default_rng(M + N + K)
+    for dtype in (np.float64, np.float32):
+        esz = np.dtype(dtype).itemsize
+        fn = L.pl_dgemm_tile_alone if dtype == np.float64 else L.pl_sgemm_tile_alone
+        A = rng.integers(-4, 5, lda * ca).astype(dtype)
+        B = rng.integers(-4, 5, ldb * cb).astype(dtype)
+        C0 = rng.integers(-4, 5, ldc * N).astype(dtype)
+        a = A.reshape(ca, lda)[:, :ra].T.astype(np.float64)
+        b = B.reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+        prod = -2.0 * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T))
+        dA, dB = Buf(pkg, A.size, dtype, 0).set(A), Buf(pkg, B.size, dtype, 0).set(B)
+        for beta in (0.0, 3.0):
+            need = int(L.pl_gemm_tile_alone_workspace_bytes(ta.encode(), tb.encode(), M, N, K, 1 if beta == 0.0 else 0, esz))
+            nh, ts = C.c_long(), C.c_int()
+            assert L.pl_gemm_tile_cut_alone(esz, ta.encode(), tb.encode(), M, N, K, 1 if beta == 0.0 else 0, need, C.byref(nh), C.byref(ts)) == 0
+            assert ts.value > 1 and 0 < nh.value < N and nh.value % 128 == 0 and need == ts.value * M * (N - nh.value) * esz
+            n_ws = need // esz
+            dW = Buf(pkg, n_ws, dtype, 0).set(np.full(n_ws, np.nan, dtype=dtype))
+            start = C0.copy()
+            if beta == 0.0:
+                start.reshape(N, ldc)[:, :M] = np.nan
+            dC = Buf(pkg, start.size, dtype, 0).set(start)
+            ref = (prod + beta * C0.reshape(N, ldc)[:, :M].T.astype(np.float64)).T.astype(dtype)
+            print("gemm_alone_cut", np.dtype(dtype).name, ta, tb, M, N, K, "head", nh.value, "tail splits", ts.value, "beta", beta, flush=True)
+            pkg.check(fn(ta.encode(), tb.encode(), M, N, K, -2.0, dA.ptr, lda, dB.ptr, ldb, beta, dC.ptr, ldc, dW.ptr, need, None), "gemm tile alone")
+            sync(pkg)
+            got = dC.get().reshape(N, ldc)
+            assert np.array_equal(got[:, :M], ref), (np.dtype(dtype).name, beta)
+            assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "N"), ("T", "T")])
 @pytest.mark.parametrize("M,N,K,splits", [(1000, 900, 520, 0), (2047, 2047, 777, 0), (130, 140, 2000, 0), (511, 2048, 4000, 4), (300, 257, 64, 1), (129, 1, 33, 0),
                                           (2500, 2400, 1100, -1)])
 def test_gemm_tile_on_operands_that_live_in_larger_blocks(pkg, L, ta, tb, M, N, K, splits):

@@ -404,11 +404,15 @@ def test_planner_time_of_a_first_call(L, pkg, monkeypatch):
                                                  (b"Dgemm", 32768, 32768, 32768, b"NN", (-1, -1, -1), 1, 20.0),
                                                  (b"Sgemm", 32768, 32768, 32768, b"NT", (-1, -1, 0), 0, 20.0)):
         best = 1e9
-        for attempt in range(30):   # the best of a few runs; a busy machine gets more of them before the test gives up
+        began = time.perf_counter()
+        attempt = 0
+        # the best of a few runs; a busy machine gets more of them (up to three seconds' worth) before the test gives up
+        while attempt < 30 or (best > bound_ms and time.perf_counter() - began < 3.0):
             t0 = time.perf_counter()
             assert L.PARALiA_autotune(db, func, M, N, K, tr[0:1], tr[1:2], loc3(*locs), bz, -1, 0, C.byref(info)) == 0
             best = min(best, (time.perf_counter() - t0) * 1e3)
-            if attempt >= 5 and best <= 0.8 * bound_ms:
+            attempt += 1
+            if attempt > 5 and best <= 0.8 * bound_ms:
                 break
         print("  planner %s %d x %d x %d: %.2f ms (T = %d, order %d)" % (func.decode(), M, N, K, best, info.T, info.order_id), flush=True)
         assert best <= bound_ms, (func, M, N, K, best)
@@ -507,6 +511,28 @@ def test_launcher_choice_for_a_product_alone_on_the_device(L, pkg, monkeypatch):
         assert alone(es, b"NN", 512, 512, 2048) == two_streams(es, b"NN", 512, 512, 2048)
         assert alone(es, b"NN", 8192, 8192, 8192)[2] == 1 and L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 8192, 8192, 8192, 1, es) == 0
         assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 6000, 6000, 16384, 1, es) <= 1 << 30
+    # cut along N where the slices of all of C cost too much: 3072^3 = 24 x 24 tiles, 21 tile columns (504 tiles, one
+    # round) unsplit, the last three split seven ways (another 504 workgroups); the workspace is the tail's slices
+    def cut(es, tr, M, N, K, beta0=1, ws=1 << 30):
+        nh, ts = C.c_long(), C.c_int()
+        assert L.pl_gemm_tile_cut_alone(es, tr[0:1], tr[1:2], M, N, K, beta0, ws, C.byref(nh), C.byref(ts)) == 0
+        return nh.value, ts.value
+    monkeypatch.delenv("PARALIA_GEMM_TAIL", raising=False)
+    for es in (8, 4):
+        assert cut(es, b"NN", 3072, 3072, 3072) == (2688, 7) and alone(es, b"NN", 3072, 3072, 3072)[2] == 1
+        assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 3072, 3072, 3072, 1, es) == 7 * 3072 * 384 * es
+        assert cut(es, b"TN", 3000, 3010, 3072) == (2688, 7)                     # ragged edges count as tiles
+        assert cut(es, b"NN", 3072, 3072, 3072, ws=6 * 3072 * 384 * es)[1] in (0, 2, 3, 4, 5, 6)   # fewer slices or none
+        assert cut(es, b"NN", 3072, 3072, 16384) == (3072, 0)                    # long K: the even split is as good
+        assert cut(es, b"NN", 4096, 4096, 4096) == (4096, 0)                     # whole rounds
+        assert cut(es, b"NN", 2560, 2560, 2560) == (2560, 0)                     # less than a round: the even split
+        assert cut(es, b"NN", 3072, 3072, 500) == (3072, 0)                      # K too short for chunks of 256
+        assert cut(es, b"NN", 3072, 3072, 3072, ws=0) == (3072, 0)
+        monkeypatch.setenv("PARALIA_GEMM_TAIL", "0")
+        assert cut(es, b"NN", 3072, 3072, 3072) == (3072, 0) and alone(es, b"NN", 3072, 3072, 3072)[2] > 1
+        assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 3072, 3072, 3072, 1, es) == alone(es, b"NN", 3072, 3072, 3072)[2] * 3072 * 3072 * es
+        monkeypatch.delenv("PARALIA_GEMM_TAIL", raising=False)
+    assert L.pl_gemm_tile_cut_alone(8, b"X", b"N", 10, 10, 10, 1, 0, None, None) != 0
     assert alone(8, b"NN", 4096, 4096, 16384) == (128, 128, 1)                   # two full rounds
     assert alone(4, b"NT", 4096, 4096, 16384) == (256, 256, 1)                   # one round of large tiles
     assert alone(4, b"NT", 4096, 4096, 16384, beta0=0)[2] == 1
@@ -517,4 +543,5 @@ def test_launcher_choice_for_a_product_alone_on_the_device(L, pkg, monkeypatch):
     f.splitk_launch_us = 1e5
     assert L.pl_gemm_set_fit(C.byref(f)) == 0
     assert alone(8, b"NN", 3072, 3072, 16384)[2] == 1 and alone(4, b"NN", 2560, 2560, 4096)[2] == 1
+    assert cut(8, b"NN", 3072, 3072, 3072) == (3072, 0)
     assert L.pl_gemm_set_fit(None) == 0
