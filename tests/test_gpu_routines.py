@@ -461,9 +461,9 @@ def test_stream_placement_probe_and_the_schedulers_own_streams(pkg, L):
         return out.value
     streams = [new_stream() for _ in range(9)]
     assert shares(streams[0], [streams[0]]) == 1
-    verdicts = [shares(streams[0], [s]) for s in streams[1:]]
-    print("  stream 0 against streams 1..8: shares =", verdicts, flush=True)
-    assert 0 in verdicts and 1 in verdicts
+    answers = [shares(streams[0], [s]) for s in streams[1:]]
+    print("  stream 0 against streams 1..8: shares =", answers, flush=True)
+    assert 0 in answers and 1 in answers
     assert shares(streams[0], streams[1:]) == 1                 # one of the eight holds its queue
     M = N = K = 768
     rng = np.random.default_rng(5)
