@@ -150,6 +150,9 @@ int pl_gemm_tile_choice_alone(int elem_size, char transA, char transB, long M, l
                               long workspace_bytes, int* tile_m, int* tile_n, int* splits);
 int pl_gemm_tile_cut_alone(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
                            long workspace_bytes, long* n_head, int* tail_splits);
+/* the launcher's own estimate of that product's time on the device in microseconds, kernels only (< 0: bad arguments) */
+double pl_gemm_tile_alone_us(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero,
+                             long workspace_bytes);
 
 /* Fitted constants of the tile-GEMM launcher's cost model: how it chooses between its macro tiles (fp32: 128 x 128,
  * 256 x 128 "wide", 256 x 256 "large") and how many ways it splits K for products with few tiles.  They describe one

@@ -82,6 +82,7 @@ _SIGS = {
     "pl_sgemm_tile_alone": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _vp]),
     "pl_gemm_tile_choice_alone": (_i, [_i, _c, _c, _l, _l, _l, _i, _l, _pi, _pi, _pi]),
     "pl_gemm_tile_cut_alone": (_i, [_i, _c, _c, _l, _l, _l, _i, _l, C.POINTER(_l), _pi]),
+    "pl_gemm_tile_alone_us": (_d, [_i, _c, _c, _l, _l, _l, _i, _l]),
     "pl_dgemm_tile_padded": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _i, _l, _l, _vp]),
     "pl_sgemm_tile_padded": (_i, [_c, _c, _l, _l, _l, _f, _vp, _l, _vp, _l, _f, _vp, _l, _vp, _l, _i, _l, _l, _vp]),
     "pl_dgemm_tile_split": (_i, [_c, _c, _l, _l, _l, _d, _vp, _l, _vp, _l, _d, _vp, _l, _vp, _l, _i, _vp]),

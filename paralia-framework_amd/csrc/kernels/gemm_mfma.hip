@@ -1049,7 +1049,7 @@ int pick_tail_alone(long M, long N, long K, long max_ws_bytes, double best_us, l
 
 // Macro tile and split count of one product (alone on the device: possibly an unsplit head of n_head columns and a
 // tail that splits K tail_splits ways).
-struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; long n_head = 0; int tail_splits = 0; };
+struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; long n_head = 0; int tail_splits = 0; double us = -1; };
 template <typename T>
 TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true,
                        int want_splits = 0, bool alone = false) {
@@ -1105,10 +1105,13 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   if (c.big || c.wide) c.splits = 1, c.kchunk = 0;
   c.tm = c.big || c.wide ? 256 : 128;
   c.tn = c.big ? 256 : 128;
+  // the model's time for the choice (a product alone on the device only: the two-stream terms price shared rounds)
+  if (alone_us >= 0) c.us = c.big ? large_us : c.wide ? wide_us : alone_us;
   if (alone_us >= 0 && !c.big && !c.wide && have_ws) {
     // (fp32: the bigger tiles lost against alone_us, so a cut that beats alone_us beats them too)
-    c.tail_splits = pick_tail_alone<T>(M, N, K, workspace_bytes, alone_us, &c.n_head, nullptr);
-    if (c.tail_splits > 1) c.splits = 1, c.kchunk = 0;
+    double cut_us = -1;
+    c.tail_splits = pick_tail_alone<T>(M, N, K, workspace_bytes, alone_us, &c.n_head, &cut_us);
+    if (c.tail_splits > 1) c.splits = 1, c.kchunk = 0, c.us = cut_us;
   }
   return c;
 }
@@ -1335,6 +1338,15 @@ extern "C" int pl_gemm_tile_cut_alone(int elem_size, char transA, char transB, l
   if (n_head) *n_head = c.tail_splits > 1 ? c.n_head : N;
   if (tail_splits) *tail_splits = c.tail_splits > 1 ? c.tail_splits : 0;
   return 0;
+}
+
+extern "C" double pl_gemm_tile_alone_us(int elem_size, char transA, char transB, long M, long N, long K, int beta_is_zero, long workspace_bytes) {
+  const bool at = (transA == 'T' || transA == 't'), an = (transA == 'N' || transA == 'n');
+  const bool bt = (transB == 'T' || transB == 't'), bnn = (transB == 'N' || transB == 'n');
+  if (!(at || an) || !(bt || bnn) || M <= 0 || N <= 0 || K <= 0 || (elem_size != 8 && elem_size != 4)) return -1.0;
+  const plk::TileChoice c = elem_size == 8 ? plk::choose_tile<double>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true)
+                                           : plk::choose_tile<float>(an, bnn, M, N, K, beta_is_zero != 0, workspace_bytes > 0, workspace_bytes, true, 0, true);
+  return c.us;
 }
 
 extern "C" long pl_gemm_tile_alone_workspace_bytes(char transA, char transB, long M, long N, long K, int beta_is_zero, int elem_size) {

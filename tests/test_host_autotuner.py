@@ -533,6 +533,21 @@ def test_launcher_choice_for_a_product_alone_on_the_device(L, pkg, monkeypatch):
         assert L.pl_gemm_tile_alone_workspace_bytes(b"N", b"N", 3072, 3072, 3072, 1, es) == alone(es, b"NN", 3072, 3072, 3072)[2] * 3072 * 3072 * es
         monkeypatch.delenv("PARALIA_GEMM_TAIL", raising=False)
     assert L.pl_gemm_tile_cut_alone(8, b"X", b"N", 10, 10, 10, 1, 0, None, None) != 0
+    # the autotuner's prediction for operands already in HBM is the launcher's estimate of that one product plus 8 us
+    # for the call; the cut is in it (3072^3: under the even split's time)
+    info = pkg.atc_info()
+    db = _shipped_db(pkg).encode()
+    for func, es in ((b"Dgemm", 8), (b"Sgemm", 4)):
+        for M, N, K in ((3072, 3072, 3072), (3072, 3072, 16384), (4096, 4096, 4096), (700, 900, 1100)):
+            assert L.PARALiA_autotune(db, func, M, N, K, b"N", b"T", loc3(0, 0, 0), 1, -1, 0, C.byref(info)) == 0
+            us = L.pl_gemm_tile_alone_us(es, b"N", b"T", M, N, K, 1, 1 << 30)    # with the database's fit, as the call above
+            assert us > 0 and info.T == max(M, N, K) and abs(info.pred_t - (us * 1e-6 + 8e-6)) < 1e-12
+        with_cut = L.pl_gemm_tile_alone_us(es, b"N", b"N", 3072, 3072, 3072, 1, 1 << 30)
+        monkeypatch.setenv("PARALIA_GEMM_TAIL", "0")
+        assert with_cut < 0.97 * L.pl_gemm_tile_alone_us(es, b"N", b"N", 3072, 3072, 3072, 1, 1 << 30)
+        monkeypatch.delenv("PARALIA_GEMM_TAIL", raising=False)
+    assert L.pl_gemm_tile_alone_us(8, b"N", b"N", 0, 10, 10, 1, 0) < 0
+    assert L.pl_gemm_set_fit(None) == 0
     assert alone(8, b"NN", 4096, 4096, 16384) == (128, 128, 1)                   # two full rounds
     assert alone(4, b"NT", 4096, 4096, 16384) == (256, 256, 1)                   # one round of large tiles
     assert alone(4, b"NT", 4096, 4096, 16384, beta0=0)[2] == 1
