@@ -172,6 +172,8 @@ typedef struct pl_gemm_fit {
   double f32_wide_fixed_us[2];      /* beta == 0, beta != 0 */
   double f32_large_gain[4];         /* large tile: 2 * f32_small_us_per_k * K / (1 + gain) per round of 256, per transpose */
   double f32_large_fixed_us[4][2];  /* per transpose; beta == 0, beta != 0 */
+  double edge_rounds[2];            /* what the guarded edge workgroups of a grid with a ragged last row or column add to a
+                                       product alone on the device, in rounds: [0] 128 x 128 tiles, [1] 256-wide tiles */
 } pl_gemm_fit;
 void pl_gemm_fit_defaults(pl_gemm_fit* fit);
 int pl_gemm_set_fit(const pl_gemm_fit* fit);   /* null: back to the built-in values */

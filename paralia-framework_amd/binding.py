@@ -25,7 +25,7 @@ class gemm_fit(C.Structure):
     _fields_ = [("lone_us_per_k", C.c_double * 2), ("lone_fixed_k", C.c_double), ("splitk_launch_us", C.c_double),
                 ("pass_bytes_per_us", C.c_double), ("f32_small_us_per_k", C.c_double), ("f32_small_fixed_us", C.c_double),
                 ("f32_wide_gain", C.c_double), ("f32_wide_fixed_us", C.c_double * 2), ("f32_large_gain", C.c_double * 4),
-                ("f32_large_fixed_us", (C.c_double * 2) * 4)]
+                ("f32_large_fixed_us", (C.c_double * 2) * 4), ("edge_rounds", C.c_double * 2)]
 
 
 def build_library(jobs=8):

@@ -36,6 +36,8 @@ KernelFit KernelFit_load(const std::string& db_dir, int dev_id) {
     else if (n == "f32_wide_gain") f.f32_wide_gain = v;
     else if (n == "f32_wide_fixed_us_beta0") f.f32_wide_fixed_us[0] = v;
     else if (n == "f32_wide_fixed_us_beta1") f.f32_wide_fixed_us[1] = v;
+    else if (n == "edge_rounds_small") f.edge_rounds[0] = v;
+    else if (n == "edge_rounds_large") f.edge_rounds[1] = v;
     else if (n == "merge_saving_us_f64") k.merge_saving_us_f64 = v;
     else if (n == "merge_saving_us_f32") { for (double& x : k.merge_saving_us_f32) x = v; }
     else if (n == "lone_share") k.lone_share = v;

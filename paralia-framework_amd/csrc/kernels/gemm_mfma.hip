@@ -914,6 +914,8 @@ inline void fit_defaults(pl_gemm_fit* f) {
   f->f32_wide_fixed_us[0] = 4.9; f->f32_wide_fixed_us[1] = 10.6;
   const double g[4] = {0.012, 0.011, 0.010, 0.010}, f0[4] = {11.4, 10.7, 11.1, 11.7}, f1[4] = {45.5, 44.5, 53.0, 54.4};
   for (int t = 0; t < 4; ++t) { f->f32_large_gain[t] = g[t]; f->f32_large_fixed_us[t][0] = f0[t]; f->f32_large_fixed_us[t][1] = f1[t]; }
+  f->edge_rounds[0] = 0.18;
+  f->edge_rounds[1] = 0.24;
 }
 inline pl_gemm_fit& fit_in_use() {
   static pl_gemm_fit f = [] { pl_gemm_fit d; fit_defaults(&d); return d; }();
@@ -1052,7 +1054,7 @@ int pick_tail_alone(long M, long N, long K, long max_ws_bytes, double best_us, l
 struct TileChoice { int tm = 128, tn = 128, splits = 1, kchunk = 0; bool big = false, wide = false; long n_head = 0; int tail_splits = 0; double us = -1; };
 template <typename T>
 TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero, bool have_ws, long workspace_bytes, bool large_allowed = true,
-                       int want_splits = 0, bool alone = false) {
+                       int want_splits = 0, bool alone = false, long m_read = 0, long n_read = 0, bool small_only = false) {
   TileChoice c;
   double alone_us = -1;   // alone: the predicted time of the 128 x 128 tile with the split count chosen for it
   if (want_splits >= 1) {
@@ -1087,15 +1089,39 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   const int bi = beta_zero ? 0 : 1;
   auto tiles_of = [&](long tm, long tn) { return ((M + tm - 1) / tm) * ((N + tn - 1) / tn); };
   const double k_us = fit.f32_small_us_per_k * (double)K;
+  // Alone on the device, a grid with a ragged last row or column (edge workgroups that may not read to the tile's edge
+  // take the guarded loop, and nothing else fills the units that wait for them) costs a fraction of a round more,
+  // whatever the number of rounds: fp32 256 x 256 tiles, 4096 x 4096 x 4096 910 us, 3712 or 4000 x 4096 x 4096 1122
+  // (one round: + 0.24), 5760 x 5632 2026 against 1823 (two: + 0.23 of one), 8192 x 8064 3835 against 3628 (four: + 0.23
+  // of one); 128 x 128 tiles 4000 x 4096 x 4096 998 against 926 (+ 0.16 of a round), 8000^2 x 4096 3742 against 3657 (+ 0.19).
+  // Without the term the large tile was taken for every such shape that fills its rounds and ran up to 27 % behind
+  // the small one (3712 x 4224 x 1024).
+  const long mr = m_read > 0 ? m_read : M, nr = n_read > 0 ? n_read : N;
+  auto edge = [&](long tm, long tn) { return alone_us >= 0 && ((M % tm != 0 && mr < (M + tm - 1) / tm * tm) || (N % tn != 0 && nr < (N + tn - 1) / tn * tn)); };
+  const double large_round = fit.f32_large_fixed_us[tr][bi] + 2.0 * k_us / (1.0 + fit.f32_large_gain[tr]);
+  const double wide_round = fit.f32_wide_fixed_us[bi] + 2.0 * k_us / fit.f32_wide_gain;
+  // (a round of small tiles as pick_splits_alone prices it)
+  const double lone_c1 = fit.lone_us_per_k[sizeof(T) == 8 ? 0 : 1];
+  const double small_round = fit.lone_fixed_k * lone_c1 + (double)(c.kchunk > 0 ? c.kchunk : K) * lone_c1 * fit.f32_small_us_per_k / fit.lone_us_per_k[1];
+  const double small_edge_us = edge(128, 128) ? fit.edge_rounds[0] * small_round : 0.0;
+  // the small tile's best, alone: one launch (split or not) or the head / tail cut
+  long cut_head = 0;
+  int cut_splits = 0;
+  if (alone_us >= 0 && have_ws) {
+    double cut_us = -1;
+    cut_splits = pick_tail_alone<T>(M, N, K, workspace_bytes, alone_us, &cut_head, &cut_us);
+    if (cut_splits > 1) alone_us = cut_us;
+  }
+  if (alone_us >= 0) alone_us += small_edge_us;
   const double small_us = alone_us >= 0 ? alone_us : (double)((tiles_of(128, 128) + 511) / 512) * (fit.f32_small_fixed_us + k_us);
-  const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * (fit.f32_large_fixed_us[tr][bi] + 2.0 * k_us / (1.0 + fit.f32_large_gain[tr]));
-  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * (fit.f32_wide_fixed_us[bi] + 2.0 * k_us / fit.f32_wide_gain);
+  const double large_us = (double)((tiles_of(256, 256) + 255) / 256) * large_round + (edge(256, 256) ? fit.edge_rounds[1] * large_round : 0.0);
+  const double wide_us = (double)((tiles_of(256, 128) + 511) / 512) * wide_round + (edge(256, 128) ? fit.edge_rounds[0] * wide_round : 0.0);
   // PARALIA_GEMM_LARGE_TILE: "0" small tiles only, "1" the large tile for every call, "2" the wide tile wherever it
   // exists (NN), unset: the model
   const char* const pin = getenv("PARALIA_GEMM_LARGE_TILE");
   const int pinv = (pin && *pin) ? atoi(pin) : -1;
   // (alone, the bigger tiles are weighed against the split small tile too; a caller's own split count keeps the small one)
-  const bool other = sizeof(T) == 4 && (c.splits == 1 || alone_us >= 0) && pinv != 0;
+  const bool other = sizeof(T) == 4 && (c.splits == 1 || alone_us >= 0) && pinv != 0 && !small_only;
   // partly filled rounds cost the bigger tiles more than the model's rounding says (measured: -1 % at 3072 and 5120)
   auto fills = [](long tiles, long places) { return 10 * tiles >= 9 * ((tiles + places - 1) / places) * places; };
   const bool wide_ok = other && an && bnn && (pinv == 2 || (pinv < 0 && fills(tiles_of(256, 128), 512)));
@@ -1107,19 +1133,14 @@ TileChoice choose_tile(bool an, bool bnn, long M, long N, long K, bool beta_zero
   c.tn = c.big ? 256 : 128;
   // the model's time for the choice (a product alone on the device only: the two-stream terms price shared rounds)
   if (alone_us >= 0) c.us = c.big ? large_us : c.wide ? wide_us : alone_us;
-  if (alone_us >= 0 && !c.big && !c.wide && have_ws) {
-    // (fp32: the bigger tiles lost against alone_us, so a cut that beats alone_us beats them too)
-    double cut_us = -1;
-    c.tail_splits = pick_tail_alone<T>(M, N, K, workspace_bytes, alone_us, &c.n_head, &cut_us);
-    if (c.tail_splits > 1) c.splits = 1, c.kchunk = 0, c.us = cut_us;
-  }
+  if (cut_splits > 1 && !c.big && !c.wide) c.tail_splits = cut_splits, c.n_head = cut_head, c.splits = 1, c.kchunk = 0;
   return c;
 }
 
 template <typename T>
 int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, long lda, const T* B, long ldb, T beta,
                 T* C, long ldc, hipStream_t stream, T* workspace = nullptr, long workspace_bytes = 0, int want_splits = 0,
-                bool alone = false, long m_read = 0, long n_read = 0) {
+                bool alone = false, long m_read = 0, long n_read = 0, bool small_only = false) {
   using Tr = Traits<T>;
   const bool at = (ta == 'T' || ta == 't'), an = (ta == 'N' || ta == 'n');
   const bool bt = (tb == 'T' || tb == 't'), bnn = (tb == 'N' || tb == 'n');
@@ -1144,11 +1165,12 @@ int launch_gemm(char ta, char tb, long M, long N, long K, T alpha, const T* A, l
   // a K-major operand loaded straight into LDS takes eight rows per request with 32-bit lane offsets: leading dimensions
   // beyond that keep the tiles that stage through registers
   const bool dma_fits = (!at || lda * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES) && (!bnn || ldb * (long)sizeof(T) <= PLK_DMA_MAX_LD_BYTES);
-  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits, alone);
+  const TileChoice choice = choose_tile<T>(an, bnn, M, N, K, beta == T(0), workspace != nullptr, workspace_bytes, dma_fits, want_splits, alone, m_read, n_read, small_only);
   if (choice.tail_splits > 1) {
-    // head: whole tile columns, unsplit; tail: the remaining columns of op(B) and C with K split
+    // head: whole tile columns, unsplit, in the 128 x 128 tiles the cut was priced with; tail: the remaining columns of
+    // op(B) and C with K split
     const long nh = choice.n_head;
-    const int rc = launch_gemm<T>(ta, tb, M, nh, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, 0, 1, false, m_read, n_read);
+    const int rc = launch_gemm<T>(ta, tb, M, nh, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, 0, 1, false, m_read, n_read, true);
     if (rc != 0) return rc;
     return launch_gemm<T>(ta, tb, M, N - nh, K, alpha, A, lda, bnn ? B + nh * ldb : B + nh, ldb, beta, C + nh * ldc, ldc, stream, workspace,
                           workspace_bytes, choice.tail_splits, false, m_read, n_read - nh);
@@ -1238,6 +1260,7 @@ extern "C" int pl_gemm_set_fit(const pl_gemm_fit* fit) {
   bool large_sane = true;
   for (int t = 0; t < 4; ++t) large_sane = large_sane && fit->f32_large_gain[t] > -0.5 && fit->f32_large_fixed_us[t][0] >= 0 && fit->f32_large_fixed_us[t][1] >= 0;
   if (!sane || !large_sane || fit->f32_wide_fixed_us[0] < 0 || fit->f32_wide_fixed_us[1] < 0) return PL_ERR_ARG;
+  if (!(fit->edge_rounds[0] >= 0 && fit->edge_rounds[0] <= 2 && fit->edge_rounds[1] >= 0 && fit->edge_rounds[1] <= 2)) return PL_ERR_ARG;
   plk::fit_in_use() = *fit;
   return 0;
 }

@@ -494,6 +494,15 @@ static void bench_fit(const std::string& db, bool quick) {
     f.f32_large_fixed_us[t][0] = std::max(0.0, a0);
     f.f32_large_fixed_us[t][1] = std::max(0.0, a1);
   }
+  // what the guarded edge workgroups of a ragged grid add to a product alone on the device, in rounds: 4000 x 4096 x 4096
+  // against 4096^3, fp32 NT -- one round of 256 large tiles, two rounds of 512 small ones
+  {
+    const double whole_l = per_launch_us(false, 'N', 'T', 4096, 4096, 4096, 0.0, 1), ragged_l = per_launch_us(false, 'N', 'T', 4000, 4096, 4096, 0.0, 1);
+    f.edge_rounds[1] = std::min(2.0, std::max(0.0, (ragged_l - whole_l) / whole_l));
+    setenv("PARALIA_GEMM_LARGE_TILE", "0", 1);
+    const double whole_s = per_launch_us(false, 'N', 'T', 4096, 4096, 4096, 0.0, 1), ragged_s = per_launch_us(false, 'N', 'T', 4000, 4096, 4096, 0.0, 1);
+    f.edge_rounds[0] = std::min(2.0, std::max(0.0, (ragged_s - whole_s) / (0.5 * whole_s)));
+  }
   unsetenv("PARALIA_GEMM_LARGE_TILE");
   // what joining the k-steps of a C tile into one launch saves per launch saved, as the scheduler issues them (beta = 1,
   // two streams, the launcher's own tile choice): 32 launches of 4096^3 against 8 of 4096 x 4096 x 16384, the same
@@ -532,6 +541,7 @@ static void bench_fit(const std::string& db, bool quick) {
           f.lone_us_per_k[0], f.lone_us_per_k[1], f.lone_fixed_k, f.splitk_launch_us, f.pass_bytes_per_us);
   fprintf(fp, "f32_small_us_per_k: %.6g\nf32_small_fixed_us: %.6g\nf32_wide_gain: %.6g\nf32_wide_fixed_us_beta0: %.6g\nf32_wide_fixed_us_beta1: %.6g\n",
           f.f32_small_us_per_k, f.f32_small_fixed_us, f.f32_wide_gain, f.f32_wide_fixed_us[0], f.f32_wide_fixed_us[1]);
+  fprintf(fp, "edge_rounds_small: %.6g\nedge_rounds_large: %.6g\n", f.edge_rounds[0], f.edge_rounds[1]);
   static const char* const trans[4] = {"NN", "NT", "TN", "TT"};
   for (int t = 0; t < 4; ++t)
     fprintf(fp, "f32_large_gain_%s: %.6g\nf32_large_fixed_us_beta0_%s: %.6g\nf32_large_fixed_us_beta1_%s: %.6g\nmerge_saving_us_f32_%s: %.6g\n", trans[t],
@@ -544,6 +554,7 @@ static void bench_fit(const std::string& db, bool quick) {
           f.lone_us_per_k[0], f.lone_us_per_k[1], f.lone_fixed_k, f.splitk_launch_us, f.pass_bytes_per_us / 1e6, k.geadd_bytes_per_s / 1e12);
   fprintf(stderr, "kernel fit: fp32 small %.4f us per k + %.1f us; wide gain %.3f, fixed %.1f | %.1f us; slab +%.2f us\n", f.f32_small_us_per_k,
           f.f32_small_fixed_us, f.f32_wide_gain, f.f32_wide_fixed_us[0], f.f32_wide_fixed_us[1], k.slab_fixed_us);
+  fprintf(stderr, "kernel fit: ragged edge + %.3f (128 x 128 tiles) / + %.3f (256-wide) of a round\n", f.edge_rounds[0], f.edge_rounds[1]);
   for (int t = 0; t < 4; ++t)
     fprintf(stderr, "kernel fit: fp32 large %s gain %.3f, fixed %.1f | %.1f us\n", trans[t], f.f32_large_gain[t], f.f32_large_fixed_us[t][0], f.f32_large_fixed_us[t][1]);
   for (auto s : st) pl_stream_destroy(s);

@@ -233,6 +233,9 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
         elif k.startswith("merge_saving_us_f32"):
             # 2 % of the difference of two 30 ms timings (the median of five): a few microseconds either way
             assert 0.0 <= kf[k] <= 30.0 and abs(kf[k] - kf_shipped[k]) <= 8.0, (k, kf[k], kf_shipped[k])
+    # (a difference of two launch times of a millisecond each, as a share of a round)
+    for k in ("edge_rounds_small", "edge_rounds_large"):
+        assert 0.05 <= kf[k] <= 0.5 and abs(kf[k] - kf_shipped[k]) <= 0.08, (k, kf[k], kf_shipped[k])
     assert 0.5 * kf_shipped["lone_fixed_k"] < kf["lone_fixed_k"] < 2.0 * kf_shipped["lone_fixed_k"]
     assert 1.0 < kf["splitk_launch_us"] < 10.0 and 0 <= kf["slab_fixed_us"] < 6.0
     for k in ("pass_bytes_per_us", "geadd_bytes_per_s"):
@@ -262,3 +265,4 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
     got = binding.gemm_fit()
     pkg.check(L.pl_gemm_get_fit(C.byref(got)), "get fit")
     assert abs(got.lone_us_per_k[0] - kf_shipped["lone_us_per_k_f64"]) < 1e-9 and abs(got.f32_large_gain[1] - kf_shipped["f32_large_gain_NT"]) < 1e-9
+    assert abs(got.edge_rounds[0] - kf_shipped["edge_rounds_small"]) < 1e-9 and abs(got.edge_rounds[1] - kf_shipped["edge_rounds_large"]) < 1e-9

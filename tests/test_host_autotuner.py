@@ -551,6 +551,21 @@ def test_launcher_choice_for_a_product_alone_on_the_device(L, pkg, monkeypatch):
     assert alone(8, b"NN", 4096, 4096, 16384) == (128, 128, 1)                   # two full rounds
     assert alone(4, b"NT", 4096, 4096, 16384) == (256, 256, 1)                   # one round of large tiles
     assert alone(4, b"NT", 4096, 4096, 16384, beta0=0)[2] == 1
+    # a grid of large tiles with a ragged edge pays a quarter of a round for its guarded workgroups: 3712 = 14.5 x 256
+    # keeps the small tile (29 x 128), until the fit says edges are free
+    assert alone(4, b"NT", 3712, 4096, 4096)[:2] == (128, 128) and alone(4, b"NT", 3840, 4096, 4096)[:2] == (256, 256)
+    f = binding.gemm_fit()
+    L.pl_gemm_fit_defaults(C.byref(f))
+    assert 0.05 < f.edge_rounds[0] < 0.5 and 0.05 < f.edge_rounds[1] < 0.5
+    whole, ragged = L.pl_gemm_tile_alone_us(8, b"N", b"N", 4096, 4096, 4096, 1, 0), L.pl_gemm_tile_alone_us(8, b"N", b"N", 4000, 4096, 4096, 1, 0)
+    assert 1.05 * whole < ragged < 1.15 * whole                                  # two rounds + 0.18 of one
+    f.edge_rounds[0] = f.edge_rounds[1] = 0.0
+    assert L.pl_gemm_set_fit(C.byref(f)) == 0
+    assert alone(4, b"NT", 3712, 4096, 4096)[:2] == (256, 256)
+    assert L.pl_gemm_tile_alone_us(8, b"N", b"N", 4000, 4096, 4096, 1, 0) == whole
+    f.edge_rounds[1] = 3.0
+    assert L.pl_gemm_set_fit(C.byref(f)) != 0                                    # out of range: refused as a whole
+    assert L.pl_gemm_set_fit(None) == 0
     assert L.pl_gemm_tile_choice_alone(8, b"X", b"N", 10, 10, 10, 1, 0, None, None, None) != 0
     assert L.pl_gemm_tile_choice_alone(2, b"N", b"N", 10, 10, 10, 1, 0, None, None, None) != 0
     f = binding.gemm_fit()
