@@ -235,7 +235,7 @@ def test_deploy_tool_rebuilds_the_shipped_database(run_program, pkg, L, bindir, 
             assert 0.0 <= kf[k] <= 30.0 and abs(kf[k] - kf_shipped[k]) <= 8.0, (k, kf[k], kf_shipped[k])
     # (a difference of two launch times of a millisecond each, as a share of a round)
     for k in ("edge_rounds_small", "edge_rounds_large"):
-        assert 0.05 <= kf[k] <= 0.5 and abs(kf[k] - kf_shipped[k]) <= 0.08, (k, kf[k], kf_shipped[k])
+        assert 0.03 <= kf[k] <= 0.6 and abs(kf[k] - kf_shipped[k]) <= 0.10, (k, kf[k], kf_shipped[k])
     assert 0.5 * kf_shipped["lone_fixed_k"] < kf["lone_fixed_k"] < 2.0 * kf_shipped["lone_fixed_k"]
     assert 1.0 < kf["splitk_launch_us"] < 10.0 and 0 <= kf["slab_fixed_us"] < 6.0
     for k in ("pass_bytes_per_us", "geadd_bytes_per_s"):
