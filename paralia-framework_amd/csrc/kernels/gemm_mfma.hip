@@ -914,8 +914,8 @@ inline void fit_defaults(pl_gemm_fit* f) {
   f->f32_wide_fixed_us[0] = 4.9; f->f32_wide_fixed_us[1] = 10.6;
   const double g[4] = {0.012, 0.011, 0.010, 0.010}, f0[4] = {11.4, 10.7, 11.1, 11.7}, f1[4] = {45.5, 44.5, 53.0, 54.4};
   for (int t = 0; t < 4; ++t) { f->f32_large_gain[t] = g[t]; f->f32_large_fixed_us[t][0] = f0[t]; f->f32_large_fixed_us[t][1] = f1[t]; }
-  f->edge_rounds[0] = 0.18;
-  f->edge_rounds[1] = 0.24;
+  f->edge_rounds[0] = 0.155;
+  f->edge_rounds[1] = 0.236;
 }
 inline pl_gemm_fit& fit_in_use() {
   static pl_gemm_fit f = [] { pl_gemm_fit d; fit_defaults(&d); return d; }();
