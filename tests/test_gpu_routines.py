@@ -654,6 +654,114 @@ def test_gemm_routines_random_shapes_exact_on_integers(pkg, L, seed, monkeypatch
     assert np.array_equal(got[:, M:], C0.reshape(N, ldc)[:, M:])
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_gemm_routines_random_unaligned_operands_exact_on_integers(pkg, L, seed):
+    """PARALiA_dgemm / PARALiA_sgemm on random problems whose operands start anywhere in a 16-byte unit and have any
+    leading dimension, odd ones included: one dimension of at least 2048 (where device-resident A and B are multiplied
+    from aligned copies, and where products alone on the device are cut in head and tail), two calls in three with
+    every operand in HBM, the others with pinned, pageable and device operands mixed; now and then the device memory is
+    given back between calls.  Integer operands: bit for bit numpy's fp64 result, nothing written outside C's M x N
+    elements, A and B unchanged."""
+    rng = np.random.default_rng(730000 + seed)
+    dtype = np.float64 if rng.integers(2) else np.float32
+    ta, tb = "NT"[rng.integers(2)], "NT"[rng.integers(2)]
+    T = int([512, 1024, -1, -1][rng.integers(4)])
+    dims = [int(rng.integers(2048, 4400)), int(rng.integers(1, 4400)), int(rng.integers(1, 3000))]
+    rng.shuffle(dims)
+    M, N, K = dims
+    locs = [0, 0, 0] if rng.integers(3) > 0 else [int([-1, -2, 0][rng.integers(3)]) for _ in range(3)]
+    ra, ca = (M, K) if ta == "N" else (K, M)
+    rb, cb = (K, N) if tb == "N" else (N, K)
+    lda, ldb, ldc = ra + int(rng.integers(0, 4)), rb + int(rng.integers(0, 4)), M + int(rng.integers(0, 4))
+    oa, ob, oc = int(rng.integers(0, 4)), int(rng.integers(0, 4)), int(rng.integers(0, 4))
+    A = rng.integers(-3, 4, lda * ca + oa).astype(dtype)
+    B = rng.integers(-3, 4, ldb * cb + ob).astype(dtype)
+    C0 = rng.integers(-3, 4, ldc * N + oc).astype(dtype)
+    alpha, beta = [(1.0, 0.0), (2.0, -1.0), (-1.0, 1.0), (1.0, 0.0)][rng.integers(4)]
+    a = A[oa:].reshape(ca, lda)[:, :ra].T.astype(np.float64)
+    b = B[ob:].reshape(cb, ldb)[:, :rb].T.astype(np.float64)
+    c0 = C0[oc:].reshape(N, ldc)
+    ref = (alpha * ((a if ta == "N" else a.T) @ (b if tb == "N" else b.T)) + beta * c0[:, :M].T.astype(np.float64)).T.astype(dtype)
+    start = C0.copy()
+    if beta == 0.0:
+        start[oc:].reshape(N, ldc)[:, :M] = np.nan
+    bA, bB, bC = place(pkg, A, locs[0]), place(pkg, B, locs[1]), place(pkg, start, locs[2])
+    info = pkg.atc_info()
+    fn = L.PARALiA_dgemm if dtype == np.float64 else L.PARALiA_sgemm
+    print("gemm unaligned", np.dtype(dtype).name, ta, tb, M, N, K, "T", T, "locs", locs, "ld", lda, ldb, ldc, "offsets", oa, ob, oc, alpha, beta, flush=True)
+    pkg.check(fn(ta.encode(), tb.encode(), M, N, K, alpha, bA.at(oa), lda, bB.at(ob), ldb, beta, bC.at(oc), ldc, T, 0, C.byref(info)), "gemm")
+    flat = bC.get()
+    got = flat[oc:].reshape(N, ldc)
+    assert np.array_equal(got[:, :M], ref)
+    assert np.array_equal(got[:, M:], c0[:, M:]) and np.array_equal(flat[:oc], C0[:oc])
+    assert np.array_equal(bA.get(), A) and np.array_equal(bB.get(), B)
+    if seed % 7 == 6:
+        L.PARALiA_dev_cache_free(0)
+
+
+def _strided(rng, count, inc, off):
+    return rng.integers(-3, 4, off + 1 + (count - 1) * abs(inc) + int(rng.integers(0, 3))).astype(np.float64)
+
+
+def _view(v, count, inc, off):
+    s = v[off: off + 1 + (count - 1) * abs(inc): abs(inc)]
+    return s[::-1] if inc < 0 else s
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_blas12_routines_random_problems_exact_on_integers(pkg, L, seed):
+    """PARALiA_dgemv / PARALiA_daxpy / PARALiA_ddot on random problems: any placement of every operand, increments of
+    1, 2, 3 and -1, operands that start anywhere in a cache line, odd leading dimensions, preset tile sizes or the
+    library's own, alpha / beta pairs with beta = 0 over NaN and alpha = 0.  Integer operands: bit for bit numpy's
+    result (ddot: added to the 5.0 the result holds), nothing else written, inputs unchanged."""
+    rng = np.random.default_rng(910000 + seed)
+    kind = ["gemv", "gemv", "axpy", "dot"][rng.integers(4)]
+    info = pkg.atc_info()
+    if kind == "gemv":
+        tr = "NT"[rng.integers(2)]
+        M, N = int(rng.integers(1, 5000)), int(rng.integers(1, 5000))
+        lda, oa = M + int(rng.integers(0, 4)), int(rng.integers(0, 3))
+        incx, incy = int([1, 1, 2, -1, 3][rng.integers(5)]), int([1, 1, 2, -1][rng.integers(4)])
+        ox, oy = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        nx, ny = (N, M) if tr == "N" else (M, N)
+        T = int([256, 512, 1000, 2048, -1, -1][rng.integers(6)])
+        locs = [int([0, 0, -1, -2][rng.integers(4)]) for _ in range(3)]
+        A = rng.integers(-3, 4, lda * N + oa).astype(np.float64)
+        x, y0 = _strided(rng, nx, incx, ox), _strided(rng, ny, incy, oy)
+        alpha, beta = [(1.0, 0.0), (2.0, -1.0), (-1.0, 1.0), (0.0, 2.0), (1.0, 1.0)][rng.integers(5)]
+        a = A[oa:].reshape(N, lda)[:, :M].T
+        ref = y0.copy()
+        yv = _view(ref, ny, incy, oy)
+        start = y0.copy()
+        if beta == 0.0:
+            _view(start, ny, incy, oy)[:] = np.nan
+        yv[:] = alpha * ((a if tr == "N" else a.T) @ _view(x, nx, incx, ox)) + (beta * yv if beta != 0.0 else 0.0)
+        bA, bx, by = place(pkg, A, locs[0]), place(pkg, x, locs[1]), place(pkg, start, locs[2])
+        print("dgemv", tr, M, N, "lda", lda, "inc", incx, incy, "offsets", oa, ox, oy, "T", T, "locs", locs, alpha, beta, flush=True)
+        pkg.check(L.PARALiA_dgemv(tr.encode(), M, N, alpha, bA.at(oa), lda, bx.at(ox), incx, beta, by.at(oy), incy, T, 0, C.byref(info)), "dgemv")
+        assert np.array_equal(by.get(), ref) and np.array_equal(bA.get(), A) and np.array_equal(bx.get(), x)
+        return
+    N = int(rng.integers(1, 3_000_000)) if rng.integers(3) else int(rng.integers(1, 3000))
+    incx, incy = int([1, 1, 1, 2, -1, 3][rng.integers(6)]), int([1, 1, 1, 2, -1][rng.integers(5)])
+    ox, oy = int(rng.integers(0, 17)), int(rng.integers(0, 17))
+    T = int([1 << 16, 100000, -1, -1][rng.integers(4)])
+    locs = [int([0, 0, -1, -2][rng.integers(4)]) for _ in range(2)]
+    x, y0 = _strided(rng, N, incx, ox), _strided(rng, N, incy, oy)
+    bx, by = place(pkg, x, locs[0]), place(pkg, y0, locs[1])
+    print(kind, N, "inc", incx, incy, "offsets", ox, oy, "T", T, "locs", locs, flush=True)
+    if kind == "axpy":
+        alpha = float([2.0, -1.0, 1.0, 0.0][rng.integers(4)])
+        ref = y0.copy()
+        _view(ref, N, incy, oy)[:] += alpha * _view(x, N, incx, ox)
+        pkg.check(L.PARALiA_daxpy(N, alpha, bx.at(ox), incx, by.at(oy), incy, T, C.byref(info)), "daxpy")
+        assert np.array_equal(by.get(), ref) and np.array_equal(bx.get(), x)
+    else:
+        res = C.c_double(5.0)
+        pkg.check(L.PARALiA_ddot(N, bx.at(ox), incx, by.at(oy), incy, C.byref(res), T, C.byref(info)), "ddot")
+        assert res.value == 5.0 + float(np.dot(_view(x, N, incx, ox), _view(y0, N, incy, oy)))
+        assert np.array_equal(by.get(), y0) and np.array_equal(bx.get(), x)
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 @pytest.mark.parametrize("M,N,K,pads,offs", [(2049, 2051, 301, (0, 0, 0), (0, 0)), (2304, 2100, 500, (1, 3, 1), (0, 0)),
                                              (2200, 2300, 260, (0, 0, 0), (1, 1)), (2048, 100, 300, (1, 1, 1), (0, 0))])
