@@ -178,6 +178,42 @@ __global__ __launch_bounds__(GEMV_WG) void gemv_final_kernel(long len, long chun
   *yp = beta == 0.0 ? alpha * s : fma(alpha, s, beta * *yp);
 }
 
+// The same for a short y with many chunks (a wide op = N or a tall op = T matrix: 128 x 4194304 has 2064 chunks of
+// 128 sums, and one thread per element of y adding them one after the other took 490 us of a 1100 us call).  A workgroup
+// takes 16 elements of y and cuts the chunks into 16 runs, one per thread of an element; a thread adds its run in four
+// interleaved sums, the sixteen runs are combined in LDS in run order.  The order depends on the shape only.
+constexpr int GEMV_FIN_ROWS = 16, GEMV_FIN_RUNS = GEMV_WG / GEMV_FIN_ROWS, GEMV_FIN_WIDE_FROM = 64;
+__global__ __launch_bounds__(GEMV_WG) void gemv_final_wide_kernel(long len, long chunks, const double* __restrict__ partial, double alpha,
+                                                                  double beta, double* __restrict__ y, long incy) {
+  __shared__ double red[GEMV_FIN_RUNS][GEMV_FIN_ROWS];
+  const int r = threadIdx.x % GEMV_FIN_ROWS, run = threadIdx.x / GEMV_FIN_ROWS;
+  const long i = (long)blockIdx.x * GEMV_FIN_ROWS + r;
+  double s = 0.0;
+  if (i < len) {
+    const long per = (chunks + GEMV_FIN_RUNS - 1) / GEMV_FIN_RUNS;
+    const long c0 = run * per, c1 = c0 + per < chunks ? c0 + per : chunks;
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    long c = c0;
+    for (; c + 3 < c1; c += 4) {
+      a0 += partial[c * len + i];
+      a1 += partial[(c + 1) * len + i];
+      a2 += partial[(c + 2) * len + i];
+      a3 += partial[(c + 3) * len + i];
+    }
+    for (; c < c1; ++c) a0 += partial[c * len + i];
+    s = (a0 + a1) + (a2 + a3);
+  }
+  red[run][r] = s;
+  __syncthreads();
+  if (run == 0 && i < len) {
+    s = red[0][r];
+#pragma unroll
+    for (int k = 1; k < GEMV_FIN_RUNS; ++k) s += red[k][r];
+    double* yp = y + i * incy;
+    *yp = beta == 0.0 ? alpha * s : fma(alpha, s, beta * *yp);
+  }
+}
+
 // Launches the chunk kernel and the final kernel on `stream`; `workspace` receives the chunks' partial sums.
 static int launch_gemv(char trans, long M, long N, double alpha, const double* A, long lda, const double* x, long incx, double beta,
                        double* y, long incy, double* workspace, void* stream) {
@@ -210,7 +246,11 @@ static int launch_gemv(char trans, long M, long N, double alpha, const double* A
     if (s.vec == 2) hipLaunchKernelGGL(gemv_t_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
     else hipLaunchKernelGGL(gemv_t_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
   }
-  hipLaunchKernelGGL(gemv_final_kernel, dim3(fin_blocks), dim3(GEMV_WG), 0, st, len_y, s.chunks, (const double*)workspace, alpha, beta, ys, incy);
+  if (s.chunks >= GEMV_FIN_WIDE_FROM)
+    hipLaunchKernelGGL(gemv_final_wide_kernel, dim3((unsigned)((len_y + GEMV_FIN_ROWS - 1) / GEMV_FIN_ROWS)), dim3(GEMV_WG), 0, st, len_y, s.chunks,
+                       (const double*)workspace, alpha, beta, ys, incy);
+  else
+    hipLaunchKernelGGL(gemv_final_kernel, dim3(fin_blocks), dim3(GEMV_WG), 0, st, len_y, s.chunks, (const double*)workspace, alpha, beta, ys, incy);
   return hipGetLastError() == hipSuccess ? 0 : PL_ERR_HIP;
 }
 
