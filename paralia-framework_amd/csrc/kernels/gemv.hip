@@ -6,8 +6,10 @@
 // independent loads in flight, not for the matrix cores:
 //   op = N  lanes run down the rows (a wave reads 1 KiB of one column per load), the four waves of a workgroup take
 //           every fourth column of a column chunk and are combined through LDS;
-//   op = T  a wave owns four adjacent columns and walks down their rows, sharing each x load between the four dot
-//           products, then reduces with wavefront shuffles.
+//   op = T  four adjacent columns at a time, walked down their rows with each x load shared between the four dot
+//           products and reduced with wavefront shuffles: by one wave (a workgroup takes sixteen columns) for short
+//           columns, by the four waves of a workgroup together (every fourth block of rows each, combined through LDS)
+//           from 2048 rows on.
 // Long reductions are split into chunks (grid.y) so that about GEMV_TARGET_WGS workgroups are in flight whatever the
 // shape; every chunk writes its partial sums to a workspace and a small second kernel adds them in chunk order and
 // applies alpha and beta.  The summation order therefore depends only on (op, M, N), never on timing.
@@ -26,12 +28,14 @@ constexpr int GEMV_WG = 256;
 constexpr long GEMV_TARGET_WGS = 2048;
 constexpr long GEMV_N_MIN_COLS = 64;    // columns per chunk at least (16 per wave)
 constexpr long GEMV_T_MIN_ROWS = 2048;  // rows per chunk at least
+constexpr long GEMV_T_ROWSPLIT_FROM = 2048;  // op = T: from this many rows on the waves of a workgroup share their columns
 
 struct GemvShape {
   long blocks_x;  // row blocks (N) or column groups (T)
   long chunks;    // grid.y
   long per_chunk; // columns (N) or rows (T) per chunk
   int vec;        // rows per lane in one load: 2 when 16-byte loads are possible, else 1
+  bool rowsplit;  // op = T: the four waves of a workgroup share four columns and split the rows
   long len_y;
 };
 
@@ -42,6 +46,7 @@ __host__ inline GemvShape gemv_shape(bool trans, long M, long N, long lda, const
   // wants an even M, op = N gives the one lane that holds an odd last row an 8-byte load (16383 x 16383 with lda =
   // 16384: 5.4 -> 6.7 TB/s)
   s.vec = (lda % 2 == 0 && ((unsigned long long)A % 16) == 0 && (!trans || M % 2 == 0)) ? 2 : 1;
+  s.rowsplit = false;
   if (!trans) {
     s.len_y = M;
     s.blocks_x = (M + 64 * s.vec - 1) / (64 * s.vec);
@@ -54,7 +59,12 @@ __host__ inline GemvShape gemv_shape(bool trans, long M, long N, long lda, const
     s.chunks = (N + s.per_chunk - 1) / s.per_chunk;
   } else {
     s.len_y = N;
-    s.blocks_x = (N + 15) / 16;
+    // long columns: a workgroup takes four columns and reads 4 KiB of each at a time (its waves take every fourth block
+    // of rows) instead of sixteen columns 1 KiB at a time -- 4 GiB matrices, 16384 x 32768: 6.47 -> 6.81 TB/s, 4096 x
+    // 131072: 6.25 -> 6.73, 2048 x 262144: 6.56 -> 7.05, 1048576 x 512: 6.38 -> 6.75; short columns leave waves without
+    // rows (256 x 2097152: 6.47 -> 3.92) and keep a wave per four columns
+    s.rowsplit = M >= GEMV_T_ROWSPLIT_FROM;
+    s.blocks_x = s.rowsplit ? (N + 3) / 4 : (N + 15) / 16;
     long want = (GEMV_TARGET_WGS + s.blocks_x - 1) / s.blocks_x;
     long most = M / GEMV_T_MIN_ROWS > 0 ? M / GEMV_T_MIN_ROWS : 1;
     s.chunks = want < most ? want : most;
@@ -134,8 +144,44 @@ __global__ __launch_bounds__(GEMV_WG) void gemv_n_kernel(long M, long N, const d
 template <int VEC>
 __global__ __launch_bounds__(GEMV_WG) void gemv_t_kernel(long M, long N, const double* __restrict__ A, long lda,
                                                          const double* __restrict__ x, long incx, double* __restrict__ partial,
-                                                         long rows_per_chunk) {
+                                                         long rows_per_chunk, int rowsplit) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (rowsplit) {
+    // the four waves share four columns and take every fourth block of 64 * VEC rows: the workgroup reads 4 KiB of each
+    // column at a time
+    __shared__ double red[4][4];
+    const long col0 = (long)blockIdx.x * 4;
+    const int ncols = N - col0 < 4 ? (int)(N - col0) : 4;
+    const long r0 = (long)blockIdx.y * rows_per_chunk;
+    const long r1 = r0 + rows_per_chunk < M ? r0 + rows_per_chunk : M;
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    const double* base = A + col0 * lda;
+    if (ncols == 4) {
+      for (long m = r0 + ((long)wave * 64 + lane) * VEC; m < r1; m += 4 * 64 * VEC) {
+        double xv[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) xv[v] = x[(m + v) * incx];
+        typename RowVec<VEC>::type a[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] = RowVec<VEC>::load(base + c * lda + m);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = RowVec<VEC>::dot_into(acc[c], a[c], xv);
+      }
+    } else {
+      for (long m = r0 + wave * 64 + lane; m < r1; m += 256) {
+        const double xv = x[m * incx];
+        for (int c = 0; c < ncols; ++c) acc[c] = fma(base[c * lda + m], xv, acc[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      for (int off = 32; off > 0; off >>= 1) acc[c] += __shfl_down(acc[c], off, 64);
+    if (lane == 0)
+      for (int c = 0; c < 4; ++c) red[wave][c] = acc[c];
+    __syncthreads();
+    if (threadIdx.x < ncols) partial[(long)blockIdx.y * N + col0 + threadIdx.x] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+    return;
+  }
   const long col0 = ((long)blockIdx.x * 4 + wave) * 4;
   if (col0 >= N) return;
   const int ncols = N - col0 < 4 ? (int)(N - col0) : 4;
@@ -243,8 +289,9 @@ static int launch_gemv(char trans, long M, long N, double alpha, const double* A
     if (s.vec == 2) hipLaunchKernelGGL(gemv_n_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
     else hipLaunchKernelGGL(gemv_n_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
   } else {
-    if (s.vec == 2) hipLaunchKernelGGL(gemv_t_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
-    else hipLaunchKernelGGL(gemv_t_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk);
+    const int rs = s.rowsplit ? 1 : 0;
+    if (s.vec == 2) hipLaunchKernelGGL(gemv_t_kernel<2>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk, rs);
+    else hipLaunchKernelGGL(gemv_t_kernel<1>, grid, dim3(GEMV_WG), 0, st, M, N, A, lda, xs, incx, workspace, s.per_chunk, rs);
   }
   if (s.chunks >= GEMV_FIN_WIDE_FROM)
     hipLaunchKernelGGL(gemv_final_wide_kernel, dim3((unsigned)((len_y + GEMV_FIN_ROWS - 1) / GEMV_FIN_ROWS)), dim3(GEMV_WG), 0, st, len_y, s.chunks,
